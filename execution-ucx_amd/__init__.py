@@ -1,0 +1,28 @@
+"""MI355X-native tensor-bundle path for execution-ucx (Axon).
+
+Gathers N DLPack tensors into one contiguous HBM send buffer with a per-tensor
+header and scatters a received buffer back, with hand-written HIP kernels for
+gfx950 behind a C ABI (``include/axon_rocm.h``).  The HIP library is required:
+nothing here computes on the CPU.
+"""
+from . import _capi
+from ._capi import (AxonRocmError, HeaderError, LengthError, MismatchError, NoDeviceError,
+                    UnsupportedMemoryError)
+from .bundle import BundlePlan, PackedBundle, TensorMeta, pack_bundle, unpack_bundle
+from .device import (CpuDevice, Device, DeviceType, RocmDevice, auto_detect, cpu, device_count,
+                     rocm)
+from .dlpack import DLPackExport, TensorView, extract, extract_many
+from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager
+
+__version__ = "0.1.0"
+
+
+def library_path() -> str:
+    return _capi.LIBRARY_PATH
+
+
+def tune(**kwargs) -> None:
+    """Set process-wide kernel tunables (read when a plan builds its tables)."""
+    lib = _capi.load()
+    for k, v in kwargs.items():
+        _capi.check(lib.axr_tune_set(k.encode(), int(v)))

@@ -1,0 +1,240 @@
+"""Tensor-bundle marshalling: N tensors <-> one contiguous HBM payload + header.
+
+Sender side replaces the reference's ``InvokeContext.to_ucx_buffer_vec``
+(axon/python/src/bindings_runtime_helpers.hpp:437-467), which builds one iov
+entry per tensor and lets UCX gather them: here the tensors are gathered by one
+HIP kernel launch into a pool buffer that goes out as a single contiguous
+``ucx_am_data``.  Receiver side replaces the iov scatter of
+``connection_recv_buffer(key, UcxBufferVec)``: the contiguous payload is
+either split into zero-copy views (``UcxBuffer::to_buffer_vec``,
+ucx_context/ucx_context_data.hpp:641-665) or scattered by one kernel launch
+into destination tensors.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Any, Callable, List, Optional, Sequence, Tuple
+
+from . import _capi
+from .dlpack import DLPackExport, TensorArray, TensorView, extract_many
+from .memory import DevicePool, PoolBuffer
+
+
+@dataclass(frozen=True)
+class TensorMeta:
+    """Fields of the reference's TensorMeta (rpc_core/utils/tensor_meta.hpp:77-82)
+    as carried by the bundle header, plus the packed offset and size."""
+
+    device: Tuple[int, int]
+    ndim: int
+    dtype: Tuple[int, int, int]
+    byte_offset: int
+    shape: Tuple[int, ...]
+    offset: int
+    nbytes: int
+
+
+def _stream_handle(stream) -> Optional[int]:
+    if stream is None:
+        return None
+    if isinstance(stream, int):
+        return stream or None
+    for attr in ("cuda_stream", "handle", "ptr"):
+        if hasattr(stream, attr):
+            return int(getattr(stream, attr)) or None
+    raise TypeError(f"cannot take a stream handle from {type(stream).__name__}")
+
+
+class BundlePlan:
+    """Layout + device tables of one bundle (``axr_plan_t``)."""
+
+    def __init__(self, handle: int, keepalive: Any = None):
+        self._lib = _capi.load()
+        self._h = handle
+        self._keep = keepalive
+
+    # ---- construction
+    @classmethod
+    def create(cls, tensors: Sequence[Any], align: int = 1) -> "BundlePlan":
+        """Sender side: ``tensors`` are DLPack producers (or TensorViews), laid
+        out in argument order.  ``align=1`` is the reference's tight layout."""
+        lib = _capi.load()
+        views = extract_many(tensors)
+        arr = TensorArray(views)
+        h = C.c_void_p()
+        _capi.check(lib.axr_plan_create(arr.pointer(), arr.count, align, 0, C.byref(h)))
+        return cls(h.value, keepalive=views)
+
+    @classmethod
+    def from_header(cls, header: bytes) -> "BundlePlan":
+        lib = _capi.load()
+        buf = bytes(header)
+        h = C.c_void_p()
+        _capi.check(lib.axr_plan_from_header(buf, len(buf), C.byref(h)))
+        return cls(h.value)
+
+    def bind(self, tensors: Sequence[Any]) -> "BundlePlan":
+        views = extract_many(tensors)
+        arr = TensorArray(views)
+        _capi.check(self._lib.axr_plan_bind(self._h, arr.pointer(), arr.count))
+        self._keep = views
+        return self
+
+    # ---- queries
+    @property
+    def num_tensors(self) -> int:
+        n = C.c_size_t()
+        _capi.check(self._lib.axr_plan_num_tensors(self._h, C.byref(n)))
+        return n.value
+
+    @property
+    def payload_bytes(self) -> int:
+        n = C.c_uint64()
+        _capi.check(self._lib.axr_plan_payload_bytes(self._h, C.byref(n)))
+        return n.value
+
+    @property
+    def data_bytes(self) -> int:
+        n = C.c_uint64()
+        _capi.check(self._lib.axr_plan_data_bytes(self._h, C.byref(n)))
+        return n.value
+
+    @property
+    def header(self) -> bytes:
+        p, n = C.c_void_p(), C.c_size_t()
+        _capi.check(self._lib.axr_plan_header(self._h, C.byref(p), C.byref(n)))
+        return C.string_at(p.value, n.value) if n.value else b""
+
+    def layout(self) -> Tuple[List[int], List[int]]:
+        n = self.num_tensors
+        offs = (C.c_uint64 * max(n, 1))()
+        sizes = (C.c_uint64 * max(n, 1))()
+        _capi.check(self._lib.axr_plan_layout(self._h, offs, sizes))
+        return list(offs[:n]), list(sizes[:n])
+
+    def metas(self) -> List[TensorMeta]:
+        offs, sizes = self.layout()
+        out = []
+        t = _capi.Tensor()
+        for i in range(len(offs)):
+            _capi.check(self._lib.axr_plan_tensor_meta(self._h, i, C.byref(t)))
+            out.append(TensorMeta(
+                device=(t.device_type, t.device_id), ndim=t.ndim,
+                dtype=(t.dtype_code, t.dtype_bits, t.dtype_lanes), byte_offset=0,
+                shape=tuple(t.shape[d] for d in range(t.ndim)), offset=offs[i], nbytes=sizes[i]))
+        return out
+
+    def launch_info(self) -> dict:
+        info = _capi.LaunchInfo()
+        _capi.check(self._lib.axr_plan_launch_info(self._h, C.byref(info)))
+        return {f: getattr(info, f) for f, _ in info._fields_ if f != "reserved"}
+
+    def segments(self) -> List[dict]:
+        n = C.c_size_t()
+        _capi.check(self._lib.axr_plan_segments(self._h, None, 0, C.byref(n)))
+        arr = (_capi.SegmentInfo * max(n.value, 1))()
+        _capi.check(self._lib.axr_plan_segments(self._h, arr, n.value, C.byref(n)))
+        out = []
+        for s in arr[:n.value]:
+            out.append({
+                "tensor": s.tensor, "mode": s.mode, "address": s.address, "offset": s.offset,
+                "run_bytes": s.run_bytes, "nbytes": s.nbytes, "pad": s.pad, "ndim": s.ndim,
+                "granule": s.granule, "tiles": s.tiles,
+                "shape": tuple(s.shape[:s.ndim]), "stride_bytes": tuple(s.stride_bytes[:s.ndim]),
+            })
+        return out
+
+    # ---- data movement
+    def pack(self, payload: int, payload_bytes: int, stream=None) -> None:
+        _capi.check(self._lib.axr_pack(self._h, payload, payload_bytes, _stream_handle(stream)))
+
+    def unpack(self, payload: int, payload_bytes: int, stream=None) -> None:
+        _capi.check(self._lib.axr_unpack(self._h, payload, payload_bytes, _stream_handle(stream)))
+
+    def split(self, payload: int, payload_bytes: int) -> List[Tuple[int, int]]:
+        n = self.num_tensors
+        views = (_capi.Buffer * max(n, 1))()
+        _capi.check(self._lib.axr_plan_split(self._h, payload, payload_bytes, views))
+        return [(views[i].data or 0, views[i].size) for i in range(n)]
+
+    def close(self) -> None:
+        if self._h:
+            _capi.check(self._lib.axr_plan_free(self._h))
+            self._h = None
+            self._keep = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            if self._h:
+                self._lib.axr_plan_free(self._h)
+        except Exception:  # noqa: BLE001
+            pass
+
+
+@dataclass
+class PackedBundle:
+    """What goes on the wire: the AM header bytes and the contiguous payload
+    (``ucx_am_data{header, buffer, buffer_type=ROCM, mem_h}``,
+    ucx_context/ucx_context_def.h:80-93)."""
+
+    header: bytes
+    payload: PoolBuffer
+    payload_bytes: int
+    plan: BundlePlan
+
+    @property
+    def mem_h(self):
+        return self.payload.mem_h
+
+
+def pack_bundle(tensors: Sequence[Any], align: int = 256, pool: Optional[DevicePool] = None,
+                stream=None) -> PackedBundle:
+    """Gather ``tensors`` into one pool buffer on ``stream`` (asynchronous)."""
+    plan = BundlePlan.create(tensors, align=align)
+    pool = pool or DevicePool.default()
+    nbytes = plan.payload_bytes
+    buf = pool.alloc(max(nbytes, 1), 256)
+    plan.pack(buf.data, nbytes, stream)
+    return PackedBundle(plan.header, buf, nbytes, plan)
+
+
+def unpack_bundle(header: bytes, payload: Any, payload_bytes: Optional[int] = None,
+                  out: Optional[Sequence[Any]] = None, stream=None,
+                  from_dlpack_fn: Optional[Callable[[Any], Any]] = None):
+    """Receiver side.
+
+    With ``out`` (DLPack producers of matching size): scatter the payload into
+    them with one kernel launch and return the plan (keep it until the stream
+    has drained).  Without ``out``: zero-copy mode, the payload is split at the
+    header's offsets and each piece is returned as a DLPack producer over the
+    payload memory (``from_dlpack_fn`` converts them, e.g. ``torch.from_dlpack``),
+    typed and shaped from the header.
+    """
+    if isinstance(payload, PoolBuffer):
+        ptr, size = payload.data, payload.size
+    else:
+        ptr, size = int(payload), payload_bytes
+    if payload_bytes is not None:
+        size = payload_bytes
+    plan = BundlePlan.from_header(header)
+    if out is not None:
+        plan.bind(out)
+        plan.unpack(ptr, size, stream)
+        return plan
+    pieces = plan.split(ptr, size)
+    metas = plan.metas()
+    owner = payload  # every view keeps the payload block alive
+    results = []
+    for (p, n), m in zip(pieces, metas):
+        exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLROCM, m.device[1],
+                           release=(lambda keep=owner: None))
+        results.append(from_dlpack_fn(exp) if from_dlpack_fn else exp)
+    plan.close()
+    return results

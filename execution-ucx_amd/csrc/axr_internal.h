@@ -1,0 +1,116 @@
+// Internal declarations shared by the planner (host only), the runtime shim
+// and the HIP kernels.  Nothing here is part of the C ABI.
+#ifndef AXR_INTERNAL_H_
+#define AXR_INTERNAL_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "axon_rocm.h"
+
+namespace axr {
+
+// ---------------------------------------------------------------- device tables
+//
+// One pack or unpack is ONE kernel launch that walks a segment table resident
+// in HBM.  A segment is one tensor (or one slice of a tensor with many strided
+// outer dimensions); it is cut into tiles of at most kTileBytes that never
+// cross a contiguous run, and tiles are numbered consecutively over the whole
+// bundle.  Each wavefront owns a contiguous range of tile ids.
+
+constexpr uint32_t kWaveLanes = 64;
+constexpr uint32_t kVecBytes = 16;                           // one dwordx4 per lane
+constexpr uint32_t kRowBytes = kWaveLanes * kVecBytes;       // 1 KiB per wave-wide access
+constexpr uint32_t kMaxTileRows = 16;
+constexpr uint32_t kThreadsPerWorkgroup = 256;
+constexpr uint32_t kWavesPerWorkgroup = kThreadsPerWorkgroup / kWaveLanes;
+constexpr uint32_t kMaxOuterDims = 6;
+
+constexpr uint32_t kSegPadMask = 0xfffu;         // meta bits 0..11: zero bytes after segment
+constexpr uint32_t kSegDimsShift = 12;           // meta bits 12..31: 1 + dims index
+constexpr uint32_t kSegFillOnly = 0xfffffu;      // dims field value: segment only writes zeros
+constexpr uint32_t kMaxAlign = 4096;
+
+struct Seg {              // 32 bytes
+  uint64_t ptr;           // tensor-side address of the first element
+  uint64_t off;           // payload offset of the segment's first byte
+  uint64_t run_bytes;     // bytes per contiguous run (whole segment when not strided)
+  uint32_t tile_begin;    // id of the segment's first tile
+  uint32_t meta;          // pad | (dims index + 1) << 12
+};
+static_assert(sizeof(Seg) == 32, "Seg layout");
+
+constexpr uint32_t kModeRunTiles = 0;   // every tile is a piece of one contiguous run
+constexpr uint32_t kModeElements = 1;   // tile covers packed bytes; lanes decode granules
+
+struct Dims {             // 96 bytes, one per strided segment
+  uint32_t mode;
+  uint32_t ndim;          // outer (non-run) dimensions after collapsing, <= kMaxOuterDims
+  uint32_t tiles_per_run; // kModeRunTiles
+  uint32_t granule;       // kModeElements: bytes moved per lane access (1,2,4,8,16)
+  uint64_t nbytes;        // bytes of the whole segment
+  uint32_t shape[kMaxOuterDims];
+  int64_t stride[kMaxOuterDims];   // bytes, outermost first
+};
+static_assert(sizeof(Dims) == 96, "Dims layout");
+
+struct KernelArgs {
+  const Seg* segs;            // nseg + 1 entries, last is a sentinel with tile_begin == ntiles
+  const Dims* dims;
+  const uint32_t* wave_seg;   // first segment of each wavefront's tile range
+  uint8_t* payload;
+  uint32_t nseg;
+  uint32_t ntiles;
+  uint32_t tiles_per_wave;
+  uint32_t reserved;
+};
+
+struct LaunchConfig {
+  uint32_t workgroups = 0;
+  uint32_t tiles_per_wave = 0;
+  uint32_t tile_rows = 8;
+  bool nontemporal = true;
+  bool elements = false;   // some segment uses kModeElements
+};
+
+// ---------------------------------------------------------------- tunables
+
+struct Tunables {
+  int64_t waves_per_cu = 32;      // wavefronts per compute unit the grid is sized for
+  int64_t tile_rows = 8;          // 1 KiB rows per tile (4, 8 or 16)
+  int64_t nontemporal = 1;        // non-temporal loads/stores in the copy loops
+  int64_t gather_run_bytes = 512; // strided runs shorter than this use element mode
+  int64_t min_tiles_per_wave = 1;
+};
+Tunables& tunables();
+
+// ---------------------------------------------------------------- errors
+
+int fail(int status, const std::string& message);   // records thread-local message
+int check_hip(int hip_error, const char* what);     // 0 or AXR_ERR_HIP
+
+// ---------------------------------------------------------------- kernels (axr_kernels.hip)
+
+int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& cfg,
+                         void* stream);
+int launch_fill(void* dst, int value, size_t bytes, void* stream);
+
+// ---------------------------------------------------------------- runtime (axr_runtime.cpp)
+
+int device_compute_units(int* cus);
+// Cached pinned-host + device block pair used for plan tables.
+struct TableBlock {
+  void* host = nullptr;
+  void* device = nullptr;
+  size_t bytes = 0;
+  int device_id = -1;
+};
+int table_block_acquire(size_t bytes, TableBlock* block);
+void table_block_release(TableBlock* block);
+
+}  // namespace axr
+
+#endif  // AXR_INTERNAL_H_

@@ -1,0 +1,456 @@
+// HIP kernels of the tensor-bundle path, written for gfx950 (64-lane
+// wavefronts, no matrix cores involved: this is pure data movement bound by
+// HBM bandwidth).
+//
+// One launch moves a whole bundle.  Every wavefront owns a contiguous range of
+// tile ids, finds its first segment in a host-built per-wave index (one scalar
+// load instead of a search), and walks forward through the segment table.  A
+// tile is at most ROWS x 1 KiB; a wave moves it with ROWS independent 16-byte
+// loads per lane issued back to back, then ROWS 16-byte stores, so each wave
+// keeps ROWS KiB in flight and every access is a fully coalesced 1 KiB row.
+#include <hip/hip_runtime.h>
+
+#include "axr_internal.h"
+
+namespace axr {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Tensor and payload bytes are addressed through explicit global-address-space
+// pointers (addresses arrive as integers in the segment table, which would
+// otherwise make every access a flat one); the tables themselves are read
+// through the constant address space so wave-uniform reads become scalar loads.
+#define AXR_GLOBAL __attribute__((address_space(1)))
+#define AXR_CONST __attribute__((address_space(4)))
+typedef AXR_GLOBAL uint8_t* gbytes;
+typedef const AXR_GLOBAL uint8_t* gcbytes;
+typedef AXR_GLOBAL u32x4* gvec;
+typedef const AXR_GLOBAL u32x4* gcvec;
+
+// 16-byte accesses.  Stores are always 16-byte aligned (the copy aligns the
+// destination first); loads carry no alignment promise: gfx950 serves unaligned
+// global accesses in hardware, so a source that is not congruent to its
+// destination modulo 16 costs straddling reads, not a different code path.
+typedef u32x4 __attribute__((aligned(1))) u32x4_loose;
+
+template <bool NT>
+__device__ __forceinline__ u32x4 load16(gcbytes p) {
+  const AXR_GLOBAL u32x4_loose* q = reinterpret_cast<const AXR_GLOBAL u32x4_loose*>(p);
+  if constexpr (NT) {
+    return __builtin_nontemporal_load(q);
+  } else {
+    return *q;
+  }
+}
+
+template <bool NT>
+__device__ __forceinline__ void store16(gbytes p, u32x4 v) {
+  gvec q = reinterpret_cast<gvec>(p);
+  if constexpr (NT) {
+    __builtin_nontemporal_store(v, q);
+  } else {
+    *q = v;
+  }
+}
+
+__device__ __forceinline__ uint32_t uniform(uint32_t v) {
+  return __builtin_amdgcn_readfirstlane(v);
+}
+
+__device__ __forceinline__ gbytes as_global(uint64_t address) {
+  return reinterpret_cast<gbytes>(address);
+}
+
+// Wave-cooperative copy of n <= ROWS KiB bytes.  src, dst and n are
+// wave-uniform, lane_off is lane * 16.  Handles any alignment: a byte head
+// brings dst to 16 bytes, the body moves 1 KiB rows, a byte tail finishes.
+template <uint32_t ROWS, bool NT>
+__device__ __forceinline__ void wave_copy(gcbytes src, gbytes dst, uint32_t n, uint32_t lane,
+                                          uint32_t lane_off) {
+  const uint32_t mis = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u;
+  if (mis != 0) {
+    uint32_t head = 16u - mis;
+    head = head < n ? head : n;
+    if (lane < head) dst[lane] = src[lane];
+    src += head;
+    dst += head;
+    n -= head;
+  }
+  u32x4 v[ROWS];
+  if (n == ROWS * kRowBytes) {
+#pragma unroll
+    for (uint32_t k = 0; k < ROWS; ++k) v[k] = load16<NT>(src + lane_off + k * kRowBytes);
+#pragma unroll
+    for (uint32_t k = 0; k < ROWS; ++k) store16<NT>(dst + lane_off + k * kRowBytes, v[k]);
+    return;
+  }
+  const uint32_t body = n & ~15u;
+  if (body != 0) {
+    // Partial tile: every lane loads (out-of-range lanes re-read the last
+    // vector, which keeps all ROWS loads unconditional and in flight
+    // together); only the stores are masked.
+    const uint32_t last = body - kVecBytes;
+#pragma unroll
+    for (uint32_t k = 0; k < ROWS; ++k) {
+      const uint32_t o = lane_off + k * kRowBytes;
+      v[k] = load16<NT>(src + (o < last ? o : last));
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < ROWS; ++k) {
+      const uint32_t o = lane_off + k * kRowBytes;
+      if (o < body) store16<NT>(dst + o, v[k]);
+    }
+  }
+  const uint32_t tail = n & 15u;
+  if (lane < tail) dst[body + lane] = src[body + lane];
+}
+
+__device__ __forceinline__ void wave_zero(gbytes dst, uint32_t n, uint32_t lane) {
+  for (uint32_t i = lane; i < n; i += kWaveLanes) dst[i] = 0;
+}
+
+template <typename T>
+__device__ __forceinline__ void move_as(gcbytes src, gbytes dst) {
+  typedef T __attribute__((aligned(1))) loose;   // no alignment promise on either side
+  *reinterpret_cast<AXR_GLOBAL loose*>(dst) = *reinterpret_cast<const AXR_GLOBAL loose*>(src);
+}
+
+__device__ __forceinline__ void move_granule_dyn(uint32_t g, gcbytes src, gbytes dst) {
+  switch (g) {
+    case 16: move_as<u32x4>(src, dst); break;
+    case 8: move_as<uint64_t>(src, dst); break;
+    case 4: move_as<uint32_t>(src, dst); break;
+    case 2: move_as<uint16_t>(src, dst); break;
+    default: move_as<uint8_t>(src, dst); break;
+  }
+}
+
+typedef const AXR_CONST Seg* seg_table;
+typedef const AXR_CONST Dims* dims_table;
+
+// Byte offset of run `run` inside a strided tensor; dims are right-aligned in
+// the table (unused leading entries have extent 1, stride 0).
+__device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
+  int64_t off = 0;
+  const uint32_t nd = dm->ndim;
+#pragma unroll
+  for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
+    if (static_cast<uint32_t>(d) + nd >= kMaxOuterDims) {
+      const uint32_t extent = dm->shape[d];
+      const uint32_t next = run / extent;
+      const uint32_t idx = run - next * extent;
+      off += static_cast<int64_t>(idx) * dm->stride[d];
+      run = next;
+    }
+  }
+  return off;
+}
+
+// Element mode: the tile covers kTile packed bytes of a strided segment whose
+// contiguous runs are short; each lane decodes the tensor address of its own
+// granules.  Only kernels instantiated with ELEMENTS carry this code, so the
+// streaming kernels keep a small register footprint.
+template <bool PACK, uint32_t ROWS>
+__device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_bytes, dims_table dm,
+                                          gbytes pay, uint32_t q, uint32_t lane) {
+  constexpr uint32_t kTile = ROWS * kRowBytes;
+  const uint32_t g = dm->granule;
+  const uint32_t gpr = static_cast<uint32_t>(run_bytes / g);
+  const uint64_t b0 = static_cast<uint64_t>(q) * kTile;
+  const uint64_t left = dm->nbytes - b0;
+  const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
+  const uint64_t e0 = b0 / g;
+  const uint64_t run0 = e0 / gpr;
+  const uint32_t w0 = static_cast<uint32_t>(e0 - run0 * gpr);
+  uint32_t idx0[kMaxOuterDims];
+  {
+    uint64_t r = run0;
+#pragma unroll
+    for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
+      const uint32_t extent = dm->shape[d];
+      const uint64_t next = r / extent;
+      idx0[d] = static_cast<uint32_t>(r - next * extent);
+      r = next;
+    }
+  }
+  const uint32_t ng = n / g;
+  gbytes tbase = as_global(seg_ptr);
+  gbytes pbase = pay + b0;
+  for (uint32_t e = lane; e < ng; e += kWaveLanes) {
+    uint32_t w = w0 + e;
+    uint32_t carry = w / gpr;
+    w -= carry * gpr;
+    int64_t toff = static_cast<int64_t>(w) * g;
+#pragma unroll
+    for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
+      const uint32_t extent = dm->shape[d];
+      const uint64_t v = static_cast<uint64_t>(idx0[d]) + carry;
+      const uint32_t c = static_cast<uint32_t>(v / extent);
+      const uint32_t i = static_cast<uint32_t>(v - static_cast<uint64_t>(c) * extent);
+      toff += static_cast<int64_t>(i) * dm->stride[d];
+      carry = c;
+    }
+    gbytes pp = pbase + static_cast<uint64_t>(e) * g;
+    if constexpr (PACK) {
+      move_granule_dyn(g, tbase + toff, pp);
+    } else {
+      move_granule_dyn(g, pp, tbase + toff);
+    }
+  }
+}
+
+template <bool PACK, uint32_t ROWS, bool NT, bool ELEMENTS>
+__global__ __launch_bounds__(kThreadsPerWorkgroup) void bundle_kernel(KernelArgs a) {
+  constexpr uint32_t kTile = ROWS * kRowBytes;
+  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
+  const uint32_t lane_off = lane * kVecBytes;
+  const uint32_t wave = uniform(blockIdx.x * kWavesPerWorkgroup + (threadIdx.x >> 6));
+  uint32_t t = wave * a.tiles_per_wave;
+  if (t >= a.ntiles) return;
+  const uint32_t t_end =
+      (a.ntiles - t > a.tiles_per_wave) ? t + a.tiles_per_wave : a.ntiles;
+  seg_table segs = reinterpret_cast<seg_table>(reinterpret_cast<uintptr_t>(a.segs));
+  dims_table dims = reinterpret_cast<dims_table>(reinterpret_cast<uintptr_t>(a.dims));
+  const AXR_CONST uint32_t* wave_seg =
+      reinterpret_cast<const AXR_CONST uint32_t*>(reinterpret_cast<uintptr_t>(a.wave_seg));
+  gbytes payload = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(a.payload));
+  uint32_t s = wave_seg[wave];
+  uint64_t seg_ptr = segs[s].ptr, seg_off = segs[s].off, seg_run = segs[s].run_bytes;
+  uint32_t seg_begin = segs[s].tile_begin, seg_meta = segs[s].meta;
+  uint32_t seg_end = segs[s + 1].tile_begin;
+
+  while (t < t_end) {
+    if (t >= seg_end) {   // wave-uniform: step to the next segment
+      ++s;
+      seg_ptr = segs[s].ptr;
+      seg_off = segs[s].off;
+      seg_run = segs[s].run_bytes;
+      seg_begin = segs[s].tile_begin;
+      seg_meta = segs[s].meta;
+      seg_end = segs[s + 1].tile_begin;
+      continue;
+    }
+    const uint32_t q = t - seg_begin;
+    const uint32_t pad = seg_meta & kSegPadMask;
+    const uint32_t dsel = seg_meta >> kSegDimsShift;
+    const bool last = (t + 1 == seg_end);
+    gbytes pay = payload + seg_off;
+    if (dsel == 0) {
+      // one contiguous run
+      const uint64_t boff = static_cast<uint64_t>(q) * kTile;
+      const uint64_t left = seg_run - boff;
+      const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
+      gbytes ten = as_global(seg_ptr) + boff;
+      if constexpr (PACK) {
+        wave_copy<ROWS, NT>(ten, pay + boff, n, lane, lane_off);
+        if (last && pad) wave_zero(pay + seg_run, pad, lane);
+      } else {
+        wave_copy<ROWS, NT>(pay + boff, ten, n, lane, lane_off);
+      }
+    } else if (dsel == kSegFillOnly) {
+      if constexpr (PACK) wave_zero(pay, pad, lane);
+    } else {
+      dims_table dm = dims + (dsel - 1);
+      if (dm->mode == kModeRunTiles) {
+        const uint32_t tpr = dm->tiles_per_run;
+        const uint32_t run = q / tpr;
+        const uint32_t piece = q - run * tpr;
+        const uint64_t boff = static_cast<uint64_t>(piece) * kTile;
+        const uint64_t left = seg_run - boff;
+        const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
+        gbytes ten = as_global(seg_ptr) + run_offset(dm, run) + boff;
+        gbytes p = pay + static_cast<uint64_t>(run) * seg_run + boff;
+        if constexpr (PACK) {
+          wave_copy<ROWS, NT>(ten, p, n, lane, lane_off);
+        } else {
+          wave_copy<ROWS, NT>(p, ten, n, lane, lane_off);
+        }
+      } else if constexpr (ELEMENTS) {
+        element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
+      }
+      if constexpr (PACK) {
+        if (last && pad) wave_zero(pay + dm->nbytes, pad, lane);
+      }
+    }
+    ++t;
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(uint8_t* dst, uint8_t value, size_t bytes) {
+  // 16-byte stores on the aligned body, bytes at both ends.
+  const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const size_t head = (16u - (reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
+  const size_t h = head < bytes ? head : bytes;
+  for (size_t i = tid; i < h; i += nthreads) dst[i] = value;
+  const size_t body = (bytes - h) >> 4;
+  const uint32_t w = value * 0x01010101u;
+  const u32x4 v = {w, w, w, w};
+  u32x4* d = reinterpret_cast<u32x4*>(dst + h);
+  for (size_t i = tid; i < body; i += nthreads) d[i] = v;
+  const size_t done = h + (body << 4);
+  for (size_t i = done + tid; i < bytes; i += nthreads) dst[i] = value;
+}
+
+__global__ __launch_bounds__(256) void divide_by_two_kernel(float* data, size_t count) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) data[i] /= 2.0f;
+}
+
+__global__ __launch_bounds__(256) void compare_kernel(const uint8_t* a, const uint8_t* b,
+                                                      size_t bytes,
+                                                      unsigned long long* mismatches) {
+  const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  unsigned long long local = 0;
+  for (size_t i = tid; i < bytes; i += nthreads) local += (a[i] != b[i]) ? 1u : 0u;
+  if (local) atomicAdd(mismatches, local);
+}
+
+__global__ __launch_bounds__(256) void checksum_kernel(const uint8_t* data, size_t bytes,
+                                                       uint64_t start,
+                                                       unsigned long long* sum) {
+  const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  unsigned long long local = 0;
+  for (size_t i = tid; i < bytes; i += nthreads) {
+    const uint64_t wgt = 1u + ((start + i) % 65521u);
+    local += static_cast<unsigned long long>(data[i]) * wgt;
+  }
+  atomicAdd(sum, local);
+}
+
+__global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__ dst,
+                                                             const u32x4* __restrict__ src,
+                                                             size_t nvec) {
+  const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = tid; i < nvec; i += nthreads) dst[i] = src[i];
+}
+
+template <bool PACK, uint32_t ROWS>
+int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
+  const dim3 grid(cfg.workgroups), block(kThreadsPerWorkgroup);
+  if (cfg.elements) {
+    // strided tensors with short runs are present: the general kernel
+    hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, false, true>), grid, block, 0, stream, args);
+  } else if (cfg.nontemporal) {
+    hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, true, false>), grid, block, 0, stream, args);
+  } else {
+    hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, false, false>), grid, block, 0, stream, args);
+  }
+  return check_hip(hipGetLastError(), "bundle kernel launch");
+}
+
+template <bool PACK>
+int launch_dir(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
+  switch (cfg.tile_rows) {
+    case 4: return launch_rows<PACK, 4>(args, cfg, stream);
+    case 8: return launch_rows<PACK, 8>(args, cfg, stream);
+    case 16: return launch_rows<PACK, 16>(args, cfg, stream);
+    default: return fail(AXR_ERR_INVALID, "tile_rows must be 4, 8 or 16");
+  }
+}
+
+uint32_t blocks_for(size_t items, uint32_t cap) {
+  size_t b = (items + 255) / 256;
+  if (b == 0) b = 1;
+  return static_cast<uint32_t>(b < cap ? b : cap);
+}
+
+}  // namespace
+
+int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& cfg,
+                         void* stream) {
+  if (args.ntiles == 0 || cfg.workgroups == 0) return AXR_OK;
+  // The grid must cover every tile: waves * tiles_per_wave >= ntiles.
+  const uint64_t covered = static_cast<uint64_t>(cfg.workgroups) * kWavesPerWorkgroup *
+                           cfg.tiles_per_wave;
+  if (covered < args.ntiles || args.tiles_per_wave != cfg.tiles_per_wave) {
+    return fail(AXR_ERR_INVALID, "launch geometry does not cover the tile range");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return pack ? launch_dir<true>(args, cfg, s) : launch_dir<false>(args, cfg, s);
+}
+
+int launch_fill(void* dst, int value, size_t bytes, void* stream) {
+  if (bytes == 0) return AXR_OK;
+  hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(bytes / 16 + 1, 4096)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<uint8_t*>(dst),
+                     static_cast<uint8_t>(value), bytes);
+  return check_hip(hipGetLastError(), "fill kernel launch");
+}
+
+}  // namespace axr
+
+using namespace axr;
+
+extern "C" {
+
+int axr_divide_by_two(float* data, size_t count, void* stream) {
+  if (count == 0) return AXR_OK;
+  if (!data) return fail(AXR_ERR_INVALID, "axr_divide_by_two: null data");
+  const size_t blocks = (count + 255) / 256;
+  if (blocks > 0x7fffffffu) return fail(AXR_ERR_INVALID, "axr_divide_by_two: count too large");
+  hipLaunchKernelGGL(divide_by_two_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), data, count);
+  return check_hip(hipGetLastError(), "divide_by_two launch");
+}
+
+int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mismatches) {
+  if (!mismatches) return fail(AXR_ERR_INVALID, "axr_compare: null result");
+  *mismatches = 0;
+  if (bytes == 0) return AXR_OK;
+  if (!a || !b) return fail(AXR_ERR_INVALID, "axr_compare: null range");
+  unsigned long long* dev = nullptr;
+  int rc = check_hip(hipMalloc(reinterpret_cast<void**>(&dev), sizeof(*dev)), "hipMalloc");
+  if (rc) return rc;
+  rc = check_hip(hipMemset(dev, 0, sizeof(*dev)), "hipMemset");
+  if (!rc) {
+    hipLaunchKernelGGL(compare_kernel, dim3(blocks_for(bytes, 8192)), dim3(256), 0, nullptr,
+                       static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), bytes, dev);
+    rc = check_hip(hipGetLastError(), "compare launch");
+  }
+  unsigned long long host = 0;
+  if (!rc) rc = check_hip(hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost), "hipMemcpy");
+  (void)hipFree(dev);
+  if (!rc) *mismatches = host;
+  return rc;
+}
+
+int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum) {
+  if (!sum) return fail(AXR_ERR_INVALID, "axr_checksum: null result");
+  *sum = 0;
+  if (bytes == 0) return AXR_OK;
+  if (!data) return fail(AXR_ERR_INVALID, "axr_checksum: null range");
+  unsigned long long* dev = nullptr;
+  int rc = check_hip(hipMalloc(reinterpret_cast<void**>(&dev), sizeof(*dev)), "hipMalloc");
+  if (rc) return rc;
+  rc = check_hip(hipMemset(dev, 0, sizeof(*dev)), "hipMemset");
+  if (!rc) {
+    hipLaunchKernelGGL(checksum_kernel, dim3(blocks_for(bytes, 8192)), dim3(256), 0, nullptr,
+                       static_cast<const uint8_t*>(data), bytes, start, dev);
+    rc = check_hip(hipGetLastError(), "checksum launch");
+  }
+  unsigned long long host = 0;
+  if (!rc) rc = check_hip(hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost), "hipMemcpy");
+  (void)hipFree(dev);
+  if (!rc) *sum = host;
+  return rc;
+}
+
+int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return AXR_OK;
+  if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_copy_reference: null range");
+  if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes) & 15u) {
+    return fail(AXR_ERR_INVALID, "axr_copy_reference: pointers and size must be multiples of 16");
+  }
+  const size_t nvec = bytes / 16;
+  hipLaunchKernelGGL(copy_reference_kernel, dim3(blocks_for(nvec, 256 * 32)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<u32x4*>(dst),
+                     static_cast<const u32x4*>(src), nvec);
+  return check_hip(hipGetLastError(), "copy_reference launch");
+}
+
+}  // extern "C"

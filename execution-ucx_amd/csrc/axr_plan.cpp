@@ -1,0 +1,826 @@
+// Bundle planner: layout, header codec, segment-table construction and the
+// pack / unpack entry points.
+//
+// Reference behaviour restated here:
+//   - size rule     rpc_core/utils/tensor_meta.hpp:91-104 (CalculateTensorSize)
+//   - tensor order  axon/python/src/bindings_runtime_helpers.hpp:351-414
+//   - tight concat  ucx_context/ucx_am_context/ucx_am_connection_test.cpp:1051-1108
+//   - split         ucx_context/ucx_context_data.hpp:641-665 (to_buffer_vec)
+//
+// Header wire format (all little-endian, no padding):
+//   u32 magic 0x42545841 ("AXTB") | u16 version=1 | u16 flags=0 |
+//   u32 n_tensors | u32 align | u64 payload_bytes
+//   then per tensor:
+//   u64 offset | u64 nbytes | i32 device_type | i32 device_id | i32 ndim |
+//   u8 dtype_code | u8 dtype_bits | u16 dtype_lanes | u64 byte_offset (=0) |
+//   i64 shape[ndim]
+// These are the fields of TensorMeta (tensor_meta.hpp:77-82) plus the packed
+// offset and size; strides are not sent because packed tensors are compact.
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstring>
+#include <new>
+
+#include "axr_internal.h"
+
+using namespace axr;
+
+namespace {
+
+constexpr uint32_t kMagic = 0x42545841u;
+constexpr uint16_t kVersion = 1;
+constexpr size_t kFixedHeader = 24;
+constexpr size_t kTensorHeader = 40;
+constexpr int32_t kDLCPU = 1, kDLROCM = 10, kDLROCMHost = 11;
+constexpr int kMaxNdim = 64;
+
+struct TensorRec {
+  int32_t device_type = 0, device_id = 0, ndim = 0;
+  uint8_t code = 0, bits = 0;
+  uint16_t lanes = 0;
+  size_t shape_at = 0;      // index into plan->dims64
+  bool has_strides = false;
+  size_t strides_at = 0;
+  uint64_t address = 0;     // data + byte_offset, 0 when unbound
+  uint64_t offset = 0, nbytes = 0;
+};
+
+struct HostCopy {
+  uint64_t host;
+  uint64_t offset;
+  uint64_t bytes;
+};
+
+template <typename T>
+void put(std::vector<uint8_t>& v, T x) {
+  uint8_t b[sizeof(T)];
+  std::memcpy(b, &x, sizeof(T));   // build targets are little-endian (x86-64, gfx950)
+  v.insert(v.end(), b, b + sizeof(T));
+}
+
+template <typename T>
+T get(const uint8_t* p) {
+  T x;
+  std::memcpy(&x, p, sizeof(T));
+  return x;
+}
+
+uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+bool mul_overflow(uint64_t a, uint64_t b, uint64_t* out) {
+  return __builtin_mul_overflow(a, b, out);
+}
+
+int nbytes_rule(int32_t ndim, const int64_t* shape, uint8_t bits, uint64_t* out) {
+  if (ndim == 0) {   // the reference sizes a 0-d tensor as 0 bytes
+    *out = 0;
+    return AXR_OK;
+  }
+  if (ndim < 0 || ndim > kMaxNdim) return fail(AXR_ERR_INVALID, "tensor ndim out of range");
+  if (!shape) return fail(AXR_ERR_INVALID, "tensor shape is null for ndim > 0");
+  uint64_t elems = 1;
+  for (int32_t i = 0; i < ndim; ++i) {
+    if (shape[i] < 0) return fail(AXR_ERR_INVALID, "negative tensor extent");
+    if (mul_overflow(elems, static_cast<uint64_t>(shape[i]), &elems)) {
+      // keep multiplying only to see whether a zero extent follows
+      bool zero = false;
+      for (int32_t j = 0; j < ndim; ++j) zero = zero || shape[j] == 0;
+      if (!zero) return fail(AXR_ERR_INVALID, "tensor element count overflows 64 bits");
+      elems = 0;
+      break;
+    }
+  }
+  const uint64_t item = (static_cast<uint64_t>(bits) + 7) / 8;
+  if (mul_overflow(elems, item, out)) return fail(AXR_ERR_INVALID, "tensor size overflows 64 bits");
+  return AXR_OK;
+}
+
+}  // namespace
+
+struct axr_plan {
+  uint32_t align = 1;
+  std::vector<TensorRec> tensors;
+  std::vector<int64_t> dims64;       // shapes and strides of all tensors
+  uint64_t payload_bytes = 0, data_bytes = 0;
+  std::vector<uint8_t> header;
+  bool bound = false;
+
+  // device tables
+  bool tables_built = false;
+  std::vector<Seg> segs;
+  std::vector<Dims> dims;
+  std::vector<uint32_t> wave_seg;
+  std::vector<uint32_t> seg_tensor;  // tensor index per segment (inspection)
+  std::vector<HostCopy> host_copies;
+  std::vector<uint32_t> host_copy_tensor;
+  bool overlapping_dst = false;      // some tensor has a zero stride over an extent > 1
+  uint32_t ntiles = 0;
+  LaunchConfig cfg;
+  TableBlock block;
+  size_t table_bytes = 0;
+  size_t dims_at = 0, wave_at = 0;
+  bool uploaded = false;
+  hipEvent_t upload_event = nullptr;
+  hipStream_t upload_stream = nullptr;
+  std::vector<hipStream_t> busy_streams;   // streams with launches since the last quiesce
+
+  const int64_t* shape_of(const TensorRec& t) const { return dims64.data() + t.shape_at; }
+  const int64_t* strides_of(const TensorRec& t) const {
+    return t.has_strides ? dims64.data() + t.strides_at : nullptr;
+  }
+};
+
+namespace {
+
+void compute_layout(axr_plan* p) {
+  uint64_t off = 0, data = 0;
+  for (auto& t : p->tensors) {
+    off = align_up(off, p->align);
+    t.offset = off;
+    off += t.nbytes;
+    data += t.nbytes;
+  }
+  p->payload_bytes = p->tensors.empty() ? 0 : p->tensors.back().offset + p->tensors.back().nbytes;
+  p->data_bytes = data;
+}
+
+void encode_header(axr_plan* p) {
+  std::vector<uint8_t>& h = p->header;
+  h.clear();
+  put<uint32_t>(h, kMagic);
+  put<uint16_t>(h, kVersion);
+  put<uint16_t>(h, 0);
+  put<uint32_t>(h, static_cast<uint32_t>(p->tensors.size()));
+  put<uint32_t>(h, p->align);
+  put<uint64_t>(h, p->payload_bytes);
+  for (const auto& t : p->tensors) {
+    put<uint64_t>(h, t.offset);
+    put<uint64_t>(h, t.nbytes);
+    put<int32_t>(h, t.device_type);
+    put<int32_t>(h, t.device_id);
+    put<int32_t>(h, t.ndim);
+    put<uint8_t>(h, t.code);
+    put<uint8_t>(h, t.bits);
+    put<uint16_t>(h, t.lanes);
+    put<uint64_t>(h, 0);   // byte_offset: the packed copy starts at its offset
+    const int64_t* shape = p->shape_of(t);
+    for (int32_t d = 0; d < t.ndim; ++d) put<int64_t>(h, shape[d]);
+  }
+}
+
+int check_align(uint32_t align) {
+  if (align == 0 || (align & (align - 1)) || align > kMaxAlign)
+    return fail(AXR_ERR_INVALID, "align must be a power of two in [1, 4096]");
+  return AXR_OK;
+}
+
+void invalidate_tables(axr_plan* p) {
+  p->tables_built = false;
+  p->uploaded = false;
+  p->segs.clear();
+  p->dims.clear();
+  p->wave_seg.clear();
+  p->seg_tensor.clear();
+  p->host_copies.clear();
+  p->host_copy_tensor.clear();
+  p->overlapping_dst = false;
+  p->ntiles = 0;
+}
+
+// Wait until the device no longer reads the plan's tables.  No event is
+// recorded per launch (it would put a barrier packet between back-to-back
+// bundles); the streams used since the last call are drained instead, and if
+// one of them is gone the whole device is.
+void quiesce(axr_plan* p) {
+  for (hipStream_t s : p->busy_streams) {
+    if (hipStreamSynchronize(s) != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipDeviceSynchronize();
+      break;
+    }
+  }
+  p->busy_streams.clear();
+}
+
+// ------------------------------------------------------------ table building
+
+struct Collapsed {
+  std::vector<uint64_t> extent;   // outer dims, outermost first
+  std::vector<int64_t> stride;    // bytes
+  uint64_t run_bytes = 0;
+};
+
+// Reduce (shape, element strides) to the fewest strided outer dimensions plus
+// one contiguous inner run.  Extent-1 dims vanish; adjacent dims that together
+// address a regular span merge.
+Collapsed collapse(const TensorRec& t, const int64_t* shape, const int64_t* strides,
+                   uint64_t item) {
+  Collapsed c;
+  std::vector<uint64_t> ext;
+  std::vector<int64_t> str;
+  int64_t dense = static_cast<int64_t>(item);
+  std::vector<int64_t> row_major(t.ndim);
+  for (int32_t d = t.ndim - 1; d >= 0; --d) {
+    row_major[d] = dense;
+    dense *= shape[d];
+  }
+  for (int32_t d = 0; d < t.ndim; ++d) {
+    if (shape[d] == 1) continue;
+    ext.push_back(static_cast<uint64_t>(shape[d]));
+    str.push_back(strides ? strides[d] * static_cast<int64_t>(item) : row_major[d]);
+  }
+  // merge from the inside out
+  std::vector<uint64_t> me;
+  std::vector<int64_t> ms;
+  for (size_t i = ext.size(); i-- > 0;) {
+    if (!me.empty() && str[i] == ms.back() * static_cast<int64_t>(me.back())) {
+      me.back() *= ext[i];   // outer dim continues the inner one
+    } else {
+      me.push_back(ext[i]);
+      ms.push_back(str[i]);
+    }
+  }
+  // me/ms are innermost first
+  size_t first_outer = 0;
+  if (!me.empty() && ms[0] == static_cast<int64_t>(item)) {
+    c.run_bytes = me[0] * item;
+    first_outer = 1;
+  } else {
+    c.run_bytes = item;
+  }
+  for (size_t i = me.size(); i-- > first_outer;) {
+    c.extent.push_back(me[i]);
+    c.stride.push_back(ms[i]);
+  }
+  return c;
+}
+
+struct Builder {
+  axr_plan* p;
+  uint32_t tile_bytes;
+  uint64_t tiles = 0;
+
+  int add_seg(uint32_t tensor, uint64_t ptr, uint64_t off, uint64_t run_bytes, uint64_t ntile,
+              uint32_t dsel) {
+    if (tiles + ntile > 0xffffffffull) return fail(AXR_ERR_UNSUPPORTED, "bundle has too many tiles");
+    Seg s;
+    s.ptr = ptr;
+    s.off = off;
+    s.run_bytes = run_bytes;
+    s.tile_begin = static_cast<uint32_t>(tiles);
+    s.meta = dsel << kSegDimsShift;
+    p->segs.push_back(s);
+    p->seg_tensor.push_back(tensor);
+    tiles += ntile;
+    return AXR_OK;
+  }
+
+  // Emit device segments for a strided block: `outer` strided dims (any count)
+  // around one contiguous run.  More than kMaxOuterDims dims are peeled off on
+  // the host, outermost first.
+  int add_strided(uint32_t tensor, uint64_t ptr, uint64_t off, const uint64_t* ext,
+                  const int64_t* str, size_t nd, uint64_t run_bytes) {
+    if (nd == 0) {
+      return add_seg(tensor, ptr, off, run_bytes, (run_bytes + tile_bytes - 1) / tile_bytes, 0);
+    }
+    uint64_t inner_runs = 1;
+    for (size_t d = 1; d < nd; ++d) inner_runs *= ext[d];
+    if (nd > kMaxOuterDims) {
+      for (uint64_t i = 0; i < ext[0]; ++i) {
+        int rc = add_strided(tensor, ptr + static_cast<uint64_t>(static_cast<int64_t>(i) * str[0]),
+                             off + i * inner_runs * run_bytes, ext + 1, str + 1, nd - 1, run_bytes);
+        if (rc) return rc;
+      }
+      return AXR_OK;
+    }
+    const uint64_t runs = inner_runs * ext[0];
+    const uint64_t nbytes = runs * run_bytes;
+    Dims dm;
+    std::memset(&dm, 0, sizeof(dm));
+    dm.ndim = static_cast<uint32_t>(nd);
+    dm.nbytes = nbytes;
+    for (uint32_t d = 0; d < kMaxOuterDims; ++d) {
+      dm.shape[d] = 1;
+      dm.stride[d] = 0;
+    }
+    for (size_t d = 0; d < nd; ++d) {
+      if (ext[d] > 0xffffffffull) return fail(AXR_ERR_UNSUPPORTED, "strided extent exceeds 32 bits");
+      dm.shape[kMaxOuterDims - nd + d] = static_cast<uint32_t>(ext[d]);
+      dm.stride[kMaxOuterDims - nd + d] = str[d];
+    }
+    uint64_t ntile;
+    if (run_bytes >= static_cast<uint64_t>(tunables().gather_run_bytes)) {
+      dm.mode = kModeRunTiles;
+      const uint64_t tpr = (run_bytes + tile_bytes - 1) / tile_bytes;
+      if (tpr > 0xffffffffull || runs > 0xffffffffull)
+        return fail(AXR_ERR_UNSUPPORTED, "strided tensor has too many runs");
+      dm.tiles_per_run = static_cast<uint32_t>(tpr);
+      ntile = runs * tpr;
+    } else {
+      dm.mode = kModeElements;
+      uint32_t g = 16;
+      while (g > 1 && (run_bytes % g) != 0) g >>= 1;
+      dm.granule = g;
+      ntile = (nbytes + tile_bytes - 1) / tile_bytes;
+    }
+    if (p->dims.size() + 1 >= kSegFillOnly)
+      return fail(AXR_ERR_UNSUPPORTED, "too many strided tensors in one bundle");
+    p->dims.push_back(dm);
+    return add_seg(tensor, ptr, off, run_bytes, ntile, static_cast<uint32_t>(p->dims.size()));
+  }
+
+  // Host (kDLCPU) tensors move with one async copy per contiguous run.
+  int add_host(uint32_t tensor, uint64_t ptr, uint64_t off, const uint64_t* ext,
+               const int64_t* str, size_t nd, uint64_t run_bytes) {
+    if (nd == 0) {
+      if (p->host_copies.size() >= (1u << 20))
+        return fail(AXR_ERR_UNSUPPORTED, "host tensor needs more than 2^20 copies");
+      p->host_copies.push_back({ptr, off, run_bytes});
+      p->host_copy_tensor.push_back(tensor);
+      return AXR_OK;
+    }
+    uint64_t inner = run_bytes;
+    for (size_t d = 1; d < nd; ++d) inner *= ext[d];
+    for (uint64_t i = 0; i < ext[0]; ++i) {
+      int rc = add_host(tensor, ptr + static_cast<uint64_t>(static_cast<int64_t>(i) * str[0]),
+                        off + i * inner, ext + 1, str + 1, nd - 1, run_bytes);
+      if (rc) return rc;
+    }
+    return AXR_OK;
+  }
+};
+
+int build_tables(axr_plan* p) {
+  if (p->tables_built) return AXR_OK;
+  if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
+  invalidate_tables(p);
+  const Tunables& tn = tunables();
+  Builder b{p, static_cast<uint32_t>(tn.tile_rows) * kRowBytes};
+
+  for (size_t i = 0; i < p->tensors.size(); ++i) {
+    const TensorRec& t = p->tensors[i];
+    if (t.nbytes == 0) continue;
+    const uint64_t item = (static_cast<uint64_t>(t.bits) + 7) / 8;
+    const uint64_t end = t.offset + t.nbytes;
+    const uint64_t pad = std::min<uint64_t>(align_up(end, p->align), p->payload_bytes) - end;
+    const int64_t* shape = p->shape_of(t);
+    const int64_t* strides = p->strides_of(t);
+    if (strides) {
+      for (int32_t d = 0; d < t.ndim; ++d)
+        if (strides[d] == 0 && shape[d] > 1) p->overlapping_dst = true;
+    }
+    Collapsed c = collapse(t, shape, strides, item);
+    const size_t first = p->segs.size();
+    int rc;
+    if (t.device_type == kDLROCM || t.device_type == kDLROCMHost) {
+      rc = b.add_strided(static_cast<uint32_t>(i), t.address, t.offset, c.extent.data(),
+                         c.stride.data(), c.extent.size(), c.run_bytes);
+      if (rc) return rc;
+      if (pad) p->segs.back().meta |= static_cast<uint32_t>(pad);
+    } else if (t.device_type == kDLCPU) {
+      rc = b.add_host(static_cast<uint32_t>(i), t.address, t.offset, c.extent.data(),
+                      c.stride.data(), c.extent.size(), c.run_bytes);
+      if (rc) return rc;
+      if (pad) {
+        rc = b.add_seg(static_cast<uint32_t>(i), 0, end, 0, 1, kSegFillOnly);
+        if (rc) return rc;
+        p->segs.back().meta |= static_cast<uint32_t>(pad);
+      }
+    } else {
+      return fail(AXR_ERR_UNSUPPORTED,
+                  "Unsupported memory type: DLPack device " + std::to_string(t.device_type));
+    }
+    (void)first;
+  }
+  p->ntiles = static_cast<uint32_t>(b.tiles);
+  Seg sentinel;
+  std::memset(&sentinel, 0, sizeof(sentinel));
+  sentinel.tile_begin = p->ntiles;
+  p->segs.push_back(sentinel);
+
+  // launch geometry
+  int cus = 256;
+  if (device_compute_units(&cus) != AXR_OK || cus <= 0) cus = 256;
+  const uint64_t waves = static_cast<uint64_t>(cus) * static_cast<uint64_t>(tn.waves_per_cu);
+  uint64_t tpw = (p->ntiles + waves - 1) / waves;
+  if (tpw < static_cast<uint64_t>(tn.min_tiles_per_wave)) tpw = tn.min_tiles_per_wave;
+  if (tpw == 0) tpw = 1;
+  const uint64_t per_wg = tpw * kWavesPerWorkgroup;
+  p->cfg.tiles_per_wave = static_cast<uint32_t>(tpw);
+  p->cfg.workgroups = static_cast<uint32_t>((p->ntiles + per_wg - 1) / per_wg);
+  p->cfg.tile_rows = static_cast<uint32_t>(tn.tile_rows);
+  p->cfg.nontemporal = tn.nontemporal != 0;
+  p->cfg.elements = false;
+  for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode == kModeElements;
+
+  const size_t nwaves = static_cast<size_t>(p->cfg.workgroups) * kWavesPerWorkgroup;
+  p->wave_seg.assign(nwaves, 0);
+  size_t s = 0;
+  const size_t nseg = p->segs.size() - 1;
+  for (size_t w = 0; w < nwaves; ++w) {
+    const uint64_t t0 = static_cast<uint64_t>(w) * tpw;
+    if (t0 >= p->ntiles) break;
+    while (s + 1 < nseg && p->segs[s + 1].tile_begin <= t0) ++s;
+    p->wave_seg[w] = static_cast<uint32_t>(s);
+  }
+
+  p->dims_at = align_up(p->segs.size() * sizeof(Seg), 16);
+  p->wave_at = align_up(p->dims_at + p->dims.size() * sizeof(Dims), 16);
+  p->table_bytes = p->wave_at + p->wave_seg.size() * sizeof(uint32_t);
+  p->tables_built = true;
+  return AXR_OK;
+}
+
+int ensure_uploaded(axr_plan* p, hipStream_t stream) {
+  if (p->ntiles == 0) return AXR_OK;
+  if (!p->uploaded) {
+    if (p->block.host && (p->block.bytes < p->table_bytes)) {
+      quiesce(p);
+      table_block_release(&p->block);
+    }
+    if (!p->block.host) {
+      int rc = table_block_acquire(p->table_bytes, &p->block);
+      if (rc) return rc;
+    } else {
+      quiesce(p);   // previous launches may still read the old tables
+    }
+    uint8_t* h = static_cast<uint8_t*>(p->block.host);
+    std::memcpy(h, p->segs.data(), p->segs.size() * sizeof(Seg));
+    if (!p->dims.empty()) std::memcpy(h + p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims));
+    std::memcpy(h + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t));
+    int rc = check_hip(hipMemcpyAsync(p->block.device, h, p->table_bytes, hipMemcpyHostToDevice,
+                                      stream),
+                       "hipMemcpyAsync(plan tables)");
+    if (rc) return rc;
+    if (!p->upload_event) {
+      rc = check_hip(hipEventCreateWithFlags(&p->upload_event, hipEventDisableTiming),
+                     "hipEventCreate");
+      if (rc) return rc;
+    }
+    rc = check_hip(hipEventRecord(p->upload_event, stream), "hipEventRecord");
+    if (rc) return rc;
+    p->upload_stream = stream;
+    p->uploaded = true;
+  } else if (stream != p->upload_stream) {
+    int rc = check_hip(hipStreamWaitEvent(stream, p->upload_event, 0), "hipStreamWaitEvent");
+    if (rc) return rc;
+  }
+  return AXR_OK;
+}
+
+int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* stream_) {
+  if (!p) return fail(AXR_ERR_INVALID, "null plan");
+  if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
+  if (payload_bytes < p->payload_bytes)
+    return fail(AXR_ERR_LENGTH, "payload buffer is smaller than the plan's payload");
+  if (p->payload_bytes == 0) return AXR_OK;
+  if (!payload) return fail(AXR_ERR_INVALID, "null payload");
+  int rc = build_tables(p);
+  if (rc) return rc;
+  if (!pack && p->overlapping_dst)
+    return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  for (const HostCopy& hc : p->host_copies) {
+    void* dev = static_cast<uint8_t*>(payload) + hc.offset;
+    void* host = reinterpret_cast<void*>(hc.host);
+    rc = pack ? check_hip(hipMemcpyAsync(dev, host, hc.bytes, hipMemcpyDefault, stream),
+                          "hipMemcpyAsync(host tensor -> payload)")
+              : check_hip(hipMemcpyAsync(host, dev, hc.bytes, hipMemcpyDefault, stream),
+                          "hipMemcpyAsync(payload -> host tensor)");
+    if (rc) return rc;
+  }
+  if (p->ntiles == 0) return AXR_OK;
+  rc = ensure_uploaded(p, stream);
+  if (rc) return rc;
+  KernelArgs a;
+  uint8_t* d = static_cast<uint8_t*>(p->block.device);
+  a.segs = reinterpret_cast<const Seg*>(d);
+  a.dims = reinterpret_cast<const Dims*>(d + p->dims_at);
+  a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
+  a.payload = static_cast<uint8_t*>(payload);
+  a.nseg = static_cast<uint32_t>(p->segs.size() - 1);
+  a.ntiles = p->ntiles;
+  a.tiles_per_wave = p->cfg.tiles_per_wave;
+  a.reserved = 0;
+  rc = launch_bundle_kernel(pack, a, p->cfg, stream);
+  if (rc) return rc;
+  if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+    p->busy_streams.push_back(stream);
+  return AXR_OK;
+}
+
+int store_tensor(axr_plan* p, const axr_tensor_t& in, TensorRec* rec) {
+  rec->device_type = in.device_type;
+  rec->device_id = in.device_id;
+  rec->ndim = in.ndim;
+  rec->code = in.dtype_code;
+  rec->bits = in.dtype_bits;
+  rec->lanes = in.dtype_lanes;
+  int rc = nbytes_rule(in.ndim, in.shape, in.dtype_bits, &rec->nbytes);
+  if (rc) return rc;
+  rec->shape_at = p->dims64.size();
+  for (int32_t d = 0; d < in.ndim; ++d) p->dims64.push_back(in.shape[d]);
+  rec->has_strides = in.strides != nullptr && in.ndim > 0;
+  if (rec->has_strides) {
+    rec->strides_at = p->dims64.size();
+    for (int32_t d = 0; d < in.ndim; ++d) p->dims64.push_back(in.strides[d]);
+  }
+  if (rec->nbytes != 0 && in.data == nullptr)
+    return fail(AXR_ERR_INVALID, "tensor data pointer is null");
+  rec->address = reinterpret_cast<uint64_t>(in.data) + in.byte_offset;
+  return AXR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int axr_tensor_nbytes(const axr_tensor_t* t, uint64_t* nbytes) {
+  if (!t || !nbytes) return fail(AXR_ERR_INVALID, "axr_tensor_nbytes: null argument");
+  return nbytes_rule(t->ndim, t->shape, t->dtype_bits, nbytes);
+}
+
+int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align, uint32_t /*flags*/,
+                    axr_plan_t** plan) {
+  if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_create: null result");
+  *plan = nullptr;
+  if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_create: null tensor array");
+  if (n > 0xffffffffull) return fail(AXR_ERR_INVALID, "axr_plan_create: too many tensors");
+  int rc = check_align(align);
+  if (rc) return rc;
+  axr_plan* p = new (std::nothrow) axr_plan();
+  if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_create: out of host memory");
+  p->align = align;
+  p->tensors.resize(n);
+  for (size_t i = 0; i < n; ++i) {
+    rc = store_tensor(p, tensors[i], &p->tensors[i]);
+    if (rc) {
+      delete p;
+      return rc;
+    }
+  }
+  compute_layout(p);
+  encode_header(p);
+  p->bound = true;
+  *plan = p;
+  return AXR_OK;
+}
+
+int axr_plan_free(axr_plan_t* plan) {
+  if (!plan) return AXR_OK;
+  quiesce(plan);
+  if (plan->uploaded && plan->upload_event) (void)hipEventSynchronize(plan->upload_event);
+  table_block_release(&plan->block);
+  if (plan->upload_event) (void)hipEventDestroy(plan->upload_event);
+  delete plan;
+  return AXR_OK;
+}
+
+int axr_plan_num_tensors(const axr_plan_t* plan, size_t* n) {
+  if (!plan || !n) return fail(AXR_ERR_INVALID, "axr_plan_num_tensors: null argument");
+  *n = plan->tensors.size();
+  return AXR_OK;
+}
+
+int axr_plan_payload_bytes(const axr_plan_t* plan, uint64_t* bytes) {
+  if (!plan || !bytes) return fail(AXR_ERR_INVALID, "axr_plan_payload_bytes: null argument");
+  *bytes = plan->payload_bytes;
+  return AXR_OK;
+}
+
+int axr_plan_data_bytes(const axr_plan_t* plan, uint64_t* bytes) {
+  if (!plan || !bytes) return fail(AXR_ERR_INVALID, "axr_plan_data_bytes: null argument");
+  *bytes = plan->data_bytes;
+  return AXR_OK;
+}
+
+int axr_plan_layout(const axr_plan_t* plan, uint64_t* offsets, uint64_t* sizes) {
+  if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_layout: null plan");
+  for (size_t i = 0; i < plan->tensors.size(); ++i) {
+    if (offsets) offsets[i] = plan->tensors[i].offset;
+    if (sizes) sizes[i] = plan->tensors[i].nbytes;
+  }
+  return AXR_OK;
+}
+
+int axr_plan_tensor_meta(const axr_plan_t* plan, size_t i, axr_tensor_t* meta) {
+  if (!plan || !meta) return fail(AXR_ERR_INVALID, "axr_plan_tensor_meta: null argument");
+  if (i >= plan->tensors.size()) return fail(AXR_ERR_INVALID, "axr_plan_tensor_meta: index out of range");
+  const TensorRec& t = plan->tensors[i];
+  meta->data = nullptr;
+  meta->device_type = t.device_type;
+  meta->device_id = t.device_id;
+  meta->ndim = t.ndim;
+  meta->dtype_code = t.code;
+  meta->dtype_bits = t.bits;
+  meta->dtype_lanes = t.lanes;
+  meta->shape = t.ndim ? const_cast<int64_t*>(plan->shape_of(t)) : nullptr;
+  meta->strides = const_cast<int64_t*>(plan->strides_of(t));
+  meta->byte_offset = 0;
+  return AXR_OK;
+}
+
+int axr_plan_header(const axr_plan_t* plan, const void** header, size_t* length) {
+  if (!plan || !header || !length) return fail(AXR_ERR_INVALID, "axr_plan_header: null argument");
+  *header = plan->header.data();
+  *length = plan->header.size();
+  return AXR_OK;
+}
+
+int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan) {
+  if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_from_header: null result");
+  *plan = nullptr;
+  if (!header) return fail(AXR_ERR_INVALID, "axr_plan_from_header: null header");
+  const uint8_t* h = static_cast<const uint8_t*>(header);
+  if (length < kFixedHeader) return fail(AXR_ERR_HEADER, "bundle header shorter than its fixed part");
+  if (get<uint32_t>(h) != kMagic) return fail(AXR_ERR_HEADER, "bundle header has a wrong magic");
+  if (get<uint16_t>(h + 4) != kVersion) return fail(AXR_ERR_HEADER, "bundle header version not supported");
+  if (get<uint16_t>(h + 6) != 0) return fail(AXR_ERR_HEADER, "bundle header has unknown flags");
+  const uint32_t n = get<uint32_t>(h + 8);
+  const uint32_t align = get<uint32_t>(h + 12);
+  const uint64_t payload = get<uint64_t>(h + 16);
+  if (check_align(align) != AXR_OK) return fail(AXR_ERR_HEADER, "bundle header has a bad alignment");
+  if (static_cast<uint64_t>(n) * kTensorHeader > length - kFixedHeader)
+    return fail(AXR_ERR_HEADER, "bundle header truncated");
+  axr_plan* p = new (std::nothrow) axr_plan();
+  if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_from_header: out of host memory");
+  p->align = align;
+  p->tensors.resize(n);
+  size_t at = kFixedHeader;
+  for (uint32_t i = 0; i < n; ++i) {
+    if (length - at < kTensorHeader) {
+      delete p;
+      return fail(AXR_ERR_HEADER, "bundle header truncated");
+    }
+    TensorRec& t = p->tensors[i];
+    const uint64_t off = get<uint64_t>(h + at);
+    const uint64_t nb = get<uint64_t>(h + at + 8);
+    t.device_type = get<int32_t>(h + at + 16);
+    t.device_id = get<int32_t>(h + at + 20);
+    t.ndim = get<int32_t>(h + at + 24);
+    t.code = get<uint8_t>(h + at + 28);
+    t.bits = get<uint8_t>(h + at + 29);
+    t.lanes = get<uint16_t>(h + at + 30);
+    const uint64_t byte_offset = get<uint64_t>(h + at + 32);
+    at += kTensorHeader;
+    if (t.ndim < 0 || t.ndim > kMaxNdim ||
+        static_cast<size_t>(t.ndim) * 8 > length - at || byte_offset != 0) {
+      delete p;
+      return fail(AXR_ERR_HEADER, "bundle header has a bad tensor record");
+    }
+    t.shape_at = p->dims64.size();
+    for (int32_t d = 0; d < t.ndim; ++d) p->dims64.push_back(get<int64_t>(h + at + 8 * d));
+    at += static_cast<size_t>(t.ndim) * 8;
+    uint64_t rule = 0;
+    if (nbytes_rule(t.ndim, p->dims64.data() + t.shape_at, t.bits, &rule) != AXR_OK || rule != nb) {
+      delete p;
+      return fail(AXR_ERR_HEADER, "bundle header tensor size does not follow from its shape");
+    }
+    t.nbytes = nb;
+    t.offset = off;   // checked against the layout rule below
+  }
+  if (at != length) {
+    delete p;
+    return fail(AXR_ERR_HEADER, "bundle header has trailing bytes");
+  }
+  std::vector<uint64_t> sent(n);
+  for (uint32_t i = 0; i < n; ++i) sent[i] = p->tensors[i].offset;
+  compute_layout(p);
+  bool ok = p->payload_bytes == payload;
+  for (uint32_t i = 0; i < n && ok; ++i) ok = sent[i] == p->tensors[i].offset;
+  if (!ok) {
+    delete p;
+    return fail(AXR_ERR_HEADER, "bundle header offsets do not follow the layout rule");
+  }
+  p->header.assign(h, h + length);
+  p->bound = false;
+  *plan = p;
+  return AXR_OK;
+}
+
+int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {
+  if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_bind: null plan");
+  if (n != plan->tensors.size())
+    return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor count differs from the plan");
+  if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_bind: null tensor array");
+  // validate everything before touching the plan
+  for (size_t i = 0; i < n; ++i) {
+    const TensorRec& t = plan->tensors[i];
+    const axr_tensor_t& in = tensors[i];
+    uint64_t nb = 0;
+    int rc = nbytes_rule(in.ndim, in.shape, in.dtype_bits, &nb);
+    if (rc) return rc;
+    if (nb != t.nbytes || (nb != 0 && (in.dtype_bits + 7) / 8 != (t.bits + 7) / 8))
+      return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor " + std::to_string(i) +
+                                        " does not match the plan's size or element width");
+    if (nb != 0 && !in.data) return fail(AXR_ERR_INVALID, "axr_plan_bind: null tensor data");
+  }
+  quiesce(plan);
+  invalidate_tables(plan);
+  std::vector<int64_t> dims64;
+  std::vector<TensorRec> recs(n);
+  {
+    axr_plan tmp;   // reuse store_tensor's bookkeeping
+    for (size_t i = 0; i < n; ++i) {
+      int rc = store_tensor(&tmp, tensors[i], &recs[i]);
+      if (rc) return rc;
+    }
+    dims64.swap(tmp.dims64);
+  }
+  for (size_t i = 0; i < n; ++i) {
+    recs[i].offset = plan->tensors[i].offset;
+    recs[i].nbytes = plan->tensors[i].nbytes;
+  }
+  // The header keeps describing what was sent; the bound records describe memory.
+  plan->tensors.swap(recs);
+  plan->dims64.swap(dims64);
+  plan->bound = true;
+  return AXR_OK;
+}
+
+int axr_plan_split(const axr_plan_t* plan, void* payload, size_t payload_bytes,
+                   axr_buffer_t* views) {
+  if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_split: null plan");
+  if (plan->payload_bytes > payload_bytes)
+    return fail(AXR_ERR_LENGTH, "Total size of chunks exceeds buffer size");
+  if (plan->tensors.empty()) return AXR_OK;
+  if (!views) return fail(AXR_ERR_INVALID, "axr_plan_split: null views");
+  for (size_t i = 0; i < plan->tensors.size(); ++i) {
+    views[i].data = static_cast<uint8_t*>(payload) + plan->tensors[i].offset;
+    views[i].size = plan->tensors[i].nbytes;
+  }
+  return AXR_OK;
+}
+
+int axr_pack(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream) {
+  return run(plan, true, payload, payload_bytes, stream);
+}
+
+int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes, void* stream) {
+  return run(plan, false, const_cast<void*>(payload), payload_bytes, stream);
+}
+
+int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
+  if (!plan || !info) return fail(AXR_ERR_INVALID, "axr_plan_launch_info: null argument");
+  int rc = build_tables(plan);
+  if (rc) return rc;
+  info->workgroups = plan->cfg.workgroups;
+  info->threads_per_workgroup = kThreadsPerWorkgroup;
+  info->tiles = plan->ntiles;
+  info->tile_bytes = plan->cfg.tile_rows * kRowBytes;
+  info->segments = static_cast<uint32_t>(plan->segs.size() - 1);
+  info->table_bytes = static_cast<uint32_t>(plan->table_bytes);
+  info->host_copies = static_cast<uint32_t>(plan->host_copies.size());
+  info->reserved = 0;
+  return AXR_OK;
+}
+
+int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity, size_t* count) {
+  if (!plan || !count) return fail(AXR_ERR_INVALID, "axr_plan_segments: null argument");
+  int rc = build_tables(plan);
+  if (rc) return rc;
+  const size_t nseg = plan->segs.size() - 1;
+  *count = nseg + plan->host_copies.size();
+  size_t w = 0;
+  for (size_t i = 0; i < nseg && out && w < capacity; ++i, ++w) {
+    const Seg& s = plan->segs[i];
+    axr_segment_info_t& o = out[w];
+    std::memset(&o, 0, sizeof(o));
+    o.tensor = plan->seg_tensor[i];
+    o.address = s.ptr;
+    o.offset = s.off;
+    o.run_bytes = s.run_bytes;
+    o.pad = s.meta & kSegPadMask;
+    o.tiles = plan->segs[i + 1].tile_begin - s.tile_begin;
+    const uint32_t dsel = s.meta >> kSegDimsShift;
+    if (dsel == 0) {
+      o.mode = 0;
+      o.nbytes = s.run_bytes;
+    } else if (dsel == kSegFillOnly) {
+      o.mode = 3;
+    } else {
+      const Dims& dm = plan->dims[dsel - 1];
+      o.mode = dm.mode == kModeRunTiles ? 1 : 2;
+      o.nbytes = dm.nbytes;
+      o.ndim = dm.ndim;
+      o.granule = dm.granule;
+      for (uint32_t d = 0; d < dm.ndim; ++d) {
+        o.shape[d] = dm.shape[kMaxOuterDims - dm.ndim + d];
+        o.stride_bytes[d] = dm.stride[kMaxOuterDims - dm.ndim + d];
+      }
+    }
+  }
+  for (size_t i = 0; i < plan->host_copies.size() && out && w < capacity; ++i, ++w) {
+    axr_segment_info_t& o = out[w];
+    std::memset(&o, 0, sizeof(o));
+    o.tensor = plan->host_copy_tensor[i];
+    o.mode = 4;
+    o.address = plan->host_copies[i].host;
+    o.offset = plan->host_copies[i].offset;
+    o.run_bytes = o.nbytes = plan->host_copies[i].bytes;
+  }
+  return AXR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,697 @@
+// Runtime shim: device selection, streams, events, copies and the slab pool.
+// This file (with axr_kernels.hip) is the only place that includes HIP
+// headers; host code above the C ABI never does.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <set>
+#include <unordered_map>
+#include <utility>
+
+#include "axr_internal.h"
+
+namespace axr {
+
+namespace {
+thread_local std::string g_last_error;
+}
+
+int fail(int status, const std::string& message) {
+  g_last_error = message;
+  return status;
+}
+
+int check_hip(int hip_error, const char* what) {
+  if (hip_error == hipSuccess) return AXR_OK;
+  const hipError_t e = static_cast<hipError_t>(hip_error);
+  std::string msg = std::string(what) + ": " + hipGetErrorName(e) + " (" +
+                    hipGetErrorString(e) + ")";
+  if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) return fail(AXR_ERR_NO_DEVICE, msg);
+  if (e == hipErrorOutOfMemory) return fail(AXR_ERR_NOMEM, msg);
+  return fail(AXR_ERR_HIP, msg);
+}
+
+Tunables& tunables() {
+  static Tunables t;
+  return t;
+}
+
+int device_compute_units(int* cus) {
+  static std::mutex mu;
+  static std::map<int, int> cache;
+  int dev = 0;
+  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(dev);
+  if (it == cache.end()) {
+    int n = 0;
+    rc = check_hip(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev),
+                   "hipDeviceGetAttribute");
+    if (rc) return rc;
+    it = cache.emplace(dev, n).first;
+  }
+  *cus = it->second;
+  return AXR_OK;
+}
+
+// ------------------------------------------------------------ table blocks
+//
+// Plan tables are staged in pinned host memory and copied to a device block
+// with one async copy.  Both halves are recycled through a size-bucketed
+// free list so that steady-state planning performs no driver allocation.
+
+namespace {
+struct TableCache {
+  std::mutex mu;
+  std::multimap<std::pair<int, size_t>, TableBlock> free_blocks;
+};
+TableCache& table_cache() {
+  static TableCache* c = new TableCache();   // leaked on purpose: outlives static dtors
+  return *c;
+}
+size_t bucket_bytes(size_t bytes) {
+  size_t b = 4096;
+  while (b < bytes) b <<= 1;
+  return b;
+}
+}  // namespace
+
+int table_block_acquire(size_t bytes, TableBlock* block) {
+  int dev = 0;
+  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc) return rc;
+  const size_t want = bucket_bytes(bytes);
+  TableCache& c = table_cache();
+  {
+    std::lock_guard<std::mutex> lock(c.mu);
+    auto it = c.free_blocks.find({dev, want});
+    if (it != c.free_blocks.end()) {
+      *block = it->second;
+      c.free_blocks.erase(it);
+      return AXR_OK;
+    }
+  }
+  TableBlock b;
+  b.bytes = want;
+  b.device_id = dev;
+  rc = check_hip(hipHostMalloc(&b.host, want, hipHostMallocDefault), "hipHostMalloc(table)");
+  if (rc) return rc;
+  rc = check_hip(hipMalloc(&b.device, want), "hipMalloc(table)");
+  if (rc) {
+    (void)hipHostFree(b.host);
+    return rc;
+  }
+  *block = b;
+  return AXR_OK;
+}
+
+void table_block_release(TableBlock* block) {
+  if (!block->host) return;
+  TableCache& c = table_cache();
+  std::lock_guard<std::mutex> lock(c.mu);
+  c.free_blocks.emplace(std::make_pair(block->device_id, block->bytes), *block);
+  *block = TableBlock();
+}
+
+}  // namespace axr
+
+using namespace axr;
+
+// ================================================================ slab pool
+
+struct axr_pool {
+  struct Slab {
+    char* base = nullptr;
+    size_t bytes = 0;
+    void* mem_h = nullptr;
+    size_t live = 0;   // blocks handed out from this slab
+  };
+  int device = 0;
+  size_t slab_bytes = 0;
+  std::mutex mu;
+  std::map<char*, Slab> slabs;                 // by base address
+  std::map<char*, size_t> free_by_addr;        // free block -> size
+  std::set<std::pair<size_t, char*>> free_by_size;
+  std::unordered_map<void*, std::pair<char*, size_t>> live;   // user ptr -> (block, size)
+  axr_register_fn reg = nullptr;
+  axr_unregister_fn unreg = nullptr;
+  void* user = nullptr;
+  uint64_t allocated = 0, peak = 0;
+
+  static constexpr size_t kGranule = 256;
+
+  void add_free(char* p, size_t n) {
+    // coalesce with the neighbours that lie in the same slab
+    auto next = free_by_addr.lower_bound(p);
+    if (next != free_by_addr.end() && p + n == next->first && same_slab(p, next->first)) {
+      n += next->second;
+      free_by_size.erase({next->second, next->first});
+      next = free_by_addr.erase(next);
+    }
+    if (next != free_by_addr.begin()) {
+      auto prev = std::prev(next);
+      if (prev->first + prev->second == p && same_slab(prev->first, p)) {
+        p = prev->first;
+        n += prev->second;
+        free_by_size.erase({prev->second, prev->first});
+        free_by_addr.erase(prev);
+      }
+    }
+    free_by_addr[p] = n;
+    free_by_size.insert({n, p});
+  }
+  Slab* slab_of(char* p) {
+    auto it = slabs.upper_bound(p);
+    if (it == slabs.begin()) return nullptr;
+    --it;
+    return (p < it->second.base + it->second.bytes) ? &it->second : nullptr;
+  }
+  bool same_slab(char* a, char* b) { return slab_of(a) == slab_of(b); }
+};
+
+namespace {
+
+struct DeviceGuard {
+  int prev = -1;
+  bool switched = false;
+  int enter(int device) {
+    int rc = check_hip(hipGetDevice(&prev), "hipGetDevice");
+    if (rc) return rc;
+    if (prev != device) {
+      rc = check_hip(hipSetDevice(device), "hipSetDevice");
+      if (rc) return rc;
+      switched = true;
+    }
+    return AXR_OK;
+  }
+  ~DeviceGuard() {
+    if (switched) (void)hipSetDevice(prev);
+  }
+};
+
+size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int pool_grow(axr_pool* pool, size_t need) {
+  size_t bytes = pool->slab_bytes > need ? pool->slab_bytes : round_up(need, 2u << 20);
+  DeviceGuard guard;
+  int rc = guard.enter(pool->device);
+  if (rc) return rc;
+  void* base = nullptr;
+  rc = check_hip(hipMalloc(&base, bytes), "hipMalloc(slab)");
+  if (rc) return rc;
+  axr_pool::Slab slab;
+  slab.base = static_cast<char*>(base);
+  slab.bytes = bytes;
+  if (pool->reg) {
+    const int rr = pool->reg(pool->user, base, bytes, &slab.mem_h);
+    if (rr != 0) {
+      (void)hipFree(base);
+      return fail(AXR_ERR_HIP, "slab registration callback failed with " + std::to_string(rr));
+    }
+  }
+  pool->slabs[slab.base] = slab;
+  pool->add_free(slab.base, bytes);
+  return AXR_OK;
+}
+
+void pool_release_slab(axr_pool* pool, axr_pool::Slab& slab) {
+  if (slab.mem_h && pool->unreg) pool->unreg(pool->user, slab.mem_h);
+  (void)hipFree(slab.base);
+}
+
+std::mutex g_default_pool_mu;
+std::map<int, axr_pool*> g_default_pools;
+
+}  // namespace
+
+extern "C" {
+
+// ---------------------------------------------------------------- status
+
+const char* axr_status_string(int status) {
+  switch (status) {
+    case AXR_OK: return "AXR_OK";
+    case AXR_ERR_INVALID: return "AXR_ERR_INVALID";
+    case AXR_ERR_NOMEM: return "AXR_ERR_NOMEM";
+    case AXR_ERR_HIP: return "AXR_ERR_HIP";
+    case AXR_ERR_LENGTH: return "AXR_ERR_LENGTH";
+    case AXR_ERR_UNSUPPORTED: return "AXR_ERR_UNSUPPORTED";
+    case AXR_ERR_NO_MESSAGE: return "AXR_ERR_NO_MESSAGE";
+    case AXR_ERR_NOT_IMPLEMENTED: return "AXR_ERR_NOT_IMPLEMENTED";
+    case AXR_ERR_HEADER: return "AXR_ERR_HEADER";
+    case AXR_ERR_MISMATCH: return "AXR_ERR_MISMATCH";
+    case AXR_ERR_NO_DEVICE: return "AXR_ERR_NO_DEVICE";
+    case AXR_ERR_BUSY: return "AXR_ERR_BUSY";
+    default: return "AXR_ERR_?";
+  }
+}
+
+const char* axr_last_error(void) { return g_last_error.c_str(); }
+
+const char* axr_version(void) { return "0.1.0"; }
+
+int axr_dl_device_to_memory_type(int32_t t) {
+  switch (t) {
+    case 2: return AXR_MEM_CUDA;
+    case 13: return AXR_MEM_CUDA_MANAGED;
+    case 10: return AXR_MEM_ROCM;
+    case 11: return AXR_MEM_ROCM_MANAGED;
+    case 1: return AXR_MEM_HOST;
+    default: return AXR_MEM_UNKNOWN;
+  }
+}
+
+int32_t axr_memory_type_to_dl_device(int m) {
+  switch (m) {
+    case AXR_MEM_CUDA: return 2;
+    case AXR_MEM_CUDA_MANAGED: return 13;
+    case AXR_MEM_ROCM: return 10;
+    case AXR_MEM_ROCM_MANAGED: return 11;
+    case AXR_MEM_ZE_HOST:
+    case AXR_MEM_ZE_DEVICE:
+    case AXR_MEM_ZE_MANAGED: return 14;
+    default: return 1;   // HOST, RDMA, UNKNOWN
+  }
+}
+
+int axr_tune_set(const char* key, int64_t value) {
+  if (!key) return fail(AXR_ERR_INVALID, "axr_tune_set: null key");
+  Tunables& t = tunables();
+  const std::string k(key);
+  if (k == "waves_per_cu") {
+    if (value < 1 || value > 64) return fail(AXR_ERR_INVALID, "waves_per_cu must be 1..64");
+    t.waves_per_cu = value;
+  } else if (k == "tile_rows") {
+    if (value != 4 && value != 8 && value != 16)
+      return fail(AXR_ERR_INVALID, "tile_rows must be 4, 8 or 16");
+    t.tile_rows = value;
+  } else if (k == "nontemporal") {
+    t.nontemporal = value ? 1 : 0;
+  } else if (k == "gather_run_bytes") {
+    if (value < 1) return fail(AXR_ERR_INVALID, "gather_run_bytes must be positive");
+    t.gather_run_bytes = value;
+  } else if (k == "min_tiles_per_wave") {
+    if (value < 1) return fail(AXR_ERR_INVALID, "min_tiles_per_wave must be positive");
+    t.min_tiles_per_wave = value;
+  } else {
+    return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
+  }
+  return AXR_OK;
+}
+
+int axr_tune_get(const char* key, int64_t* value) {
+  if (!key || !value) return fail(AXR_ERR_INVALID, "axr_tune_get: null argument");
+  const Tunables& t = tunables();
+  const std::string k(key);
+  if (k == "waves_per_cu") *value = t.waves_per_cu;
+  else if (k == "tile_rows") *value = t.tile_rows;
+  else if (k == "nontemporal") *value = t.nontemporal;
+  else if (k == "gather_run_bytes") *value = t.gather_run_bytes;
+  else if (k == "min_tiles_per_wave") *value = t.min_tiles_per_wave;
+  else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
+  return AXR_OK;
+}
+
+// ---------------------------------------------------------------- device
+
+int axr_device_count(int* count) {
+  if (!count) return fail(AXR_ERR_INVALID, "axr_device_count: null result");
+  *count = 0;
+  const hipError_t e = hipGetDeviceCount(count);
+  if (e == hipErrorNoDevice) {
+    *count = 0;
+    return AXR_OK;
+  }
+  return check_hip(e, "hipGetDeviceCount");
+}
+
+int axr_device_get(int* device) {
+  if (!device) return fail(AXR_ERR_INVALID, "axr_device_get: null result");
+  return check_hip(hipGetDevice(device), "hipGetDevice");
+}
+
+int axr_device_set(int device) { return check_hip(hipSetDevice(device), "hipSetDevice"); }
+
+int axr_device_push(int device, int* token) {
+  if (!token) return fail(AXR_ERR_INVALID, "axr_device_push: null token");
+  int prev = 0;
+  int rc = check_hip(hipGetDevice(&prev), "hipGetDevice");
+  if (rc) return rc;
+  rc = check_hip(hipSetDevice(device), "hipSetDevice");
+  if (rc) return rc;
+  *token = prev;
+  return AXR_OK;
+}
+
+int axr_device_pop(int token) { return check_hip(hipSetDevice(token), "hipSetDevice"); }
+
+int axr_device_synchronize(void) {
+  return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+}
+
+int axr_device_info(int* compute_units, uint64_t* total_mem, uint64_t* free_mem) {
+  if (compute_units) {
+    int rc = device_compute_units(compute_units);
+    if (rc) return rc;
+  }
+  if (total_mem || free_mem) {
+    size_t f = 0, t = 0;
+    int rc = check_hip(hipMemGetInfo(&f, &t), "hipMemGetInfo");
+    if (rc) return rc;
+    if (total_mem) *total_mem = t;
+    if (free_mem) *free_mem = f;
+  }
+  return AXR_OK;
+}
+
+int axr_stream_create(void** stream) {
+  if (!stream) return fail(AXR_ERR_INVALID, "axr_stream_create: null result");
+  hipStream_t s = nullptr;
+  // Default priority on purpose; non-blocking so it does not serialise with the null stream.
+  int rc = check_hip(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate");
+  if (rc) return rc;
+  *stream = s;
+  return AXR_OK;
+}
+
+int axr_stream_destroy(void* stream) {
+  if (!stream) return AXR_OK;
+  return check_hip(hipStreamDestroy(static_cast<hipStream_t>(stream)), "hipStreamDestroy");
+}
+
+int axr_stream_synchronize(void* stream) {
+  return check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)),
+                   "hipStreamSynchronize");
+}
+
+int axr_stream_wait_event(void* stream, void* event) {
+  if (!event) return fail(AXR_ERR_INVALID, "axr_stream_wait_event: null event");
+  return check_hip(hipStreamWaitEvent(static_cast<hipStream_t>(stream),
+                                      static_cast<hipEvent_t>(event), 0),
+                   "hipStreamWaitEvent");
+}
+
+int axr_event_create(void** event) {
+  if (!event) return fail(AXR_ERR_INVALID, "axr_event_create: null result");
+  hipEvent_t e = nullptr;
+  int rc = check_hip(hipEventCreate(&e), "hipEventCreate");
+  if (rc) return rc;
+  *event = e;
+  return AXR_OK;
+}
+
+int axr_event_destroy(void* event) {
+  if (!event) return AXR_OK;
+  return check_hip(hipEventDestroy(static_cast<hipEvent_t>(event)), "hipEventDestroy");
+}
+
+int axr_event_record(void* event, void* stream) {
+  if (!event) return fail(AXR_ERR_INVALID, "axr_event_record: null event");
+  return check_hip(hipEventRecord(static_cast<hipEvent_t>(event),
+                                  static_cast<hipStream_t>(stream)),
+                   "hipEventRecord");
+}
+
+int axr_event_synchronize(void* event) {
+  if (!event) return fail(AXR_ERR_INVALID, "axr_event_synchronize: null event");
+  return check_hip(hipEventSynchronize(static_cast<hipEvent_t>(event)), "hipEventSynchronize");
+}
+
+int axr_event_query(void* event, int* done) {
+  if (!event || !done) return fail(AXR_ERR_INVALID, "axr_event_query: null argument");
+  const hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
+  if (e == hipSuccess) {
+    *done = 1;
+    return AXR_OK;
+  }
+  if (e == hipErrorNotReady) {
+    *done = 0;
+    return AXR_OK;
+  }
+  return check_hip(e, "hipEventQuery");
+}
+
+int axr_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!start || !stop || !ms) return fail(AXR_ERR_INVALID, "axr_event_elapsed_ms: null argument");
+  return check_hip(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start),
+                                       static_cast<hipEvent_t>(stop)),
+                   "hipEventElapsedTime");
+}
+
+// ---------------------------------------------------------------- memory
+
+int axr_mem_alloc(int memory_type, size_t bytes, size_t alignment, void** ptr) {
+  if (!ptr) return fail(AXR_ERR_INVALID, "axr_mem_alloc: null result");
+  *ptr = nullptr;
+  switch (memory_type) {
+    case AXR_MEM_HOST: {
+      // std::malloc like the reference's device manager (ucx_cuda_memory_manager.hpp:93);
+      // over-aligned requests go through aligned_alloc.
+      void* p = nullptr;
+      if (alignment > alignof(max_align_t)) {
+        if (alignment & (alignment - 1)) return fail(AXR_ERR_INVALID, "alignment not a power of two");
+        p = std::aligned_alloc(alignment, round_up(bytes ? bytes : 1, alignment));
+      } else {
+        p = std::malloc(bytes ? bytes : 1);
+      }
+      if (!p) return fail(AXR_ERR_NOMEM, "host allocation failed");
+      *ptr = p;
+      return AXR_OK;
+    }
+    case AXR_MEM_ROCM: {
+      axr_pool_t* pool = nullptr;
+      int rc = axr_pool_default(&pool);
+      if (rc) return rc;
+      return axr_pool_alloc(pool, bytes, alignment, ptr, nullptr);
+    }
+    case AXR_MEM_ROCM_MANAGED: {
+      void* p = nullptr;
+      int rc = check_hip(hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault),
+                         "hipHostMalloc");
+      if (rc) return rc;
+      *ptr = p;
+      return AXR_OK;
+    }
+    default:
+      return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
+  }
+}
+
+int axr_mem_free(int memory_type, void* ptr, size_t /*bytes*/) {
+  if (!ptr) return AXR_OK;
+  switch (memory_type) {
+    case AXR_MEM_HOST:
+      std::free(ptr);
+      return AXR_OK;
+    case AXR_MEM_ROCM: {
+      // the block may come from any device's default pool
+      std::lock_guard<std::mutex> lock(g_default_pool_mu);
+      for (auto& kv : g_default_pools) {
+        if (axr_pool_free(kv.second, ptr) == AXR_OK) return AXR_OK;
+      }
+      return fail(AXR_ERR_INVALID, "axr_mem_free: pointer not owned by a default pool");
+    }
+    case AXR_MEM_ROCM_MANAGED:
+      return check_hip(hipHostFree(ptr), "hipHostFree");
+    default:
+      return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
+  }
+}
+
+static int copy_kind(int dst_type, int src_type, hipMemcpyKind* kind) {
+  auto is_host = [](int t) { return t == AXR_MEM_HOST || t == AXR_MEM_ROCM_MANAGED; };
+  auto is_dev = [](int t) { return t == AXR_MEM_ROCM; };
+  if (is_host(dst_type) && is_host(src_type)) *kind = hipMemcpyHostToHost;
+  else if (is_host(dst_type) && is_dev(src_type)) *kind = hipMemcpyDeviceToHost;
+  else if (is_dev(dst_type) && is_host(src_type)) *kind = hipMemcpyHostToDevice;
+  else if (is_dev(dst_type) && is_dev(src_type)) *kind = hipMemcpyDeviceToDevice;
+  else return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory copy combination");
+  return AXR_OK;
+}
+
+int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t bytes) {
+  if (bytes == 0) return AXR_OK;
+  if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_memcpy: null pointer");
+  hipMemcpyKind kind;
+  int rc = copy_kind(dst_type, src_type, &kind);
+  if (rc) return rc;
+  if (dst_type == AXR_MEM_HOST && src_type == AXR_MEM_HOST) {
+    std::memcpy(dst, src, bytes);
+    return AXR_OK;
+  }
+  return check_hip(hipMemcpy(dst, src, bytes, kind), "hipMemcpy");
+}
+
+int axr_memcpy_async(int dst_type, void* dst, int src_type, const void* src, size_t bytes,
+                     void* stream) {
+  if (bytes == 0) return AXR_OK;
+  if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_memcpy_async: null pointer");
+  hipMemcpyKind kind;
+  int rc = copy_kind(dst_type, src_type, &kind);
+  if (rc) return rc;
+  return check_hip(hipMemcpyAsync(dst, src, bytes, kind, static_cast<hipStream_t>(stream)),
+                   "hipMemcpyAsync");
+}
+
+int axr_memset_async(void* dst, int value, size_t bytes, void* stream) {
+  if (bytes == 0) return AXR_OK;
+  if (!dst) return fail(AXR_ERR_INVALID, "axr_memset_async: null pointer");
+  return launch_fill(dst, value, bytes, stream);
+}
+
+// ---------------------------------------------------------------- pool
+
+int axr_pool_create(int device, size_t slab_bytes, axr_pool_t** pool) {
+  if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_create: null result");
+  int count = 0;
+  int rc = axr_device_count(&count);
+  if (rc) return rc;
+  if (device < 0 || device >= count)
+    return fail(AXR_ERR_NO_DEVICE, "axr_pool_create: no such device " + std::to_string(device));
+  axr_pool* p = new (std::nothrow) axr_pool();
+  if (!p) return fail(AXR_ERR_NOMEM, "axr_pool_create: out of host memory");
+  p->device = device;
+  p->slab_bytes = slab_bytes ? round_up(slab_bytes, 2u << 20) : (256u << 20);
+  *pool = p;
+  return AXR_OK;
+}
+
+int axr_pool_destroy(axr_pool_t* pool) {
+  if (!pool) return AXR_OK;
+  {
+    std::lock_guard<std::mutex> lock(pool->mu);
+    if (!pool->live.empty()) return fail(AXR_ERR_BUSY, "axr_pool_destroy: blocks still allocated");
+    DeviceGuard guard;
+    (void)guard.enter(pool->device);
+    for (auto& kv : pool->slabs) pool_release_slab(pool, kv.second);
+    pool->slabs.clear();
+  }
+  delete pool;
+  return AXR_OK;
+}
+
+int axr_pool_default(axr_pool_t** pool) {
+  if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_default: null result");
+  int dev = 0;
+  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lock(g_default_pool_mu);
+  auto it = g_default_pools.find(dev);
+  if (it == g_default_pools.end()) {
+    axr_pool_t* p = nullptr;
+    rc = axr_pool_create(dev, 0, &p);
+    if (rc) return rc;
+    it = g_default_pools.emplace(dev, p).first;
+  }
+  *pool = it->second;
+  return AXR_OK;
+}
+
+int axr_pool_set_registrar(axr_pool_t* pool, axr_register_fn reg, axr_unregister_fn unreg,
+                           void* user) {
+  if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_set_registrar: null pool");
+  std::lock_guard<std::mutex> lock(pool->mu);
+  if (!pool->slabs.empty())
+    return fail(AXR_ERR_BUSY, "axr_pool_set_registrar: pool already holds slabs");
+  pool->reg = reg;
+  pool->unreg = unreg;
+  pool->user = user;
+  return AXR_OK;
+}
+
+int axr_pool_alloc(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr, void** mem_h) {
+  if (!pool || !ptr) return fail(AXR_ERR_INVALID, "axr_pool_alloc: null argument");
+  *ptr = nullptr;
+  if (mem_h) *mem_h = nullptr;
+  if (alignment == 0) alignment = 1;
+  if (alignment & (alignment - 1)) return fail(AXR_ERR_INVALID, "alignment not a power of two");
+  const size_t g = axr_pool::kGranule;
+  const size_t need = round_up(bytes ? bytes : 1, g);
+  // Blocks start on 256-byte boundaries; larger alignments over-allocate and shift.
+  const size_t slack = alignment > g ? alignment : 0;
+  std::lock_guard<std::mutex> lock(pool->mu);
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    auto it = pool->free_by_size.lower_bound({need + slack, nullptr});
+    if (it != pool->free_by_size.end()) {
+      char* block = it->second;
+      const size_t have = it->first;
+      pool->free_by_size.erase(it);
+      pool->free_by_addr.erase(block);
+      char* user_ptr = block;
+      if (slack) {
+        user_ptr = reinterpret_cast<char*>(
+            round_up(reinterpret_cast<uintptr_t>(block), alignment));
+      }
+      const size_t used = static_cast<size_t>(user_ptr - block) + need;
+      if (have > used) pool->add_free(block + used, have - used);
+      pool->live[user_ptr] = {block, used};
+      axr_pool::Slab* slab = pool->slab_of(block);
+      slab->live++;
+      pool->allocated += used;
+      if (pool->allocated > pool->peak) pool->peak = pool->allocated;
+      *ptr = user_ptr;
+      if (mem_h) *mem_h = slab->mem_h;
+      return AXR_OK;
+    }
+    int rc = pool_grow(pool, need + slack);
+    if (rc) return rc;
+  }
+  return fail(AXR_ERR_NOMEM, "axr_pool_alloc: no block after growing the pool");
+}
+
+int axr_pool_free(axr_pool_t* pool, void* ptr) {
+  if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_free: null pool");
+  if (!ptr) return AXR_OK;
+  std::lock_guard<std::mutex> lock(pool->mu);
+  auto it = pool->live.find(ptr);
+  if (it == pool->live.end()) return fail(AXR_ERR_INVALID, "axr_pool_free: unknown pointer");
+  char* block = it->second.first;
+  const size_t used = it->second.second;
+  pool->live.erase(it);
+  pool->slab_of(block)->live--;
+  pool->allocated -= used;
+  pool->add_free(block, used);
+  return AXR_OK;
+}
+
+int axr_pool_trim(axr_pool_t* pool) {
+  if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_trim: null pool");
+  std::lock_guard<std::mutex> lock(pool->mu);
+  DeviceGuard guard;
+  int rc = guard.enter(pool->device);
+  if (rc) return rc;
+  for (auto it = pool->slabs.begin(); it != pool->slabs.end();) {
+    axr_pool::Slab& slab = it->second;
+    if (slab.live == 0) {
+      // the slab is one coalesced free block
+      auto fb = pool->free_by_addr.find(slab.base);
+      if (fb != pool->free_by_addr.end() && fb->second == slab.bytes) {
+        pool->free_by_size.erase({fb->second, fb->first});
+        pool->free_by_addr.erase(fb);
+        pool_release_slab(pool, slab);
+        it = pool->slabs.erase(it);
+        continue;
+      }
+    }
+    ++it;
+  }
+  return AXR_OK;
+}
+
+int axr_pool_get_stats(axr_pool_t* pool, axr_pool_stats_t* stats) {
+  if (!pool || !stats) return fail(AXR_ERR_INVALID, "axr_pool_get_stats: null argument");
+  std::lock_guard<std::mutex> lock(pool->mu);
+  stats->slabs = pool->slabs.size();
+  stats->slab_bytes = 0;
+  for (auto& kv : pool->slabs) stats->slab_bytes += kv.second.bytes;
+  stats->allocated_bytes = pool->allocated;
+  stats->live_blocks = pool->live.size();
+  stats->peak_bytes = pool->peak;
+  return AXR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,251 @@
+"""DLPack in and out, without a compiled Python extension.
+
+Mirrors the reference's ``axon/python/src/dlpack_helpers.cpp``:
+
+* ``extract``  <- ExtractDlpackTensor (:136-156) + ExtractTensorMetaFromDlm
+  (:696-724): call ``obj.__dlpack__()``, keep the capsule as the owner, read
+  device / dtype / ndim / shape / strides / byte_offset.
+* ``DLPackExport`` <- DLPackCapsuleWrapper (dlpack_helpers.hpp:63-170): an
+  object with ``__dlpack__`` and ``__dlpack_device__`` over memory the bundle
+  path owns, consumable once by ``torch.from_dlpack`` / ``numpy.from_dlpack``.
+
+kDLROCM (10), kDLROCMHost (11) and kDLCPU (1) tensors are accepted; the
+reference maps kDLROCM to ucx_memory_type::ROCM (:92-97, :123-126) but its
+runtime refuses a rocm device (bindings_runtime.cpp:131-141).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Any, Callable, List, Optional, Sequence, Tuple
+
+from . import _capi
+
+_py = C.pythonapi
+_py.PyCapsule_IsValid.restype = C.c_int
+_py.PyCapsule_IsValid.argtypes = [C.py_object, C.c_char_p]
+_py.PyCapsule_GetPointer.restype = C.c_void_p
+_py.PyCapsule_GetPointer.argtypes = [C.py_object, C.c_char_p]
+_py.PyCapsule_SetName.restype = C.c_int
+_py.PyCapsule_SetName.argtypes = [C.py_object, C.c_char_p]
+_CAPSULE_DTOR = C.CFUNCTYPE(None, C.c_void_p)
+_py.PyCapsule_New.restype = C.py_object
+_py.PyCapsule_New.argtypes = [C.c_void_p, C.c_char_p, _CAPSULE_DTOR]
+# Variants that take the capsule as a raw address: inside a capsule destructor
+# the object's reference count is already zero and must not be touched.
+_raw_is_valid = C.PYFUNCTYPE(C.c_int, C.c_void_p, C.c_char_p)(("PyCapsule_IsValid", _py))
+_raw_get_pointer = C.PYFUNCTYPE(C.c_void_p, C.c_void_p, C.c_char_p)(("PyCapsule_GetPointer", _py))
+
+_NAME = b"dltensor"
+_NAME_USED = b"used_dltensor"
+_NAME_VERSIONED = b"dltensor_versioned"
+
+
+class _ManagedTensor(C.Structure):
+    pass
+
+
+_DELETER = C.CFUNCTYPE(None, C.POINTER(_ManagedTensor))
+_ManagedTensor._fields_ = [
+    ("dl_tensor", _capi.Tensor),
+    ("manager_ctx", C.c_void_p),
+    ("deleter", _DELETER),
+]
+
+
+class _ManagedTensorVersioned(C.Structure):
+    _fields_ = [
+        ("major", C.c_uint32),
+        ("minor", C.c_uint32),
+        ("manager_ctx", C.c_void_p),
+        ("deleter", C.c_void_p),
+        ("flags", C.c_uint64),
+        ("dl_tensor", _capi.Tensor),
+    ]
+
+
+@dataclass
+class TensorView:
+    """Plain description of one tensor, the Python face of ``axr_tensor_t``.
+
+    ``owner`` keeps the producer's memory alive (the reference holds the
+    capsule in the buffer's release function, dlpack_helpers.cpp:739-742).
+    """
+
+    data: int
+    device_type: int
+    device_id: int
+    dtype: Tuple[int, int, int]  # (code, bits, lanes)
+    shape: Tuple[int, ...]
+    strides: Optional[Tuple[int, ...]]  # elements; None = compact row-major
+    byte_offset: int = 0
+    owner: Any = None
+
+    @property
+    def ndim(self) -> int:
+        return len(self.shape)
+
+    @property
+    def itemsize(self) -> int:
+        return (self.dtype[1] + 7) // 8
+
+    @property
+    def nbytes(self) -> int:
+        # CalculateTensorSize, rpc_core/utils/tensor_meta.hpp:91-104
+        if self.ndim == 0:
+            return 0
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n * self.itemsize
+
+
+def _read(dl: _capi.Tensor, owner: Any) -> TensorView:
+    nd = dl.ndim
+    shape = tuple(dl.shape[i] for i in range(nd))
+    strides = tuple(dl.strides[i] for i in range(nd)) if dl.strides else None
+    return TensorView(
+        data=dl.data or 0,
+        device_type=dl.device_type,
+        device_id=dl.device_id,
+        dtype=(dl.dtype_code, dl.dtype_bits, dl.dtype_lanes),
+        shape=shape,
+        strides=strides,
+        byte_offset=dl.byte_offset,
+        owner=owner,
+    )
+
+
+def extract(obj: Any) -> TensorView:
+    """Describe ``obj`` (anything with ``__dlpack__``, or a capsule)."""
+    if isinstance(obj, TensorView):
+        return obj
+    capsule = obj
+    if hasattr(obj, "__dlpack__"):
+        capsule = obj.__dlpack__()
+    if _py.PyCapsule_IsValid(capsule, _NAME):
+        ptr = _py.PyCapsule_GetPointer(capsule, _NAME)
+        managed = C.cast(ptr, C.POINTER(_ManagedTensor)).contents
+        # the capsule stays unconsumed: dropping it runs the producer's deleter
+        return _read(managed.dl_tensor, (capsule, obj))
+    if _py.PyCapsule_IsValid(capsule, _NAME_VERSIONED):
+        ptr = _py.PyCapsule_GetPointer(capsule, _NAME_VERSIONED)
+        managed = C.cast(ptr, C.POINTER(_ManagedTensorVersioned)).contents
+        return _read(managed.dl_tensor, (capsule, obj))
+    raise TypeError(
+        "object does not provide a DLPack capsule named 'dltensor' "
+        f"(got {type(obj).__name__})"
+    )
+
+
+def extract_many(objs: Sequence[Any]) -> List[TensorView]:
+    return [extract(o) for o in objs]
+
+
+class TensorArray:
+    """A C array of ``axr_tensor_t`` plus the shape/stride storage it points to."""
+
+    def __init__(self, views: Sequence[TensorView]):
+        self.views = list(views)
+        n = len(self.views)
+        self.array = (_capi.Tensor * max(n, 1))()
+        total = sum(v.ndim * (2 if v.strides is not None else 1) for v in self.views)
+        self._dims = (C.c_int64 * max(total, 1))()
+        base = C.addressof(self._dims)
+        at = 0
+        for i, v in enumerate(self.views):
+            t = self.array[i]
+            t.data = v.data
+            t.device_type = v.device_type
+            t.device_id = v.device_id
+            t.ndim = v.ndim
+            t.dtype_code, t.dtype_bits, t.dtype_lanes = v.dtype
+            t.byte_offset = v.byte_offset
+            nd = v.ndim
+            if nd:
+                self._dims[at:at + nd] = v.shape
+                t.shape = C.cast(base + 8 * at, C.POINTER(C.c_int64))
+                at += nd
+                if v.strides is not None:
+                    self._dims[at:at + nd] = v.strides
+                    t.strides = C.cast(base + 8 * at, C.POINTER(C.c_int64))
+                    at += nd
+        self.count = n
+
+    def pointer(self):
+        return C.cast(self.array, C.POINTER(_capi.Tensor))
+
+
+# ---------------------------------------------------------------- export
+
+_live_exports = {}  # id -> (managed struct, shape array, release callback)
+_next_export = [1]
+
+
+@_DELETER
+def _managed_deleter(ptr):  # called by the consumer when it drops the tensor
+    key = ptr.contents.manager_ctx
+    entry = _live_exports.pop(key, None)
+    if entry is not None and entry[3] is not None:
+        entry[3]()
+
+
+@_CAPSULE_DTOR
+def _capsule_destructor(capsule_ptr):
+    # runs when a capsule is collected; an unconsumed one still owns the tensor
+    if _raw_is_valid(capsule_ptr, _NAME):
+        ptr = _raw_get_pointer(capsule_ptr, _NAME)
+        managed = C.cast(ptr, C.POINTER(_ManagedTensor))
+        managed.contents.deleter(managed)
+
+
+class DLPackExport:
+    """Single-consume DLPack producer over memory owned by this package.
+
+    ``release`` runs once, when the consumer (or an unconsumed capsule) lets go.
+    """
+
+    def __init__(self, data: int, nbytes_or_shape, dtype: Tuple[int, int, int], device_type: int,
+                 device_id: int = 0, release: Optional[Callable[[], None]] = None):
+        self._data = data
+        self._shape = tuple(nbytes_or_shape) if not isinstance(nbytes_or_shape, int) else (nbytes_or_shape,)
+        self._dtype = dtype
+        self._device = (device_type, device_id)
+        self._release = release
+        self._consumed = False
+
+    def __dlpack_device__(self):
+        return self._device
+
+    def __dlpack__(self, stream=None, max_version=None, dl_device=None, copy=None):
+        if self._consumed:
+            raise RuntimeError("DLPack capsule can only be consumed once")
+        if copy:
+            raise BufferError("this producer cannot copy")
+        self._consumed = True
+        nd = len(self._shape)
+        shape = (C.c_int64 * max(nd, 1))(*self._shape)
+        managed = _ManagedTensor()
+        dl = managed.dl_tensor
+        dl.data = self._data
+        dl.device_type, dl.device_id = self._device
+        dl.ndim = nd
+        dl.dtype_code, dl.dtype_bits, dl.dtype_lanes = self._dtype
+        dl.shape = C.cast(shape, C.POINTER(C.c_int64))
+        dl.strides = None
+        dl.byte_offset = 0
+        key = _next_export[0]
+        _next_export[0] += 1
+        managed.manager_ctx = key
+        managed.deleter = _managed_deleter
+        _live_exports[key] = (managed, shape, self, self._release)
+        return _py.PyCapsule_New(C.addressof(managed), _NAME, _capsule_destructor)
+
+    def __del__(self):
+        if not self._consumed and self._release is not None:
+            release, self._release = self._release, None
+            release()
+
+
+# DLPack dtype codes
+kDLInt, kDLUInt, kDLFloat, kDLBfloat, kDLBool = 0, 1, 2, 4, 6

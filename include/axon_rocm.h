@@ -1,0 +1,334 @@
+/*
+ * axon_rocm.h - C ABI of the MI355X (gfx950) tensor-bundle path for execution-ucx.
+ *
+ * The library behind this header replaces, for ROCm memory, the part of the
+ * reference that moves tensor payload bytes:
+ *
+ *   - the IOV gather done inside UCX when a tensor list is sent
+ *     (ucx_context/ucx_connection.cpp:401-426, send_am_iov_data) becomes ONE
+ *     pack kernel into a contiguous HBM buffer that is then sent as a plain
+ *     contiguous ucx_am_data (ucx_connection.cpp:353-374);
+ *   - the IOV scatter on receive (ucx_connection.cpp:428-453) becomes ONE
+ *     unpack kernel out of the contiguous receive buffer;
+ *   - ucx_context/cuda/ucx_cuda_memory_manager.hpp (cudaMalloc/cudaMemcpy) is
+ *     replaced by a hipMalloc slab pool + copy table (axr_pool_*, axr_memcpy*);
+ *   - ucx_context/cuda/ucx_cuda_context.hpp (cuCtxPushCurrent/PopCurrent) is
+ *     replaced by axr_device_push / axr_device_pop.
+ *
+ * Conventions: every function returns 0 (AXR_OK) or a negative axr_status
+ * value, never throws and never aborts.  All entry points are thread-safe
+ * unless stated.  Streams and events are opaque pointers (hipStream_t /
+ * hipEvent_t underneath); a NULL stream is the device's default stream.
+ * No HIP, torch or UCX type appears in a signature.
+ */
+#ifndef AXON_ROCM_H_
+#define AXON_ROCM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AXR_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ status */
+
+typedef enum axr_status {
+  AXR_OK = 0,
+  AXR_ERR_INVALID = -1,         /* bad argument (null pointer, bad shape ...)   */
+  AXR_ERR_NOMEM = -2,           /* host or device allocation failed             */
+  AXR_ERR_HIP = -3,             /* a HIP runtime call failed (see last error)   */
+  AXR_ERR_LENGTH = -4,          /* sizes exceed the buffer they must fit in;
+                                   the reference throws std::length_error here
+                                   (ucx_context/ucx_context_data.hpp:644-646)   */
+  AXR_ERR_UNSUPPORTED = -5,     /* memory type / layout this build cannot move;
+                                   the reference throws std::runtime_error
+                                   ("Unsupported memory type",
+                                   cuda/ucx_cuda_memory_manager.hpp:103,150)    */
+  AXR_ERR_NO_MESSAGE = -6,      /* unknown receive key; UCS_ERR_NO_MESSAGE in
+                                   ucx_am_context.hpp:1570-1574                 */
+  AXR_ERR_NOT_IMPLEMENTED = -7, /* recv_buffer on an eager message;
+                                   UCS_ERR_NOT_IMPLEMENTED, :1643-1651          */
+  AXR_ERR_HEADER = -8,          /* malformed bundle header                      */
+  AXR_ERR_MISMATCH = -9,        /* bound tensors do not match the plan's metas  */
+  AXR_ERR_NO_DEVICE = -10,      /* no usable ROCm device in this process        */
+  AXR_ERR_BUSY = -11            /* object still has work in flight              */
+} axr_status_t;
+
+/* Human-readable name of a status code (static storage). */
+AXR_API const char* axr_status_string(int status);
+/* Message of the last failure on the calling thread (thread-local storage). */
+AXR_API const char* axr_last_error(void);
+/* Library version, "major.minor.patch". */
+AXR_API const char* axr_version(void);
+
+/* ------------------------------------------------------------ memory types */
+
+/* Same numbering as ucx_memory_type_t (ucx_context/ucx_context_def.h:27-39),
+ * so values can be passed through unchanged. */
+typedef enum axr_memory_type {
+  AXR_MEM_HOST = 0,
+  AXR_MEM_CUDA = 1,
+  AXR_MEM_CUDA_MANAGED = 2,
+  AXR_MEM_ROCM = 3,
+  AXR_MEM_ROCM_MANAGED = 4,
+  AXR_MEM_RDMA = 5,
+  AXR_MEM_ZE_HOST = 6,
+  AXR_MEM_ZE_DEVICE = 7,
+  AXR_MEM_ZE_MANAGED = 8,
+  AXR_MEM_UNKNOWN = 9
+} axr_memory_type_t;
+
+/* DLPack device type -> memory type and back, the tables of
+ * axon/python/src/dlpack_helpers.cpp:82-134 (kDLROCM=10 <-> ROCM,
+ * kDLROCMHost=11 <-> ROCM_MANAGED, kDLCPU=1 <-> HOST, kDLCUDA=2 <-> CUDA,
+ * kDLCUDAManaged=13 <-> CUDA_MANAGED, kDLOneAPI=14 -> UNKNOWN, else UNKNOWN). */
+AXR_API int axr_dl_device_to_memory_type(int32_t dl_device_type);
+AXR_API int32_t axr_memory_type_to_dl_device(int memory_type);
+
+/* ----------------------------------------------------------------- tensors */
+
+/* Layout-identical to DLTensor (dlpack.h, v0.8 / v1.x): a binding may pass
+ * &managed->dl_tensor copied into an array of these.  `strides` (in elements)
+ * may be NULL for a compact row-major tensor, as DLPack allows. */
+typedef struct axr_tensor {
+  void* data;
+  int32_t device_type; /* DLDeviceType: 1 CPU, 10 ROCM, 11 ROCMHost ...        */
+  int32_t device_id;
+  int32_t ndim;
+  uint8_t dtype_code; /* DLDataTypeCode: 0 int, 1 uint, 2 float, 4 bfloat ...  */
+  uint8_t dtype_bits;
+  uint16_t dtype_lanes;
+  int64_t* shape;
+  int64_t* strides;
+  uint64_t byte_offset;
+} axr_tensor_t;
+
+/* Same as ucx_buffer_t (ucx_context/ucx_context_def.h:58-61). */
+typedef struct axr_buffer {
+  void* data;
+  size_t size;
+} axr_buffer_t;
+
+/* Bytes a tensor occupies in a bundle: prod(shape) * ceil(bits/8), 0 when
+ * ndim == 0, lanes and strides ignored.  Restates CalculateTensorSize
+ * (rpc_core/utils/tensor_meta.hpp:91-104).  Negative extents -> AXR_ERR_INVALID. */
+AXR_API int axr_tensor_nbytes(const axr_tensor_t* t, uint64_t* nbytes);
+
+/* ------------------------------------------------------------------ device */
+
+AXR_API int axr_device_count(int* count);
+AXR_API int axr_device_get(int* device);
+AXR_API int axr_device_set(int device);
+/* Thread-level activation used by the ROCm UcxAutoDeviceContext: push makes
+ * `device` current on the calling thread and returns the previous one in
+ * *token; pop restores it.  Replaces cuCtxPushCurrent / cuCtxPopCurrent of
+ * ucx_context/cuda/ucx_cuda_context.hpp:55-72. */
+AXR_API int axr_device_push(int device, int* token);
+AXR_API int axr_device_pop(int token);
+AXR_API int axr_device_synchronize(void);
+/* Compute units and bytes of device memory of the current device. */
+AXR_API int axr_device_info(int* compute_units, uint64_t* total_mem, uint64_t* free_mem);
+
+AXR_API int axr_stream_create(void** stream);
+AXR_API int axr_stream_destroy(void* stream);
+AXR_API int axr_stream_synchronize(void* stream);
+/* Make `stream` wait for `event` (hipStreamWaitEvent). */
+AXR_API int axr_stream_wait_event(void* stream, void* event);
+
+AXR_API int axr_event_create(void** event);
+AXR_API int axr_event_destroy(void* event);
+AXR_API int axr_event_record(void* event, void* stream);
+AXR_API int axr_event_synchronize(void* event);
+/* 1 in *done when the event has completed, 0 when still pending. */
+AXR_API int axr_event_query(void* event, int* done);
+AXR_API int axr_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ------------------------------------------------------------------ memory */
+
+/* allocate / deallocate / memcpy of UcxMemoryResourceManager
+ * (ucx_context/ucx_memory_resource.hpp:99-123) for one memory type each:
+ * HOST -> malloc'ed pageable memory, ROCM -> device memory from the process
+ * default pool (axr_pool_default), ROCM_MANAGED -> pinned, device-visible host
+ * memory.  Other types -> AXR_ERR_UNSUPPORTED. */
+AXR_API int axr_mem_alloc(int memory_type, size_t bytes, size_t alignment, void** ptr);
+AXR_API int axr_mem_free(int memory_type, void* ptr, size_t bytes);
+/* Blocking copy between any two of HOST / ROCM / ROCM_MANAGED; the table
+ * of ucx_cuda_memory_manager.hpp:62-78 extended with the pinned type. */
+AXR_API int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t bytes);
+/* Same, enqueued on `stream`; pageable host memory makes it synchronous. */
+AXR_API int axr_memcpy_async(int dst_type, void* dst, int src_type, const void* src,
+                             size_t bytes, void* stream);
+/* Fill `bytes` bytes with `value` on `stream` (fill kernel, safe to capture). */
+AXR_API int axr_memset_async(void* dst, int value, size_t bytes, void* stream);
+
+/* ------------------------------------------------------------- device pool */
+
+typedef struct axr_pool axr_pool_t;
+
+/* Called once per slab the pool obtains from hipMalloc / before it returns
+ * the slab with hipFree.  The C++ memory resource wires these to
+ * ucx_am_context::register_ucx_memory / unregister_ucx_memory
+ * (ucx_context/ucx_am_context/ucx_am_context.cpp:1128-1147, ucp_mem_map) so a
+ * whole slab is registered once and every allocation carved from it carries
+ * the slab's ucp_mem_h. */
+typedef int (*axr_register_fn)(void* user, void* addr, size_t length, void** mem_h);
+typedef void (*axr_unregister_fn)(void* user, void* mem_h);
+
+/* Pool of device memory on `device`: slabs of at least `slab_bytes` (0 = 256 MiB
+ * default), carved at 256-byte granularity, freed blocks coalesced. */
+AXR_API int axr_pool_create(int device, size_t slab_bytes, axr_pool_t** pool);
+/* Fails with AXR_ERR_BUSY while allocations are outstanding. */
+AXR_API int axr_pool_destroy(axr_pool_t* pool);
+/* Process-wide pool of the current device, created on first use. */
+AXR_API int axr_pool_default(axr_pool_t** pool);
+AXR_API int axr_pool_set_registrar(axr_pool_t* pool, axr_register_fn reg,
+                                   axr_unregister_fn unreg, void* user);
+/* *mem_h (may be NULL) receives the registration handle of the slab the
+ * block lies in, NULL when no registrar is installed; it is what goes into
+ * ucx_am_data_t::mem_h (ucx_context/ucx_context_def.h:80-93). */
+AXR_API int axr_pool_alloc(axr_pool_t* pool, size_t bytes, size_t alignment,
+                           void** ptr, void** mem_h);
+AXR_API int axr_pool_free(axr_pool_t* pool, void* ptr);
+/* Return fully free slabs to the driver. */
+AXR_API int axr_pool_trim(axr_pool_t* pool);
+
+typedef struct axr_pool_stats {
+  uint64_t slabs;
+  uint64_t slab_bytes;      /* bytes held from the driver                     */
+  uint64_t allocated_bytes; /* bytes handed out (rounded to 256)              */
+  uint64_t live_blocks;
+  uint64_t peak_bytes;
+} axr_pool_stats_t;
+AXR_API int axr_pool_get_stats(axr_pool_t* pool, axr_pool_stats_t* stats);
+
+/* ------------------------------------------------------------ bundle plans */
+
+typedef struct axr_plan axr_plan_t;
+
+/* Sender side.  Lays the n tensors out in argument order (the order
+ * InvokeContext::add_tensor establishes,
+ * axon/python/src/bindings_runtime_helpers.hpp:351-414):
+ *   offset[0] = 0, offset[i+1] = align_up(offset[i] + nbytes[i], align).
+ * align == 1 is the reference layout: what a contiguous receiver sees after
+ * an IOV send (ucx_am_connection_test.cpp:1051-1108) and what
+ * UcxBuffer::to_buffer_vec splits (ucx_context_data.hpp:641-665).
+ * align must be a power of two <= 4096.  Gap bytes are written as zero by
+ * axr_pack.  Tensors may be strided views (strides != NULL, not row-major):
+ * they are packed as their C-order element sequence; the reference would
+ * ship the first nbytes of storage instead (dlpack_helpers.cpp:776-780).
+ * Every tensor must be device-accessible (kDLROCM / kDLROCMHost) or kDLCPU;
+ * kDLCPU tensors are moved with hipMemcpyAsync, one copy per contiguous run.
+ * The plan copies shapes and strides; `tensors` may be freed on return. */
+AXR_API int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align,
+                            uint32_t flags, axr_plan_t** plan);
+AXR_API int axr_plan_free(axr_plan_t* plan);
+
+AXR_API int axr_plan_num_tensors(const axr_plan_t* plan, size_t* n);
+/* Bytes of the packed buffer, gaps included. */
+AXR_API int axr_plan_payload_bytes(const axr_plan_t* plan, uint64_t* bytes);
+/* Sum of tensor sizes (gaps excluded): the algorithmic payload P. */
+AXR_API int axr_plan_data_bytes(const axr_plan_t* plan, uint64_t* bytes);
+/* offsets[i], sizes[i] for i < n; either array may be NULL. */
+AXR_API int axr_plan_layout(const axr_plan_t* plan, uint64_t* offsets, uint64_t* sizes);
+/* Metadata of tensor i with data == NULL, byte_offset == 0 and shape/strides
+ * pointing into the plan (valid until axr_plan_free).  On a plan made by
+ * axr_plan_from_header strides is NULL: packed tensors are compact. */
+AXR_API int axr_plan_tensor_meta(const axr_plan_t* plan, size_t i, axr_tensor_t* meta);
+
+/* Serialised per-tensor header (offset, size, device, dtype, shape) that
+ * travels as the AM header next to the payload; it carries the fields of
+ * TensorMeta (rpc_core/utils/tensor_meta.hpp:77-82) with byte_offset fixed at
+ * 0.  Little-endian, fixed layout, documented in axr_plan.cpp.  The pointer is
+ * owned by the plan. */
+AXR_API int axr_plan_header(const axr_plan_t* plan, const void** header, size_t* length);
+
+/* Receiver side: rebuild the layout from a received header.  The plan has no
+ * tensor addresses until axr_plan_bind. */
+AXR_API int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan);
+/* Attach (or replace) the tensor-side addresses: sources for axr_pack,
+ * destinations for axr_unpack.  dtype bits and shape of tensors[i] must give
+ * the same nbytes and element size as the plan's tensor i; strides may differ
+ * (unpack into views).  Overlapping destinations (a stride of 0 on an extent
+ * above 1) are refused for unpack. */
+AXR_API int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n);
+
+/* Zero-copy receive mode: views[i] = {payload + offset[i], nbytes[i]}, the
+ * result of UcxBuffer::to_buffer_vec(sizes) (ucx_context_data.hpp:641-665).
+ * AXR_ERR_LENGTH when the plan needs more than payload_bytes. */
+AXR_API int axr_plan_split(const axr_plan_t* plan, void* payload, size_t payload_bytes,
+                           axr_buffer_t* views);
+
+/* Gather the bound tensors into payload[0, payload_bytes) / scatter payload
+ * into the bound tensors, asynchronously on `stream`.  `payload` must be
+ * device-accessible memory; payload_bytes must be >= axr_plan_payload_bytes
+ * (AXR_ERR_LENGTH otherwise).  The first call uploads the plan's device
+ * tables on the same stream.  A plan may be packed/unpacked any number of
+ * times; concurrent calls on one plan from two threads are not allowed. */
+AXR_API int axr_pack(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream);
+AXR_API int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes,
+                       void* stream);
+
+/* Launch geometry of a plan's kernel, for profiling reports. */
+typedef struct axr_launch_info {
+  uint32_t workgroups;
+  uint32_t threads_per_workgroup;
+  uint32_t tiles;          /* work units the kernel walks                     */
+  uint32_t tile_bytes;
+  uint32_t segments;       /* device segment-table entries                    */
+  uint32_t table_bytes;    /* device table size                               */
+  uint32_t host_copies;    /* hipMemcpyAsync calls used for kDLCPU tensors     */
+  uint32_t reserved;
+} axr_launch_info_t;
+AXR_API int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info);
+
+/* One entry of the device segment table, for inspection and tests. */
+typedef struct axr_segment_info {
+  uint32_t tensor;        /* index of the tensor the segment belongs to       */
+  uint32_t mode;          /* 0 one run, 1 strided run tiles, 2 strided
+                             elements, 3 zero fill only, 4 host copy          */
+  uint64_t address;       /* tensor-side address of the first element         */
+  uint64_t offset;        /* payload offset                                   */
+  uint64_t run_bytes;     /* contiguous bytes per run                         */
+  uint64_t nbytes;        /* bytes of the whole segment                       */
+  uint32_t pad;           /* zero bytes written after the segment by pack     */
+  uint32_t ndim;          /* strided outer dimensions (<= 6)                  */
+  uint32_t granule;       /* mode 2: bytes per lane access                    */
+  uint32_t tiles;
+  uint32_t shape[6];
+  int64_t stride_bytes[6];
+} axr_segment_info_t;
+/* Copies up to `capacity` entries into out (may be NULL) and stores the total
+ * number in *count.  Works without a device (the grid is then sized for 256
+ * compute units). */
+AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity,
+                              size_t* count);
+
+/* Tuning knobs (process-wide, read at plan creation): "waves_per_cu",
+ * "tile_rows", "nontemporal", "gather_run_bytes".  Unknown key -> INVALID. */
+AXR_API int axr_tune_set(const char* key, int64_t value);
+AXR_API int axr_tune_get(const char* key, int64_t* value);
+
+/* -------------------------------------------------- verification utilities */
+
+/* data[i] /= 2.0f in place; the device-side "process" step of the reference's
+ * send -> process -> reply tests
+ * (ucx_am_context/ucx_am_context_test_cuda_helper.cu:23-78). */
+AXR_API int axr_divide_by_two(float* data, size_t count, void* stream);
+/* Number of differing bytes between two device-accessible ranges (blocking). */
+AXR_API int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mismatches);
+/* Position-weighted checksum: sum over bytes b[i] * (1 + ((start + i) mod 65521))
+ * mod 2^64 (blocking).  Additive over a split of the range, so the checksum of
+ * a packed buffer equals the sum of its tensors' checksums taken with
+ * start = offset[i]. */
+AXR_API int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum);
+/* Plain device copy kernel (16 B per lane, grid-stride); calibration
+ * reference for profiler counters and bandwidth. */
+AXR_API int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXON_ROCM_H_ */

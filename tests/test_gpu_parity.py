@@ -1,0 +1,557 @@
+"""Parity of the HIP pack/unpack path with the CPU oracle, through the C ABI.
+
+Bit-exact is the bar everywhere: this is byte movement.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+POISON = 0xCD
+
+
+def tbytes(t):
+    """Bytes of a torch tensor's C-order element sequence, as numpy uint8."""
+    import torch
+    c = t.contiguous()
+    if c.numel() == 0:
+        return np.zeros(0, np.uint8)
+    return c.reshape(-1).view(torch.uint8).cpu().numpy()
+
+
+def device_bytes(n, gpu, fill=POISON):
+    import torch
+    return torch.full((max(n, 1),), fill, dtype=torch.uint8, device=gpu)
+
+
+def run_pack(pkg, tensors, align, gpu, base_shift=0):
+    """Pack and return (payload bytes as numpy, plan)."""
+    import torch
+    plan = pkg.BundlePlan.create(tensors, align=align)
+    n = plan.payload_bytes
+    buf = device_bytes(n + base_shift + 64, gpu)
+    plan.pack(buf.data_ptr() + base_shift, n, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    # nothing outside [shift, shift + n) may be written
+    assert (host[:base_shift] == POISON).all() and (host[base_shift + n:] == POISON).all()
+    return host[base_shift:base_shift + n], plan, buf
+
+
+def rand_bytes_tensor(rng, nbytes, gpu):
+    import torch
+    return torch.from_numpy(rng.integers(0, 256, size=nbytes, dtype=np.uint8)).to(gpu)
+
+
+# ------------------------------------------------------------------ reference KATs on device
+
+@pytest.mark.parametrize("lens", [(256, 512, 300), (512 * 1024, 256 * 1024, 800 * 1024)])
+def test_iov_to_contig_kat(pkg, orc, gpu, lens):
+    import torch
+    segs, cursor = [], 0
+    for n in lens:
+        segs.append(((np.arange(n) + cursor) % 256).astype(np.uint8))
+        cursor += n
+    dev = [torch.from_numpy(s).to(gpu) for s in segs]
+    got, plan, buf = run_pack(pkg, dev, 1, gpu)
+    expected = (np.arange(sum(lens)) % 256).astype(np.uint8)
+    assert np.array_equal(got, expected)
+    assert np.array_equal(got, orc.pack(segs, 1))
+    # iov -> iov: scatter into receiver buffers of the same lengths
+    outs = [torch.zeros(n, dtype=torch.uint8, device=gpu) for n in lens]
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+    rplan.unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    for s, o in zip(segs, outs):
+        assert np.array_equal(o.cpu().numpy(), s)
+
+
+def test_process_round_trip_kat(pkg, orc, gpu):
+    # send float(i % 256), divide by two on the device, expect (i % 256) / 2 exactly
+    import torch
+    lib = pkg._capi.load()
+    for n in (32, 1 << 20):
+        x = torch.from_numpy((np.arange(4 * n) % 256).astype(np.float32)).to(gpu)
+        parts = list(x.chunk(4))
+        got, plan, buf = run_pack(pkg, parts, 1, gpu)
+        assert np.array_equal(got.view(np.float32), (np.arange(4 * n) % 256).astype(np.float32))
+        pkg._capi.check(lib.axr_divide_by_two(buf.data_ptr(), 4 * n, None))
+        torch.cuda.synchronize()
+        back = buf.cpu().numpy()[:16 * n].view(np.float32)
+        assert np.array_equal(back, (np.arange(4 * n) % 256).astype(np.float32) / 2)
+        assert np.array_equal(back, orc.divide_by_two((np.arange(4 * n) % 256).astype(np.float32)))
+
+
+def test_buffer_to_vec_kat(pkg, gpu):
+    # fp32[2048] = i split four ways keeps the global index (axon_worker_test.cpp:1656-1774)
+    import torch
+    f = torch.arange(2048, dtype=torch.float32, device=gpu)
+    outs = [torch.zeros(512, dtype=torch.float32, device=gpu) for _ in range(4)]
+    plan = pkg.BundlePlan.create(outs, align=1)
+    assert plan.payload_bytes == 8192
+    plan.unpack(f.data_ptr(), 8192)
+    torch.cuda.synchronize()
+    for k, o in enumerate(outs):
+        assert torch.equal(o, torch.arange(512 * k, 512 * (k + 1), dtype=torch.float32, device=gpu))
+    views = plan.split(f.data_ptr(), 8192)
+    assert views == [(f.data_ptr() + 2048 * k, 2048) for k in range(4)]
+
+
+# ------------------------------------------------------------------ config 1: host tensors
+
+def test_c1_host_bundle(pkg, orc, gpu):
+    import torch
+    from execution_ucx_amd import workloads
+    srcs = workloads.host_bundle_c1(seed=0)
+    got, plan, buf = run_pack(pkg, srcs, 1, gpu)
+    assert plan.payload_bytes == 4 << 20
+    want = orc.pack([s.view(np.uint8) for s in srcs], 1)
+    assert np.array_equal(got, want)
+    outs = [np.zeros_like(s) for s in srcs]
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+    assert rplan.launch_info()["host_copies"] == 64
+    rplan.unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    for a, b in zip(srcs, outs):
+        assert a.tobytes() == b.tobytes()
+
+
+# ------------------------------------------------------------------ config 2: mixed small tensors
+
+@pytest.mark.parametrize("align", [256, 1])
+def test_c2_mixed_bundle_full(pkg, orc, gpu, align):
+    import torch
+    from execution_ucx_amd import workloads
+    spec = workloads.mixed_bundle()
+    assert len(spec.segments) == 4096
+    arena, tensors = workloads.materialize_mixed(spec, gpu, seed=0)
+    host_arena = arena.cpu().numpy()
+    chunks = [host_arena[s.arena_offset:s.arena_offset + s.nbytes] for s in spec.segments]
+    got, plan, buf = run_pack(pkg, tensors, align, gpu)           # through 4096 DLPack capsules
+    assert plan.data_bytes == spec.data_bytes
+    want = orc.pack(chunks, align)
+    assert got.size == want.size
+    assert np.array_equal(got, want)
+    offs, sizes = plan.layout()
+    assert (offs, plan.payload_bytes) == orc.layout(sizes, align)
+    # header carries dtype and shape of every tensor
+    metas = plan.metas()
+    for m, s in zip(metas, spec.segments):
+        assert m.dtype == s.dtype and m.nbytes == s.nbytes and m.device[0] == 10
+    # unpack into fresh tensors
+    outs = [torch.zeros_like(t) for t in tensors]
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+    rplan.unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    back = orc.unpack(want, sizes, align)
+    for o, b in zip(outs, back):
+        assert np.array_equal(tbytes(o), b)
+
+
+# ------------------------------------------------------------------ config 3: Llama layer
+
+def test_c3_llama_layer_full(pkg, orc, gpu):
+    import torch
+    from execution_ucx_amd import workloads
+    tensors = workloads.materialize_llama_layer(gpu, seed=0)
+    chunks = [tbytes(t) for t in tensors]
+    got, plan, buf = run_pack(pkg, tensors, 256, gpu)
+    assert plan.data_bytes == 404_766_720 == workloads.llama_layer_bytes()
+    assert np.array_equal(got, orc.pack(chunks, 256))
+    outs = [torch.empty_like(t).zero_() for t in tensors]
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+    rplan.unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    for a, b in zip(tensors, outs):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+# ------------------------------------------------------------------ alignment torture
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_arbitrary_alignment(pkg, orc, gpu, seed):
+    """Odd sizes, odd source offsets, tight layout, shifted payload base."""
+    import torch
+    rng = np.random.default_rng(seed)
+    edge = [0, 1, 2, 3, 15, 16, 17, 31, 33, 255, 256, 257, 1023, 1024, 1025, 4095, 4097,
+            8191, 8192, 8193, 16383, 16385, 3 * 8192 + 5]
+    sizes = edge + [int(x) for x in rng.integers(1, 40000, size=40)]
+    rng.shuffle(sizes)
+    arena = rand_bytes_tensor(rng, sum(sizes) + 64 * len(sizes) + 64, gpu)
+    host = arena.cpu().numpy()
+    tensors, chunks, at = [], [], 0
+    for n in sizes:
+        at += int(rng.integers(0, 33))           # any byte offset
+        tensors.append(arena[at:at + n])
+        chunks.append(host[at:at + n])
+        at += n
+    for align, shift in ((1, 0), (1, 7), (16, 3), (256, 0), (4096, 1)):
+        got, plan, buf = run_pack(pkg, tensors, align, gpu, base_shift=shift)
+        want = orc.pack(chunks, align)
+        assert np.array_equal(got, want), (align, shift)
+        # unpack into destinations at fresh odd offsets
+        dst_arena = device_bytes(sum(sizes) + 64 * len(sizes) + 64, gpu, fill=0xEE)
+        outs, spans, dat = [], [], 0
+        for n in sizes:
+            dat += int(rng.integers(0, 33))
+            outs.append(dst_arena[dat:dat + n])
+            spans.append((dat, n))
+            dat += n
+        rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+        rplan.unpack(buf.data_ptr() + shift, plan.payload_bytes)
+        torch.cuda.synchronize()
+        hd = dst_arena.cpu().numpy()
+        expect = np.full(hd.size, 0xEE, np.uint8)
+        for (o, n), c in zip(spans, chunks):
+            expect[o:o + n] = c
+        assert np.array_equal(hd, expect), (align, shift)       # bytes between tensors untouched
+
+
+# ------------------------------------------------------------------ strided views
+
+def random_torch_view(rng, parent, max_dims):
+    """A random strided view of a torch tensor (slices, steps, permutes)."""
+    ndim = parent.dim()
+    index = []
+    for d in range(ndim):
+        n = parent.shape[d]
+        lo = int(rng.integers(0, n))
+        hi = int(rng.integers(lo + 1, n + 1))
+        step = int(rng.choice([1, 1, 1, 2, 3]))
+        index.append(slice(lo, hi, step))
+    v = parent[tuple(index)]
+    if rng.random() < 0.6:
+        v = v.permute(*[int(i) for i in rng.permutation(ndim)])
+    return v
+
+
+@pytest.mark.parametrize("dtype_name", ["uint8", "bfloat16", "float32", "float64", "complex128"])
+def test_strided_gather_scatter_random(pkg, orc, gpu, dtype_name):
+    import torch
+    dt = getattr(torch, dtype_name)
+    item = torch.empty((), dtype=dt).element_size()
+    rng = np.random.default_rng(item)
+    for trial in range(12):
+        ndim = int(rng.integers(1, 6))
+        shape = [int(x) for x in rng.integers(1, 9, size=ndim)]
+        shape[-1] = int(rng.integers(1, 400))                # sometimes long inner runs
+        nbytes = int(np.prod(shape)) * item
+        parent = rand_bytes_tensor(rng, nbytes, gpu).view(dt).reshape(shape)
+        views = [random_torch_view(rng, parent, ndim) for _ in range(3)]
+        views.append(parent)                                  # a compact one in between
+        host_parent = parent.reshape(-1).view(torch.uint8).cpu().numpy()
+        chunks = []
+        for v in views:
+            start = (v.data_ptr() - parent.data_ptr())
+            chunks.append(orc.gather_strided(host_parent, start, tuple(v.shape), tuple(v.stride()), item))
+            assert np.array_equal(chunks[-1], tbytes(v))       # oracle == .contiguous()
+        for align in (1, 256):
+            got, plan, buf = run_pack(pkg, views, align, gpu)
+            assert np.array_equal(got, orc.pack(chunks, align)), (trial, align)
+            # scatter into a poisoned twin of the parent at the same views
+            twin = device_bytes(nbytes, gpu, fill=0x77).view(dt).reshape(shape)
+            tviews = [twin.as_strided(v.shape, v.stride(), v.storage_offset()) for v in views[:-1]]
+            rplan = pkg.BundlePlan.from_header(plan.header)
+            metas = rplan.metas()[:-1]
+            # unpack only the strided ones: rebuild a header-compatible plan for them
+            sub = pkg.BundlePlan.create(views[:-1], align=align)
+            sub_payload = device_bytes(sub.payload_bytes, gpu)
+            sub.pack(sub_payload.data_ptr(), sub.payload_bytes)
+            rsub = pkg.BundlePlan.from_header(sub.header).bind(tviews)
+            rsub.unpack(sub_payload.data_ptr(), sub.payload_bytes)
+            torch.cuda.synchronize()
+            expect = np.full(nbytes, 0x77, np.uint8)
+            for v, c in zip(views[:-1], chunks[:-1]):
+                orc.scatter_strided(c, expect, v.data_ptr() - parent.data_ptr(), tuple(v.shape),
+                                    tuple(v.stride()), item)
+            assert np.array_equal(twin.reshape(-1).view(torch.uint8).cpu().numpy(), expect), (trial, align)
+            assert len(metas) == len(views) - 1
+
+
+def test_strided_many_dims_and_long_runs(pkg, orc, gpu):
+    """More strided outer dimensions than the device table holds (peeled on the
+    host), runs that span several tiles, and a transposed matrix."""
+    import torch
+    rng = np.random.default_rng(42)
+    p8 = rand_bytes_tensor(rng, 3 * 4 * 3 * 4 * 3 * 4 * 3 * 4 * 40 * 2, gpu).view(torch.int16)
+    p8 = p8.reshape(3, 4, 3, 4, 3, 4, 3, 4, 40)
+    v8 = p8[:2, 1:3, :2, ::2, 1:, :3, ::2, 1:3, 4:36]          # 8 strided dims + 64 B runs
+    big = rand_bytes_tensor(rng, 64 * 40000, gpu).view(torch.float32).reshape(64, 10000)
+    vlong = big[::2, 17:9000]                                   # 35,932 B runs, 4-byte aligned only
+    mat = rand_bytes_tensor(rng, 300 * 500 * 2, gpu).view(torch.bfloat16).reshape(300, 500)
+    views = [v8, vlong, mat.t(), mat[:, 100:164]]
+    chunks = [tbytes(v) for v in views]
+    plan = pkg.BundlePlan.create(views, align=256)
+    modes = {s["mode"] for s in plan.segments()}
+    assert {1, 2} <= modes                                      # run tiles and element mode both used
+    got, plan, buf = run_pack(pkg, views, 256, gpu)
+    assert np.array_equal(got, orc.pack(chunks, 256))
+    outs = [torch.zeros_like(v, memory_format=torch.contiguous_format) for v in views]
+    pkg.BundlePlan.from_header(plan.header).bind(outs).unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    for v, o in zip(views, outs):
+        assert np.array_equal(tbytes(o), tbytes(v))
+
+
+def test_c4_kv_gather_reduced_vs_oracle(pkg, orc, gpu):
+    import torch
+    from execution_ucx_amd import workloads
+    spec = workloads.kv_gather(layers=4, blocks=64, picks=16, seed=0)
+    n = int(np.prod(spec.cache_shape))
+    a = torch.randn(n, device=gpu).to(torch.bfloat16)
+    b = torch.zeros(n, dtype=torch.bfloat16, device=gpu)
+    src = [workloads.kv_block_view(a.data_ptr(), spec, int(i)) for i in spec.src_index]
+    dst = [workloads.kv_block_view(b.data_ptr(), spec, int(i)) for i in spec.dst_index]
+    host_a = a.view(torch.uint8).cpu().numpy()
+    chunks = [orc.gather_strided(host_a, v.data - a.data_ptr(), v.shape, v.strides, 2) for v in src]
+    got, plan, buf = run_pack(pkg, src, 256, gpu)
+    assert plan.payload_bytes == spec.payload_bytes
+    assert np.array_equal(got, orc.pack(chunks, 256))
+    seg = plan.segments()[0]
+    assert (seg["mode"], seg["run_bytes"], seg["shape"]) == (1, spec.block_elems * 2, (spec.layers * 2,))
+    pkg.BundlePlan.from_header(plan.header).bind(dst).unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    expect = np.zeros(n * 2, np.uint8)
+    for v, c in zip(dst, chunks):
+        orc.scatter_strided(c, expect, v.data - b.data_ptr(), v.shape, v.strides, 2)
+    assert np.array_equal(b.view(torch.uint8).cpu().numpy(), expect)
+
+
+def test_c4_kv_gather_full_size_properties(pkg, gpu):
+    """8 GiB caches, 1 GiB payload: checked with size-independent properties on
+    the device (moved blocks equal, everything else untouched)."""
+    import torch
+    from execution_ucx_amd import workloads
+    spec = workloads.kv_gather()
+    shape = spec.cache_shape
+    a = torch.empty(shape, dtype=torch.bfloat16, device=gpu)
+    a.view(torch.int16).random_(-32768, 32767)
+    b = torch.zeros(shape, dtype=torch.bfloat16, device=gpu)
+    src = [workloads.kv_block_view(a.data_ptr(), spec, int(i)) for i in spec.src_index]
+    dst = [workloads.kv_block_view(b.data_ptr(), spec, int(i)) for i in spec.dst_index]
+    plan = pkg.BundlePlan.create(src, align=256)
+    assert plan.payload_bytes == 1 << 30 == spec.payload_bytes
+    payload = torch.empty(1 << 30, dtype=torch.uint8, device=gpu)
+    plan.pack(payload.data_ptr(), 1 << 30)
+    torch.cuda.synchronize()
+    si = torch.from_numpy(spec.src_index).to(gpu)
+    di = torch.from_numpy(spec.dst_index).to(gpu)
+    # payload == [block j][layer][kv] order == A[:, :, src].permute(2, 0, 1, ...)
+    want = a.view(torch.int16)[:, :, si].permute(2, 0, 1, 3, 4, 5).contiguous()
+    assert torch.equal(payload.view(torch.int16), want.reshape(-1))
+    del want
+    pkg.BundlePlan.from_header(plan.header).bind(dst).unpack(payload.data_ptr(), 1 << 30)
+    torch.cuda.synchronize()
+    assert torch.equal(b.view(torch.int16)[:, :, di], a.view(torch.int16)[:, :, si])
+    mask = torch.ones(spec.blocks, dtype=torch.bool, device=gpu)
+    mask[di] = False
+    assert int(b.view(torch.int16)[:, :, mask].ne(0).sum()) == 0
+
+
+def test_c5_pitched_chunk(pkg, orc, gpu):
+    """One 256 MiB chunk of 64 pitched 2-D views, and a small one against the oracle."""
+    import torch
+    from execution_ucx_amd import workloads
+    small = workloads.pitched_chunk(views=3, rows=5, cols=64)
+    big = workloads.pitched_chunk()
+    assert big.payload_bytes == 256 << 20
+    for spec, use_oracle in ((small, True), (big, False)):
+        parents = torch.empty(spec.views, spec.rows, spec.pitch, dtype=torch.bfloat16, device=gpu)
+        parents.view(torch.int16).random_(-32768, 32767)
+        views = workloads.pitched_views(parents.data_ptr(), spec)
+        plan = pkg.BundlePlan.create(views, align=256)
+        assert plan.payload_bytes == spec.payload_bytes
+        payload = device_bytes(spec.payload_bytes, gpu)
+        plan.pack(payload.data_ptr(), spec.payload_bytes)
+        torch.cuda.synchronize()
+        want = parents[:, :, :spec.cols].contiguous()
+        assert torch.equal(payload[:spec.payload_bytes].view(torch.int16), want.view(torch.int16).reshape(-1))
+        if use_oracle:
+            host = parents.view(torch.uint8).reshape(-1).cpu().numpy()
+            chunks = [orc.gather_strided(host, v.data - parents.data_ptr(), v.shape, v.strides, 2)
+                      for v in views]
+            assert np.array_equal(payload.cpu().numpy()[:spec.payload_bytes], orc.pack(chunks, 256))
+        twin = torch.zeros_like(parents)
+        tv = workloads.pitched_views(twin.data_ptr(), spec)
+        pkg.BundlePlan.from_header(plan.header).bind(tv).unpack(payload.data_ptr(), spec.payload_bytes)
+        torch.cuda.synchronize()
+        assert torch.equal(twin[:, :, :spec.cols], parents[:, :, :spec.cols])
+        assert int(twin[:, :, spec.cols:].view(torch.int16).ne(0).sum()) == 0     # pitch gap untouched
+
+
+# ------------------------------------------------------------------ checksums, compare
+
+def test_checksum_of_checksums(pkg, orc, gpu):
+    import torch
+    lib = pkg._capi.load()
+    rng = np.random.default_rng(1)
+    tensors = [rand_bytes_tensor(rng, int(n), gpu) for n in rng.integers(1, 200000, size=30)]
+    got, plan, buf = run_pack(pkg, tensors, 256, gpu)
+    offs, sizes = plan.layout()
+    total = C.c_uint64()
+    pkg._capi.check(lib.axr_checksum(buf.data_ptr(), plan.payload_bytes, 0, C.byref(total)))
+    assert total.value == orc.checksum(got, 0)
+    acc = 0
+    for t, o in zip(tensors, offs):
+        s = C.c_uint64()
+        pkg._capi.check(lib.axr_checksum(t.data_ptr(), t.numel(), o, C.byref(s)))
+        acc = (acc + s.value) % (1 << 64)
+    assert acc == total.value                    # zero gaps add nothing
+    mism = C.c_uint64(99)
+    twin = buf.clone()
+    pkg._capi.check(lib.axr_compare(buf.data_ptr(), twin.data_ptr(), plan.payload_bytes, C.byref(mism)))
+    assert mism.value == 0
+    twin[5] ^= 1
+    twin[plan.payload_bytes - 1] ^= 0x80
+    pkg._capi.check(lib.axr_compare(buf.data_ptr(), twin.data_ptr(), plan.payload_bytes, C.byref(mism)))
+    assert mism.value == 2
+
+
+# ------------------------------------------------------------------ DLPack in and out
+
+def test_dlpack_rocm_capsules_and_zero_copy_receive(pkg, gpu):
+    import torch
+    srcs = [torch.randn(1000, device=gpu), torch.randn(7, 33, device=gpu).to(torch.bfloat16),
+            torch.arange(50, device=gpu, dtype=torch.int32)]
+    view = pkg.extract(srcs[1])
+    assert view.device_type == 10 and view.dtype == (4, 16, 1) and view.shape == (7, 33)
+    stream = torch.cuda.current_stream().cuda_stream
+    packed = pkg.pack_bundle(srcs, align=256, stream=stream)
+    assert packed.payload.memory_type == 3                      # ucx_memory_type::ROCM
+    outs = pkg.unpack_bundle(packed.header, packed.payload, stream=stream,
+                             from_dlpack_fn=torch.from_dlpack)
+    torch.cuda.synchronize()
+    for a, b in zip(srcs, outs):
+        assert b.device.type == "cuda" and b.dtype == a.dtype and b.shape == a.shape
+        assert torch.equal(a, b)
+    base = packed.payload.data
+    assert [o.data_ptr() - base for o in outs] == packed.plan.layout()[0]   # views, not copies
+
+
+# ------------------------------------------------------------------ plan reuse, streams, errors
+
+def test_plan_reuse_rebind_and_streams(pkg, orc, gpu):
+    import torch
+    lib = pkg._capi.load()
+    rng = np.random.default_rng(2)
+    a = [rand_bytes_tensor(rng, n, gpu) for n in (5000, 70000, 33)]
+    b = [rand_bytes_tensor(rng, n, gpu) for n in (5000, 70000, 33)]
+    plan = pkg.BundlePlan.create(a, align=256)
+    n = plan.payload_bytes
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    pkg._capi.check(lib.axr_stream_create(C.byref(s1)))
+    pkg._capi.check(lib.axr_stream_create(C.byref(s2)))
+    p1, p2 = device_bytes(n, gpu), device_bytes(n, gpu)
+    torch.cuda.synchronize()
+    plan.pack(p1.data_ptr(), n, s1.value)
+    plan.pack(p2.data_ptr(), n, s2.value)          # second stream waits for the table upload
+    pkg._capi.check(lib.axr_stream_synchronize(s1))
+    pkg._capi.check(lib.axr_stream_synchronize(s2))
+    want = orc.pack([tbytes(t) for t in a], 256)
+    assert np.array_equal(p1.cpu().numpy()[:n], want)
+    assert np.array_equal(p2.cpu().numpy()[:n], want)
+    plan.bind(b)
+    plan.pack(p1.data_ptr(), n, s1.value)
+    pkg._capi.check(lib.axr_stream_synchronize(s1))
+    assert np.array_equal(p1.cpu().numpy()[:n], orc.pack([tbytes(t) for t in b], 256))
+    ev0, ev1 = C.c_void_p(), C.c_void_p()
+    pkg._capi.check(lib.axr_event_create(C.byref(ev0)))
+    pkg._capi.check(lib.axr_event_create(C.byref(ev1)))
+    pkg._capi.check(lib.axr_event_record(ev0, s1))
+    plan.pack(p1.data_ptr(), n, s1.value)
+    pkg._capi.check(lib.axr_event_record(ev1, s1))
+    pkg._capi.check(lib.axr_event_synchronize(ev1))
+    ms = C.c_float()
+    pkg._capi.check(lib.axr_event_elapsed_ms(ev0, ev1, C.byref(ms)))
+    assert ms.value > 0
+    for h in (ev0, ev1):
+        pkg._capi.check(lib.axr_event_destroy(h))
+    plan.close()
+    for s in (s1, s2):
+        pkg._capi.check(lib.axr_stream_destroy(s))
+
+
+def test_error_paths(pkg, gpu):
+    import torch
+    a = [torch.zeros(100, device=gpu), torch.zeros(7, device=gpu)]
+    plan = pkg.BundlePlan.create(a, align=256)
+    buf = device_bytes(1024, gpu)
+    with pytest.raises(pkg.LengthError):
+        plan.pack(buf.data_ptr(), plan.payload_bytes - 1)
+    with pytest.raises(pkg.LengthError):
+        plan.split(buf.data_ptr(), 10)
+    r = pkg.BundlePlan.from_header(plan.header)
+    with pytest.raises(pkg.AxonRocmError):
+        r.unpack(buf.data_ptr(), plan.payload_bytes)              # nothing bound yet
+    with pytest.raises(pkg.MismatchError):
+        r.bind([torch.zeros(100, device=gpu)])
+    with pytest.raises(pkg.MismatchError):
+        r.bind([torch.zeros(100, device=gpu), torch.zeros(8, device=gpu)])
+    with pytest.raises(pkg.AxonRocmError):                        # overlapping destination
+        r.bind([torch.zeros(1, device=gpu).expand(100), torch.zeros(7, device=gpu)])
+        r.unpack(buf.data_ptr(), plan.payload_bytes)
+    hdr = bytearray(plan.header)
+    hdr[0] ^= 0xFF
+    with pytest.raises(pkg.HeaderError):
+        pkg.BundlePlan.from_header(bytes(hdr))
+    # empty bundles are legal and move nothing
+    empty = pkg.BundlePlan.create([], align=1)
+    assert empty.payload_bytes == 0
+    empty.pack(0, 0)
+    zero = pkg.BundlePlan.create([torch.zeros(0, device=gpu), torch.zeros((), device=gpu)], align=256)
+    assert zero.payload_bytes == 0 and zero.layout() == ([0, 0], [0, 0])
+    zero.pack(0, 0)
+
+
+# ------------------------------------------------------------------ memory resource
+
+def test_pool_and_copy_table(pkg, gpu):
+    import torch
+    registered = []
+    pool = pkg.DevicePool(device=0, slab_bytes=4 << 20)
+    pool.set_registrar(lambda addr, n: (registered.append((addr, n)) or 0xABC0 + len(registered)),
+                       lambda h: registered.append(("unreg", h)))
+    x = pool.alloc(1000)
+    y = pool.alloc(3 << 20, alignment=4096)
+    z = pool.alloc(8 << 20)                                       # larger than a slab: own slab
+    assert x.data % 256 == 0 and y.data % 4096 == 0
+    assert x.mem_h == 0xABC1 and y.mem_h == 0xABC1 and z.mem_h == 0xABC2
+    st = pool.stats()
+    assert st["slabs"] == 2 and st["live_blocks"] == 3
+    x_addr = x.data
+    x.release()
+    x2 = pool.alloc(1000)
+    assert x2.data == x_addr                                      # freed block is reused
+    for blk in (x2, y, z):
+        blk.release()
+    assert pool.stats()["allocated_bytes"] == 0
+    pool.trim()
+    assert pool.stats()["slabs"] == 0
+    assert sorted(r for r in registered if r[0] == "unreg") == [("unreg", 0xABC1), ("unreg", 0xABC2)]
+    pool.close()
+
+    mr = pkg.RocmMemoryResourceManager()
+    HOST, ROCM, PINNED = 0, 3, 4
+    src = np.arange(100000, dtype=np.uint8)
+    d = mr.allocate(ROCM, src.size)
+    p = mr.allocate(PINNED, src.size)
+    back = np.zeros_like(src)
+    mr.memcpy(ROCM, d, HOST, src.ctypes.data, src.size)          # H2D
+    mr.memcpy(PINNED, p, ROCM, d, src.size)                      # D2H into pinned
+    mr.memcpy(HOST, back.ctypes.data, PINNED, p, src.size)       # H2H
+    assert np.array_equal(src, back)
+    d2 = mr.allocate(ROCM, src.size)
+    mr.memcpy(ROCM, d2, ROCM, d, src.size)                        # D2D
+    back[:] = 0
+    mr.memcpy(HOST, back.ctypes.data, ROCM, d2, src.size)
+    assert np.array_equal(src, back)
+    with pytest.raises(pkg.UnsupportedMemoryError):
+        mr.allocate(1, 16)                                        # ucx_memory_type::CUDA
+    with pytest.raises(pkg.UnsupportedMemoryError):
+        mr.memcpy(1, d, HOST, src.ctypes.data, 16)
+    for t, ptr in ((ROCM, d), (ROCM, d2), (PINNED, p)):
+        mr.deallocate(t, ptr, src.size)
+    with pkg.rocm(0).activate() as devobj:
+        assert devobj.get_type_string() == "rocm" and devobj.get_context_handle() == 0
