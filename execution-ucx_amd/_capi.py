@@ -222,6 +222,35 @@ PROTOTYPES = {
 _lib = None
 
 
+def _share_hip_runtime() -> None:
+    """Make this library and PyTorch use ONE HIP runtime instance.
+
+    PyTorch wheels ship their own libamdhip64.so; streams, events and device
+    pointers are only interchangeable inside one runtime instance.  The dynamic
+    loader reuses an already loaded library whose SONAME matches, so the wheel's
+    copy is loaded first (without importing torch) when it exists; otherwise the
+    system ROCm runtime named in the library's RUNPATH is used.
+    """
+    try:
+        with open("/proc/self/maps") as f:
+            if "libamdhip64" in f.read():
+                return
+    except OSError:
+        pass
+    try:
+        import importlib.util
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.submodule_search_locations:
+        return
+    for base in spec.submodule_search_locations:
+        cand = os.path.join(base, "lib", "libamdhip64.so")
+        if os.path.exists(cand):
+            C.CDLL(cand, mode=C.RTLD_GLOBAL)
+            return
+
+
 def load() -> C.CDLL:
     """Load the shared library once and attach prototypes."""
     global _lib
@@ -233,6 +262,7 @@ def load() -> C.CDLL:
             "(run `make -C execution-ucx_amd` or `__graft_entry__.build()`); "
             "there is no CPU fallback for the tensor-bundle path"
         )
+    _share_hip_runtime()
     lib = C.CDLL(LIBRARY_PATH)
     for name, (restype, argtypes) in PROTOTYPES.items():
         fn = getattr(lib, name)
