@@ -76,11 +76,14 @@ class Harness:
 
 
 class BundleSet:
-    """One independent copy of a workload: source views, payload, destination views, two plans."""
+    """One independent copy of a workload: source views, payload, destination views, two plans.
 
-    def __init__(self, h: Harness, src_views, dst_views, align, keep):
+    `check` compares source and destination on the device after a round trip."""
+
+    def __init__(self, h: Harness, src_views, dst_views, align, keep, check=None):
         pkg = h.pkg
         self.keep = keep
+        self.check = check
         self.pack_plan = pkg.BundlePlan.create(src_views, align=align)
         self.nbytes = self.pack_plan.payload_bytes
         self.data_bytes = self.pack_plan.data_bytes
@@ -110,12 +113,17 @@ def make_c2_sets(h, count, seed=0):
     from execution_ucx_amd import workloads
     spec = workloads.mixed_bundle(seed=seed)
     sets = []
+    mask = h.torch.zeros(spec.arena_bytes, dtype=h.torch.bool, device="cuda")
+    for s in spec.segments:
+        mask[s.arena_offset:s.arena_offset + s.nbytes] = True
     for k in range(count):
         arena, _ = workloads.materialize_mixed(spec, "cuda", seed=seed + k)
+        arena.mul_(mask)      # bytes between tensors are not part of the bundle: zero them
         dst = h.torch.zeros_like(arena)
         sv = workloads.mixed_views(spec, arena.data_ptr())
         dv = workloads.mixed_views(spec, dst.data_ptr())
-        sets.append(BundleSet(h, sv, dv, 256, (arena, dst)))
+        sets.append(BundleSet(h, sv, dv, 256, (arena, dst),
+                              check=lambda a=arena, d=dst: bool(h.torch.equal(a, d))))
     return spec, sets
 
 
@@ -125,8 +133,10 @@ def make_c3_sets(h, count, seed=0):
     for k in range(count):
         src = workloads.materialize_llama_layer("cuda", seed=seed + k)
         dst = [h.torch.empty_like(t) for t in src]
-        sets.append(BundleSet(h, workloads.views_of_torch(src), workloads.views_of_torch(dst), 256,
-                              (src, dst)))
+        sets.append(BundleSet(
+            h, workloads.views_of_torch(src), workloads.views_of_torch(dst), 256, (src, dst),
+            check=lambda s=src, d=dst: all(bool(h.torch.equal(x.view(h.torch.int16), y.view(h.torch.int16)))
+                                           for x, y in zip(s, d))))
     return sets
 
 
@@ -138,7 +148,13 @@ def make_c4_set(h, seed=0):
     b = h.torch.zeros(spec.cache_shape, dtype=h.torch.bfloat16, device="cuda")
     sv = [workloads.kv_block_view(a.data_ptr(), spec, int(i)) for i in spec.src_index]
     dv = [workloads.kv_block_view(b.data_ptr(), spec, int(i)) for i in spec.dst_index]
-    return BundleSet(h, sv, dv, 256, (a, b))
+    si = h.torch.from_numpy(spec.src_index).cuda()
+    di = h.torch.from_numpy(spec.dst_index).cuda()
+
+    def check():
+        ai, bi = a.view(h.torch.int16), b.view(h.torch.int16)
+        return bool(h.torch.equal(bi[:, :, di], ai[:, :, si]))
+    return BundleSet(h, sv, dv, 256, (a, b), check=check)
 
 
 def make_c5_sets(h, count):
@@ -149,8 +165,11 @@ def make_c5_sets(h, count):
         src = h.torch.empty(spec.views, spec.rows, spec.pitch, dtype=h.torch.bfloat16, device="cuda")
         src.view(h.torch.int16).random_(-32768, 32767)
         dst = h.torch.zeros_like(src)
-        sets.append(BundleSet(h, workloads.pitched_views(src.data_ptr(), spec),
-                              workloads.pitched_views(dst.data_ptr(), spec), 256, (src, dst)))
+        sets.append(BundleSet(
+            h, workloads.pitched_views(src.data_ptr(), spec),
+            workloads.pitched_views(dst.data_ptr(), spec), 256, (src, dst),
+            check=lambda s=src, d=dst, c=spec.cols: bool(h.torch.equal(
+                s.view(h.torch.int16)[:, :, :c], d.view(h.torch.int16)[:, :, :c]))))
     return sets
 
 
@@ -159,6 +178,8 @@ def verify_set(h, s):
     h.capi.check(h.lib.axr_pack(s.pp, s.ptr, s.nbytes, h.stream))
     h.capi.check(h.lib.axr_unpack(s.up, s.ptr, s.nbytes, h.stream))
     h.sync()
+    if s.check is not None and not s.check():
+        raise SystemExit("bench.py: round trip did not reproduce the source tensors")
 
 
 def rate(data_bytes, ms, steps):

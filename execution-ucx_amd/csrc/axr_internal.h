@@ -25,8 +25,8 @@ constexpr uint32_t kWaveLanes = 64;
 constexpr uint32_t kVecBytes = 16;                           // one dwordx4 per lane
 constexpr uint32_t kRowBytes = kWaveLanes * kVecBytes;       // 1 KiB per wave-wide access
 constexpr uint32_t kMaxTileRows = 16;
-constexpr uint32_t kThreadsPerWorkgroup = 256;
-constexpr uint32_t kWavesPerWorkgroup = kThreadsPerWorkgroup / kWaveLanes;
+constexpr uint32_t kMaxThreadsPerWorkgroup = 1024;
+constexpr uint32_t kXcds = 8;   // accelerator dies; workgroup i is dispatched to die i % 8
 constexpr uint32_t kMaxOuterDims = 6;
 
 constexpr uint32_t kSegPadMask = 0xfffu;         // meta bits 0..11: zero bytes after segment
@@ -65,25 +65,34 @@ struct KernelArgs {
   uint32_t nseg;
   uint32_t ntiles;
   uint32_t tiles_per_wave;
-  uint32_t reserved;
+  uint32_t xcd_remap;         // 0 or the number of workgroups per die
 };
 
 struct LaunchConfig {
   uint32_t workgroups = 0;
   uint32_t tiles_per_wave = 0;
-  uint32_t tile_rows = 8;
+  uint32_t tile_rows = 2;
+  uint32_t threads = 256;   // per workgroup, a multiple of 64
   bool nontemporal = true;
   bool elements = false;   // some segment uses kModeElements
+  bool xcd_remap = false;  // give each die a contiguous share of the wave index space
 };
 
 // ---------------------------------------------------------------- tunables
 
 struct Tunables {
-  int64_t waves_per_cu = 32;      // wavefronts per compute unit the grid is sized for
-  int64_t tile_rows = 8;          // 1 KiB rows per tile (4, 8 or 16)
+  // Tile = tile_rows KiB moved by one wavefront.  0 picks the smallest of
+  // 2, 4, 8, 16 that keeps the bundle within max_tiles tiles: small tiles and a
+  // grid of one tile per wave measured fastest on MI355X (the hardware
+  // dispatcher balances the load), larger tiles bound the per-wave index table
+  // and the host time to fill it for multi-GiB bundles.
+  int64_t tile_rows = 0;
+  int64_t max_tiles = 1 << 17;
+  int64_t max_waves = 1 << 20;    // beyond this many tiles a wave takes several
+  int64_t threads = 256;          // workgroup size
   int64_t nontemporal = 1;        // non-temporal loads/stores in the copy loops
   int64_t gather_run_bytes = 512; // strided runs shorter than this use element mode
-  int64_t min_tiles_per_wave = 1;
+  int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
 };
 Tunables& tunables();
 

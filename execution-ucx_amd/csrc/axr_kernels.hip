@@ -28,10 +28,10 @@ typedef const AXR_GLOBAL uint8_t* gcbytes;
 typedef AXR_GLOBAL u32x4* gvec;
 typedef const AXR_GLOBAL u32x4* gcvec;
 
-// 16-byte accesses.  Stores are always 16-byte aligned (the copy aligns the
-// destination first); loads carry no alignment promise: gfx950 serves unaligned
-// global accesses in hardware, so a source that is not congruent to its
-// destination modulo 16 costs straddling reads, not a different code path.
+// 16-byte accesses carry no alignment promise: gfx950 serves unaligned global
+// loads and stores in hardware, at full speed when the address happens to be
+// aligned (the 256-byte aligned layout with 16-byte aligned tensors) and with
+// straddling accesses otherwise (tight layouts with odd sizes).
 typedef u32x4 __attribute__((aligned(1))) u32x4_loose;
 
 template <bool NT>
@@ -46,7 +46,7 @@ __device__ __forceinline__ u32x4 load16(gcbytes p) {
 
 template <bool NT>
 __device__ __forceinline__ void store16(gbytes p, u32x4 v) {
-  gvec q = reinterpret_cast<gvec>(p);
+  AXR_GLOBAL u32x4_loose* q = reinterpret_cast<AXR_GLOBAL u32x4_loose*>(p);
   if constexpr (NT) {
     __builtin_nontemporal_store(v, q);
   } else {
@@ -62,48 +62,62 @@ __device__ __forceinline__ gbytes as_global(uint64_t address) {
   return reinterpret_cast<gbytes>(address);
 }
 
-// Wave-cooperative copy of n <= ROWS KiB bytes.  src, dst and n are
-// wave-uniform, lane_off is lane * 16.  Handles any alignment: a byte head
-// brings dst to 16 bytes, the body moves 1 KiB rows, a byte tail finishes.
+// Wave-cooperative copy of one tile.  src, dst and the length are
+// wave-uniform, lane_off is lane * 16.  A full tile is ROWS loads then ROWS
+// stores per lane.
 template <uint32_t ROWS, bool NT>
-__device__ __forceinline__ void wave_copy(gcbytes src, gbytes dst, uint32_t n, uint32_t lane,
-                                          uint32_t lane_off) {
-  const uint32_t mis = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u;
-  if (mis != 0) {
-    uint32_t head = 16u - mis;
-    head = head < n ? head : n;
-    if (lane < head) dst[lane] = src[lane];
-    src += head;
-    dst += head;
-    n -= head;
-  }
+__device__ __forceinline__ void wave_copy_full(gcbytes src, gbytes dst, uint32_t lane_off) {
   u32x4 v[ROWS];
-  if (n == ROWS * kRowBytes) {
 #pragma unroll
-    for (uint32_t k = 0; k < ROWS; ++k) v[k] = load16<NT>(src + lane_off + k * kRowBytes);
+  for (uint32_t k = 0; k < ROWS; ++k) v[k] = load16<NT>(src + lane_off + k * kRowBytes);
 #pragma unroll
-    for (uint32_t k = 0; k < ROWS; ++k) store16<NT>(dst + lane_off + k * kRowBytes, v[k]);
+  for (uint32_t k = 0; k < ROWS; ++k) store16<NT>(dst + lane_off + k * kRowBytes, v[k]);
+}
+
+// A partial tile (n < ROWS KiB) keeps the same shape: slot j (= lane + 64 k)
+// moves bytes [16 j, 16 j + 16) while that lies inside the range, and the first
+// slot past the last whole vector moves the final 16 bytes [n - 16, n), which
+// overlap the previous slot with identical data.  No byte loops, no second
+// memory round trip; only ranges under 16 bytes are moved bytewise.
+template <uint32_t ROWS, bool NT>
+__device__ __forceinline__ void wave_copy_partial(gcbytes src, gbytes dst, uint32_t n,
+                                                  uint32_t lane, uint32_t lane_off) {
+  if (n < kVecBytes) {
+    if (lane < n) dst[lane] = src[lane];
     return;
   }
-  const uint32_t body = n & ~15u;
-  if (body != 0) {
-    // Partial tile: every lane loads (out-of-range lanes re-read the last
-    // vector, which keeps all ROWS loads unconditional and in flight
-    // together); only the stores are masked.
-    const uint32_t last = body - kVecBytes;
+  u32x4 v[ROWS];
+  const uint32_t body = n & ~15u;            // bytes covered by whole vectors
+  const uint32_t last = n - kVecBytes;       // start of the final (possibly overlapping) vector
+  const uint32_t limit = body + ((n & 15u) ? kVecBytes : 0u);   // slots at offsets < limit store
 #pragma unroll
-    for (uint32_t k = 0; k < ROWS; ++k) {
-      const uint32_t o = lane_off + k * kRowBytes;
-      v[k] = load16<NT>(src + (o < last ? o : last));
-    }
-#pragma unroll
-    for (uint32_t k = 0; k < ROWS; ++k) {
-      const uint32_t o = lane_off + k * kRowBytes;
-      if (o < body) store16<NT>(dst + o, v[k]);
-    }
+  for (uint32_t k = 0; k < ROWS; ++k) {
+    const uint32_t o = lane_off + k * kRowBytes;
+    v[k] = load16<NT>(src + (o < body ? o : last));   // unconditional: all loads in flight together
   }
-  const uint32_t tail = n & 15u;
-  if (lane < tail) dst[body + lane] = src[body + lane];
+  // Pin every loaded value here: it keeps the compiler from sinking a load into
+  // the masked store that uses it (load -> wait -> store per slot), and it puts
+  // the single wait for the loads ahead of the first store, so no masked store
+  // is followed by a wait that would also cover that store's own completion.
+#pragma unroll
+  for (uint32_t k = 0; k < ROWS; ++k) asm volatile("" : "+v"(v[k])::"memory");
+#pragma unroll
+  for (uint32_t k = 0; k < ROWS; ++k) {
+    const uint32_t o = lane_off + k * kRowBytes;
+    if (o < limit) store16<NT>(dst + (o < body ? o : last), v[k]);
+  }
+}
+
+// `left` bytes remain in the run from this tile's start; the tile takes at
+// most ROWS KiB of them.
+template <uint32_t ROWS, bool NT>
+__device__ __forceinline__ void wave_copy(gcbytes src, gbytes dst, uint64_t left, uint32_t lane,
+                                          uint32_t lane_off) {
+  if (left >= ROWS * kRowBytes) {
+    wave_copy_full<ROWS, NT>(src, dst, lane_off);
+  } else {
+    wave_copy_partial<ROWS, NT>(src, dst, static_cast<uint32_t>(left), lane, lane_off);
+  }
 }
 
 __device__ __forceinline__ void wave_zero(gbytes dst, uint32_t n, uint32_t lane) {
@@ -201,11 +215,17 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
 }
 
 template <bool PACK, uint32_t ROWS, bool NT, bool ELEMENTS>
-__global__ __launch_bounds__(kThreadsPerWorkgroup) void bundle_kernel(KernelArgs a) {
+__global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(KernelArgs a) {
   constexpr uint32_t kTile = ROWS * kRowBytes;
   const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
   const uint32_t lane_off = lane * kVecBytes;
-  const uint32_t wave = uniform(blockIdx.x * kWavesPerWorkgroup + (threadIdx.x >> 6));
+  uint32_t wg = blockIdx.x;
+  if (a.xcd_remap) {
+    // consecutive workgroup ids land on consecutive dies; hand die d the d-th
+    // contiguous share of the index space so neighbouring tiles share an L2
+    wg = (wg % kXcds) * a.xcd_remap + wg / kXcds;
+  }
+  const uint32_t wave = uniform(wg * (blockDim.x >> 6) + (threadIdx.x >> 6));
   uint32_t t = wave * a.tiles_per_wave;
   if (t >= a.ntiles) return;
   const uint32_t t_end =
@@ -240,13 +260,12 @@ __global__ __launch_bounds__(kThreadsPerWorkgroup) void bundle_kernel(KernelArgs
       // one contiguous run
       const uint64_t boff = static_cast<uint64_t>(q) * kTile;
       const uint64_t left = seg_run - boff;
-      const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
       gbytes ten = as_global(seg_ptr) + boff;
       if constexpr (PACK) {
-        wave_copy<ROWS, NT>(ten, pay + boff, n, lane, lane_off);
+        wave_copy<ROWS, NT>(ten, pay + boff, left, lane, lane_off);
         if (last && pad) wave_zero(pay + seg_run, pad, lane);
       } else {
-        wave_copy<ROWS, NT>(pay + boff, ten, n, lane, lane_off);
+        wave_copy<ROWS, NT>(pay + boff, ten, left, lane, lane_off);
       }
     } else if (dsel == kSegFillOnly) {
       if constexpr (PACK) wave_zero(pay, pad, lane);
@@ -258,13 +277,12 @@ __global__ __launch_bounds__(kThreadsPerWorkgroup) void bundle_kernel(KernelArgs
         const uint32_t piece = q - run * tpr;
         const uint64_t boff = static_cast<uint64_t>(piece) * kTile;
         const uint64_t left = seg_run - boff;
-        const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
         gbytes ten = as_global(seg_ptr) + run_offset(dm, run) + boff;
         gbytes p = pay + static_cast<uint64_t>(run) * seg_run + boff;
         if constexpr (PACK) {
-          wave_copy<ROWS, NT>(ten, p, n, lane, lane_off);
+          wave_copy<ROWS, NT>(ten, p, left, lane, lane_off);
         } else {
-          wave_copy<ROWS, NT>(p, ten, n, lane, lane_off);
+          wave_copy<ROWS, NT>(p, ten, left, lane, lane_off);
         }
       } else if constexpr (ELEMENTS) {
         element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
@@ -331,7 +349,7 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
 
 template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
-  const dim3 grid(cfg.workgroups), block(kThreadsPerWorkgroup);
+  const dim3 grid(cfg.workgroups), block(cfg.threads);
   if (cfg.elements) {
     // strided tensors with short runs are present: the general kernel
     hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, false, true>), grid, block, 0, stream, args);
@@ -346,10 +364,12 @@ int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t str
 template <bool PACK>
 int launch_dir(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   switch (cfg.tile_rows) {
+    case 1: return launch_rows<PACK, 1>(args, cfg, stream);
+    case 2: return launch_rows<PACK, 2>(args, cfg, stream);
     case 4: return launch_rows<PACK, 4>(args, cfg, stream);
     case 8: return launch_rows<PACK, 8>(args, cfg, stream);
     case 16: return launch_rows<PACK, 16>(args, cfg, stream);
-    default: return fail(AXR_ERR_INVALID, "tile_rows must be 4, 8 or 16");
+    default: return fail(AXR_ERR_INVALID, "tile_rows must be 1, 2, 4, 8 or 16");
   }
 }
 
@@ -365,7 +385,11 @@ int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& 
                          void* stream) {
   if (args.ntiles == 0 || cfg.workgroups == 0) return AXR_OK;
   // The grid must cover every tile: waves * tiles_per_wave >= ntiles.
-  const uint64_t covered = static_cast<uint64_t>(cfg.workgroups) * kWavesPerWorkgroup *
+  if (cfg.threads == 0 || cfg.threads % kWaveLanes || cfg.threads > kMaxThreadsPerWorkgroup)
+    return fail(AXR_ERR_INVALID, "workgroup size must be a multiple of 64 up to 1024");
+  if (args.xcd_remap && (cfg.workgroups % kXcds || args.xcd_remap != cfg.workgroups / kXcds))
+    return fail(AXR_ERR_INVALID, "die remapping needs a grid that is a multiple of 8");
+  const uint64_t covered = static_cast<uint64_t>(cfg.workgroups) * (cfg.threads / kWaveLanes) *
                            cfg.tiles_per_wave;
   if (covered < args.ntiles || args.tiles_per_wave != cfg.tiles_per_wave) {
     return fail(AXR_ERR_INVALID, "launch geometry does not cover the tile range");

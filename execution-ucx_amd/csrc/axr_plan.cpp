@@ -356,7 +356,15 @@ int build_tables(axr_plan* p) {
   if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
   invalidate_tables(p);
   const Tunables& tn = tunables();
-  Builder b{p, static_cast<uint32_t>(tn.tile_rows) * kRowBytes};
+  uint32_t rows = static_cast<uint32_t>(tn.tile_rows);
+  if (rows == 0) {
+    rows = 2;
+    while (rows < kMaxTileRows &&
+           p->payload_bytes / (static_cast<uint64_t>(rows) * kRowBytes) >
+               static_cast<uint64_t>(tn.max_tiles))
+      rows *= 2;
+  }
+  Builder b{p, rows * kRowBytes};
 
   for (size_t i = 0; i < p->tensors.size(); ++i) {
     const TensorRec& t = p->tensors[i];
@@ -399,22 +407,23 @@ int build_tables(axr_plan* p) {
   sentinel.tile_begin = p->ntiles;
   p->segs.push_back(sentinel);
 
-  // launch geometry
-  int cus = 256;
-  if (device_compute_units(&cus) != AXR_OK || cus <= 0) cus = 256;
-  const uint64_t waves = static_cast<uint64_t>(cus) * static_cast<uint64_t>(tn.waves_per_cu);
-  uint64_t tpw = (p->ntiles + waves - 1) / waves;
-  if (tpw < static_cast<uint64_t>(tn.min_tiles_per_wave)) tpw = tn.min_tiles_per_wave;
+  // launch geometry: one tile per wave until the grid would exceed max_waves
+  uint64_t tpw = (p->ntiles + static_cast<uint64_t>(tn.max_waves) - 1) /
+                 static_cast<uint64_t>(tn.max_waves);
   if (tpw == 0) tpw = 1;
-  const uint64_t per_wg = tpw * kWavesPerWorkgroup;
+  p->cfg.threads = static_cast<uint32_t>(tn.threads);
+  const uint32_t waves_per_wg = p->cfg.threads / kWaveLanes;
+  const uint64_t per_wg = tpw * waves_per_wg;
   p->cfg.tiles_per_wave = static_cast<uint32_t>(tpw);
   p->cfg.workgroups = static_cast<uint32_t>((p->ntiles + per_wg - 1) / per_wg);
-  p->cfg.tile_rows = static_cast<uint32_t>(tn.tile_rows);
+  p->cfg.xcd_remap = tn.xcd_remap != 0 && p->cfg.workgroups >= 4 * kXcds;
+  if (p->cfg.xcd_remap) p->cfg.workgroups = (p->cfg.workgroups + kXcds - 1) / kXcds * kXcds;
+  p->cfg.tile_rows = rows;
   p->cfg.nontemporal = tn.nontemporal != 0;
   p->cfg.elements = false;
   for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode == kModeElements;
 
-  const size_t nwaves = static_cast<size_t>(p->cfg.workgroups) * kWavesPerWorkgroup;
+  const size_t nwaves = static_cast<size_t>(p->cfg.workgroups) * waves_per_wg;
   p->wave_seg.assign(nwaves, 0);
   size_t s = 0;
   const size_t nseg = p->segs.size() - 1;
@@ -502,7 +511,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   a.nseg = static_cast<uint32_t>(p->segs.size() - 1);
   a.ntiles = p->ntiles;
   a.tiles_per_wave = p->cfg.tiles_per_wave;
-  a.reserved = 0;
+  a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
   rc = launch_bundle_kernel(pack, a, p->cfg, stream);
   if (rc) return rc;
   if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
@@ -766,7 +775,7 @@ int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
   int rc = build_tables(plan);
   if (rc) return rc;
   info->workgroups = plan->cfg.workgroups;
-  info->threads_per_workgroup = kThreadsPerWorkgroup;
+  info->threads_per_workgroup = plan->cfg.threads;
   info->tiles = plan->ntiles;
   info->tile_bytes = plan->cfg.tile_rows * kRowBytes;
   info->segments = static_cast<uint32_t>(plan->segs.size() - 1);

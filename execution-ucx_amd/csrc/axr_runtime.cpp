@@ -282,21 +282,28 @@ int axr_tune_set(const char* key, int64_t value) {
   if (!key) return fail(AXR_ERR_INVALID, "axr_tune_set: null key");
   Tunables& t = tunables();
   const std::string k(key);
-  if (k == "waves_per_cu") {
-    if (value < 1 || value > 64) return fail(AXR_ERR_INVALID, "waves_per_cu must be 1..64");
-    t.waves_per_cu = value;
-  } else if (k == "tile_rows") {
-    if (value != 4 && value != 8 && value != 16)
-      return fail(AXR_ERR_INVALID, "tile_rows must be 4, 8 or 16");
+  if (k == "tile_rows") {
+    if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
+      return fail(AXR_ERR_INVALID, "tile_rows must be 0 (auto), 1, 2, 4, 8 or 16");
     t.tile_rows = value;
+  } else if (k == "max_tiles") {
+    if (value < 1) return fail(AXR_ERR_INVALID, "max_tiles must be positive");
+    t.max_tiles = value;
+  } else if (k == "max_waves") {
+    if (value < 1 || value > (1ll << 30)) return fail(AXR_ERR_INVALID, "max_waves must be in [1, 2^30]");
+    t.max_waves = value;
   } else if (k == "nontemporal") {
     t.nontemporal = value ? 1 : 0;
   } else if (k == "gather_run_bytes") {
-    if (value < 1) return fail(AXR_ERR_INVALID, "gather_run_bytes must be positive");
+    if (value < 1 || value > (1 << 20))
+      return fail(AXR_ERR_INVALID, "gather_run_bytes must be in [1, 2^20]");
     t.gather_run_bytes = value;
-  } else if (k == "min_tiles_per_wave") {
-    if (value < 1) return fail(AXR_ERR_INVALID, "min_tiles_per_wave must be positive");
-    t.min_tiles_per_wave = value;
+  } else if (k == "threads") {
+    if (value < 64 || value > 1024 || value % 64)
+      return fail(AXR_ERR_INVALID, "threads must be a multiple of 64 in [64, 1024]");
+    t.threads = value;
+  } else if (k == "xcd_remap") {
+    t.xcd_remap = value ? 1 : 0;
   } else {
     return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   }
@@ -307,11 +314,13 @@ int axr_tune_get(const char* key, int64_t* value) {
   if (!key || !value) return fail(AXR_ERR_INVALID, "axr_tune_get: null argument");
   const Tunables& t = tunables();
   const std::string k(key);
-  if (k == "waves_per_cu") *value = t.waves_per_cu;
-  else if (k == "tile_rows") *value = t.tile_rows;
+  if (k == "tile_rows") *value = t.tile_rows;
+  else if (k == "max_tiles") *value = t.max_tiles;
+  else if (k == "max_waves") *value = t.max_waves;
   else if (k == "nontemporal") *value = t.nontemporal;
   else if (k == "gather_run_bytes") *value = t.gather_run_bytes;
-  else if (k == "min_tiles_per_wave") *value = t.min_tiles_per_wave;
+  else if (k == "threads") *value = t.threads;
+  else if (k == "xcd_remap") *value = t.xcd_remap;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

@@ -210,6 +210,36 @@ def test_arbitrary_alignment(pkg, orc, gpu, seed):
         assert np.array_equal(hd, expect), (align, shift)       # bytes between tensors untouched
 
 
+@pytest.mark.parametrize("rows", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("threads", [64, 256, 1024])
+def test_every_kernel_instantiation(pkg, orc, gpu, rows, threads):
+    """Each tile size / workgroup size / temporal variant against the oracle,
+    with several tiles per wave forced as well."""
+    import torch
+    rng = np.random.default_rng(rows * 1000 + threads)
+    sizes = [0, 5, 16, 17, 1000, 1024, 1025, 2048, 4097, 16384, 16400, 70001, 3 * 16384 + 100]
+    sizes += [int(x) for x in rng.integers(1, 60000, size=20)]
+    tensors = [rand_bytes_tensor(rng, n, gpu) for n in sizes]
+    mat = rand_bytes_tensor(rng, 200 * 3000, gpu).reshape(200, 3000)
+    tensors += [mat[::2, 16:2064], mat.t()[5:9]]           # run tiles and element mode
+    chunks = [tbytes(t) for t in tensors]
+    try:
+        for nt, max_waves in ((1, 1 << 20), (0, 1 << 20), (1, 7)):
+            pkg.tune(tile_rows=rows, threads=threads, nontemporal=nt, max_waves=max_waves)
+            for align in (1, 256):
+                got, plan, buf = run_pack(pkg, tensors, align, gpu)
+                info = plan.launch_info()
+                assert info["tile_bytes"] == rows * 1024 and info["threads_per_workgroup"] == threads
+                assert np.array_equal(got, orc.pack(chunks, align)), (nt, max_waves, align)
+                outs = [torch.zeros_like(t, memory_format=torch.contiguous_format) for t in tensors]
+                pkg.BundlePlan.from_header(plan.header).bind(outs).unpack(buf.data_ptr(), plan.payload_bytes)
+                torch.cuda.synchronize()
+                for o, c in zip(outs, chunks):
+                    assert np.array_equal(tbytes(o), c), (nt, max_waves, align)
+    finally:
+        pkg.tune(tile_rows=0, threads=256, nontemporal=1, max_waves=1 << 20)
+
+
 # ------------------------------------------------------------------ strided views
 
 def random_torch_view(rng, parent, max_dims):
