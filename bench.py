@@ -38,6 +38,9 @@ def parse_args():
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--tune", default="", help="comma separated key=value kernel tunables")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
+                    help="also run N plain 256 MiB device copies (axr_copy_reference) so that "
+                         "profiler counters can be scaled by a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -175,6 +178,7 @@ def make_c5_sets(h, count):
 
 def verify_set(h, s):
     """One pack + unpack, then destination == source on the device."""
+    h.sync()      # inputs were produced on torch's stream, the bundle kernels run on ours
     h.capi.check(h.lib.axr_pack(s.pp, s.ptr, s.nbytes, h.stream))
     h.capi.check(h.lib.axr_unpack(s.up, s.ptr, s.nbytes, h.stream))
     h.sync()
@@ -375,6 +379,14 @@ def main():
                                   "payload_bytes_P": c4.data_bytes, "steps": k4}
         del c4
         torch.cuda.empty_cache()
+    if args.calibrate_copy:
+        n = 256 << 20
+        a = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(args.calibrate_copy):
+            pkg._capi.check(h.lib.axr_copy_reference(b.data_ptr(), a.data_ptr(), n, h.stream))
+        h.sync()
+        extras["calibration_copy_bytes"] = n
     result["extras"] = extras
 
     if not args.no_cpu:
