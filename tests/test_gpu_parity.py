@@ -100,6 +100,24 @@ def test_buffer_to_vec_kat(pkg, gpu):
     assert views == [(f.data_ptr() + 2048 * k, 2048) for k in range(4)]
 
 
+def test_golden_small_bundle(pkg, gpu):
+    """Committed vectors (tests/golden/small_bundle_v1.json): chunks -> packed bytes."""
+    import json
+    import os
+    import torch
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "small_bundle_v1.json")))
+    chunks = [np.frombuffer(bytes.fromhex(h), dtype=np.uint8) for h in fx["chunks_hex"]]
+    dev = [torch.from_numpy(c.copy()).to(gpu) for c in chunks]
+    for align, hexed in fx["packed"].items():
+        got, plan, buf = run_pack(pkg, dev, int(align), gpu)
+        assert got.tobytes().hex() == hexed
+        outs = [torch.full((c.size,), 0x11, dtype=torch.uint8, device=gpu) for c in chunks]
+        pkg.BundlePlan.from_header(plan.header).bind(outs).unpack(buf.data_ptr(), plan.payload_bytes)
+        torch.cuda.synchronize()
+        for o, c in zip(outs, chunks):
+            assert np.array_equal(o.cpu().numpy(), c)
+
+
 # ------------------------------------------------------------------ config 1: host tensors
 
 def test_c1_host_bundle(pkg, orc, gpu):

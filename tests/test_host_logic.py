@@ -1,0 +1,378 @@
+"""Host-side logic that needs no GPU: the C-ABI library loads and exports what
+the header declares, the planner agrees with the oracle, the header codec
+matches the golden fixtures, the segment table is what the design says, and
+every path that would need a device fails loudly instead of falling back."""
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def tv(pkg, ptr, shape, strides=None, dtype=(1, 8, 1), device_type=10):
+    return pkg.TensorView(data=ptr, device_type=device_type, device_id=0, dtype=dtype,
+                          shape=tuple(shape), strides=None if strides is None else tuple(strides))
+
+
+# ------------------------------------------------------------------ the C ABI itself
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "axon_rocm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"AXR_API\s+[\w\s\*]+?\b(axr_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = pkg._capi.load()
+    names = declared_functions()
+    assert len(names) >= 55
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/axon_rocm.h but not exported"
+    assert sorted(pkg._capi.PROTOTYPES) == names      # the ctypes binding covers the same set
+
+
+def test_structs_match_dlpack_and_ucx_layouts(pkg):
+    t = pkg._capi.Tensor
+    assert C.sizeof(t) == 48                           # sizeof(DLTensor) on LP64
+    assert (t.data.offset, t.device_type.offset, t.device_id.offset, t.ndim.offset) == (0, 8, 12, 16)
+    assert (t.dtype_code.offset, t.dtype_bits.offset, t.dtype_lanes.offset) == (20, 21, 22)
+    assert (t.shape.offset, t.strides.offset, t.byte_offset.offset) == (24, 32, 40)
+    assert C.sizeof(pkg._capi.Buffer) == 16            # ucx_buffer_t {void*, size_t}
+
+
+def test_status_and_version(pkg):
+    lib = pkg._capi.load()
+    assert lib.axr_version().decode().count(".") == 2
+    assert lib.axr_status_string(0) == b"AXR_OK"
+    assert lib.axr_status_string(-4) == b"AXR_ERR_LENGTH"
+    assert lib.axr_status_string(-12345).startswith(b"AXR_ERR_")
+
+
+def test_device_type_maps(pkg):
+    # axon/python/src/dlpack_helpers.cpp:82-134 and ucx_context_def.h:27-39
+    lib = pkg._capi.load()
+    to_mem = {1: 0, 2: 1, 13: 2, 10: 3, 11: 4, 14: 9, 4: 9, 7: 9, 8: 9}
+    for dl, mem in to_mem.items():
+        assert lib.axr_dl_device_to_memory_type(dl) == mem
+    to_dl = {0: 1, 1: 2, 2: 13, 3: 10, 4: 11, 5: 1, 6: 14, 7: 14, 8: 14, 9: 1}
+    for mem, dl in to_dl.items():
+        assert lib.axr_memory_type_to_dl_device(mem) == dl
+
+
+def test_tunables(pkg):
+    lib = pkg._capi.load()
+    v = C.c_int64()
+    for key, good, bad in ((b"tile_rows", 4, 3), (b"threads", 512, 100), (b"max_waves", 99, 0),
+                           (b"gather_run_bytes", 64, 0), (b"max_tiles", 1000, 0)):
+        before = C.c_int64()
+        assert lib.axr_tune_get(key, C.byref(before)) == 0
+        assert lib.axr_tune_set(key, good) == 0
+        assert lib.axr_tune_get(key, C.byref(v)) == 0 and v.value == good
+        assert lib.axr_tune_set(key, bad) == pkg._capi.AXR_ERR_INVALID
+        assert lib.axr_tune_set(key, before.value) == 0
+    assert lib.axr_tune_set(b"no_such_knob", 1) == pkg._capi.AXR_ERR_INVALID
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.tune(no_such_knob=1)
+
+
+# ------------------------------------------------------------------ size rule and layout
+
+def test_nbytes_rule_matches_oracle(pkg, orc):
+    lib = pkg._capi.load()
+    rng = np.random.default_rng(0)
+    for _ in range(300):
+        nd = int(rng.integers(0, 6))
+        shape = [int(x) for x in rng.integers(0, 9, size=nd)]
+        bits = int(rng.choice([1, 4, 8, 12, 16, 32, 64, 128]))
+        arr = pkg.dlpack.TensorArray([tv(pkg, 0x1000, shape, dtype=(0, bits, 1))])
+        out = C.c_uint64()
+        pkg._capi.check(lib.axr_tensor_nbytes(arr.pointer(), C.byref(out)))
+        assert out.value == orc.tensor_nbytes(shape, bits)
+    bad = pkg.dlpack.TensorArray([tv(pkg, 0x1000, [3, -1])])
+    assert lib.axr_tensor_nbytes(bad.pointer(), C.byref(out)) == pkg._capi.AXR_ERR_INVALID
+
+
+@pytest.mark.parametrize("align", [1, 2, 16, 256, 4096])
+def test_layout_matches_oracle(pkg, orc, align):
+    rng = np.random.default_rng(align)
+    for _ in range(20):
+        n = int(rng.integers(0, 50))
+        sizes = [int(x) for x in rng.integers(0, 5000, size=n)]
+        views = [tv(pkg, 0x10000, [s]) for s in sizes]
+        plan = pkg.BundlePlan.create(views, align=align)
+        offs, got_sizes = plan.layout()
+        want_offs, want_total = orc.layout(sizes, align)
+        assert got_sizes == sizes and offs == want_offs and plan.payload_bytes == want_total
+        assert plan.data_bytes == sum(sizes)
+        plan.close()
+
+
+@pytest.mark.parametrize("align", [0, 3, 8192])
+def test_bad_alignment_rejected(pkg, align):
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.create([tv(pkg, 0x1000, [4])], align=align)
+
+
+def test_split_matches_reference_semantics(pkg, orc):
+    kat = json.load(open(os.path.join(GOLDEN, "kat_patterns.json")))["split"]
+    buf = np.arange(kat["buffer_bytes"], dtype=np.uint8)
+    plan = pkg.BundlePlan.create([tv(pkg, 0x1000, [s]) for s in kat["sizes"]], align=1)
+    views = plan.split(buf.ctypes.data, buf.size)
+    assert [p - buf.ctypes.data for p, _ in views] == kat["offsets"] == orc.split(buf, kat["sizes"])
+    assert [n for _, n in views] == kat["sizes"]
+    over = json.load(open(os.path.join(GOLDEN, "kat_patterns.json")))["split_overflow"]
+    plan2 = pkg.BundlePlan.create([tv(pkg, 0x1000, [s]) for s in over["sizes"]], align=1)
+    with pytest.raises(pkg.LengthError):
+        plan2.split(buf.ctypes.data, over["buffer_bytes"])
+
+
+# ------------------------------------------------------------------ header
+
+def fixture_views(pkg, tensors):
+    return [tv(pkg, 0x7000_0000_0000, t["shape"], dtype=tuple(t["dtype"]), device_type=t["device"][0])
+            for t in tensors]
+
+
+def test_header_matches_golden_fixture_and_oracle(pkg, orc):
+    fx = json.load(open(os.path.join(GOLDEN, "bundle_header_v1.json")))
+    for case in fx["cases"]:
+        views = fixture_views(pkg, fx["tensors"])
+        for v, t in zip(views, fx["tensors"]):
+            v.device_id = t["device"][1]
+        plan = pkg.BundlePlan.create(views, align=case["align"])
+        assert plan.header.hex() == case["header_hex"]
+        align, total, tensors = orc.decode_header(plan.header)
+        assert align == case["align"] and total == plan.payload_bytes
+        back = pkg.BundlePlan.from_header(bytes.fromhex(case["header_hex"]))
+        assert back.layout() == plan.layout() and back.payload_bytes == plan.payload_bytes
+        for m, t in zip(back.metas(), fx["tensors"]):
+            assert m.device == tuple(t["device"]) and m.dtype == tuple(t["dtype"])
+            assert m.shape == tuple(t["shape"]) and m.byte_offset == 0
+        assert back.header == plan.header
+
+
+def test_malformed_headers_are_refused(pkg, orc):
+    good = orc.encode_header([{"device": (10, 0), "dtype": (2, 32, 1), "shape": (100,)},
+                              {"device": (10, 0), "dtype": (0, 8, 1), "shape": (7, 3)}], 256)
+    pkg.BundlePlan.from_header(good)
+
+    def broken(edit):
+        b = bytearray(good)
+        edit(b)
+        return bytes(b)
+
+    cases = {
+        "magic": broken(lambda b: b.__setitem__(0, b[0] ^ 1)),
+        "version": broken(lambda b: b.__setitem__(4, 2)),
+        "flags": broken(lambda b: b.__setitem__(6, 1)),
+        "align": broken(lambda b: b.__setitem__(12, 3)),
+        "payload size": broken(lambda b: b.__setitem__(16, b[16] ^ 1)),
+        "offset": broken(lambda b: b.__setitem__(24 + 48, 1)),      # second tensor's offset
+        "nbytes": broken(lambda b: b.__setitem__(24 + 8, b[24 + 8] ^ 1)),
+        "byte_offset": broken(lambda b: b.__setitem__(24 + 32, 1)),
+        "ndim": broken(lambda b: b.__setitem__(24 + 24, 5)),
+        "truncated": good[:-3],
+        "trailing": good + b"\0",
+        "short": good[:10],
+    }
+    for what, blob in cases.items():
+        with pytest.raises(pkg.HeaderError):
+            pkg.BundlePlan.from_header(blob)
+            pytest.fail(f"header with bad {what} accepted")
+
+
+# ------------------------------------------------------------------ segment table
+
+def seg_of(pkg, view, align=256, **tune):
+    if tune:
+        pkg.tune(**tune)
+    try:
+        plan = pkg.BundlePlan.create([view], align=align)
+        return plan.segments(), plan.launch_info()
+    finally:
+        if tune:
+            pkg.tune(tile_rows=0, gather_run_bytes=512)
+
+
+def test_compact_tensor_is_one_run(pkg):
+    segs, info = seg_of(pkg, tv(pkg, 0x10000, [3, 1, 500], strides=[500, 77, 1], dtype=(2, 32, 1)))
+    assert len(segs) == 1
+    s = segs[0]
+    assert (s["mode"], s["run_bytes"], s["nbytes"], s["ndim"]) == (0, 6000, 6000, 0)
+    assert s["tiles"] == 3 and info["tile_bytes"] == 2048 and info["tiles"] == 3
+
+
+def test_kv_block_view_collapses_to_64_runs(pkg):
+    from execution_ucx_amd import workloads
+    spec = workloads.kv_gather()
+    v = workloads.kv_block_view(0x7f00_0000_0000, spec, 17)
+    segs, info = seg_of(pkg, v)
+    assert len(segs) == 1
+    s = segs[0]
+    assert s["mode"] == 1 and s["run_bytes"] == 32768 and s["nbytes"] == 64 * 32768
+    assert s["shape"] == (64,) and s["stride_bytes"] == (4096 * 32768,)      # layer and K/V merge
+    assert s["address"] == 0x7f00_0000_0000 + 17 * 32768
+
+
+def test_pitched_view_rows(pkg):
+    from execution_ucx_amd import workloads
+    spec = workloads.pitched_chunk()
+    v = workloads.pitched_views(0x7f00_0000_0000, spec)[1]
+    segs, _ = seg_of(pkg, v)
+    s = segs[0]
+    assert (s["mode"], s["run_bytes"], s["shape"], s["stride_bytes"]) == (1, 4096, (1024,), (6144,))
+    assert s["tiles"] == 1024 * 2
+
+
+def test_short_runs_use_element_mode(pkg):
+    # transposed matrix: no contiguous inner run
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(4, 16, 1)))
+    s = segs[0]
+    assert (s["mode"], s["run_bytes"], s["granule"]) == (2, 2, 2)
+    assert s["shape"] == (30, 20) and s["stride_bytes"] == (2, 60)
+    # 24-byte runs of fp64 -> 8-byte granules; 12-byte elements -> 4-byte granules
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 3], strides=[10, 1], dtype=(2, 64, 1)))
+    assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 24, 8)
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 3], strides=[7, 2], dtype=(2, 96, 1)))
+    assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 12, 4)
+    # the threshold is a tunable
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=200)
+    assert segs[0]["mode"] == 1
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=400)
+    assert segs[0]["mode"] == 2 and segs[0]["granule"] == 4
+
+
+def test_negative_and_many_strides(pkg):
+    segs, _ = seg_of(pkg, tv(pkg, 0x20000, [4, 600], strides=[-1000, 1]))
+    assert segs[0]["stride_bytes"] == (-1000,) and segs[0]["mode"] == 1
+    # 8 strided outer dims: the two outermost are peeled on the host
+    shape = [2, 3, 2, 2, 2, 2, 2, 2, 600]
+    strides, acc = [], 700
+    for n in reversed(shape[:-1]):
+        strides.insert(0, acc)
+        acc *= n + 1                       # leave gaps so nothing merges
+    strides.append(1)
+    segs, _ = seg_of(pkg, tv(pkg, 0x100000, shape, strides=strides))
+    assert len(segs) == 6 and all(s["ndim"] == 6 and s["mode"] == 1 for s in segs)
+    assert [s["offset"] for s in segs] == [i * 64 * 600 for i in range(6)]
+    assert segs[1]["address"] - segs[0]["address"] == strides[1]
+    assert segs[3]["address"] - segs[0]["address"] == strides[0]
+
+
+def test_pads_fill_segments_and_host_copies(pkg):
+    views = [tv(pkg, 0x10000, [100]),                       # device, pad 156
+             tv(pkg, 0x20000, [0]),                         # empty: no segment
+             tv(pkg, 0x30000, [256]),                       # device, pad 0
+             tv(pkg, 0x40000, [3, 10], strides=[20, 1], device_type=1),   # host, 3 copies + fill
+             tv(pkg, 0x50000, [7], device_type=11)]         # pinned host: device segment, last
+    plan = pkg.BundlePlan.create(views, align=256)
+    segs = plan.segments()
+    dev = [s for s in segs if s["mode"] != 4]
+    host = [s for s in segs if s["mode"] == 4]
+    assert [(s["tensor"], s["mode"], s["pad"]) for s in dev] == [(0, 0, 156), (2, 0, 0), (3, 3, 226), (4, 0, 0)]
+    assert dev[2]["offset"] == 512 + 30
+    assert [(s["address"], s["offset"], s["nbytes"]) for s in host] == [
+        (0x40000, 512, 10), (0x40000 + 20, 522, 10), (0x40000 + 40, 532, 10)]
+    assert plan.launch_info()["host_copies"] == 3
+    assert plan.payload_bytes == 768 + 7
+
+
+def test_unsupported_device_type_fails(pkg):
+    plan = pkg.BundlePlan.create([tv(pkg, 0x1000, [16], device_type=2)], align=1)   # kDLCUDA
+    with pytest.raises(pkg.UnsupportedMemoryError):
+        plan.segments()
+
+
+def test_bind_validation(pkg, orc):
+    hdr = orc.encode_header([{"device": (10, 0), "dtype": (2, 32, 1), "shape": (100,)},
+                             {"device": (10, 0), "dtype": (4, 16, 1), "shape": (8, 8)}], 256)
+    plan = pkg.BundlePlan.from_header(hdr)
+    with pytest.raises(pkg.AxonRocmError):
+        plan.segments()                                          # nothing bound
+    with pytest.raises(pkg.MismatchError):
+        plan.bind([tv(pkg, 0x1000, [100], dtype=(2, 32, 1))])    # count
+    with pytest.raises(pkg.MismatchError):
+        plan.bind([tv(pkg, 0x1000, [100], dtype=(2, 32, 1)), tv(pkg, 0x2000, [8, 9], dtype=(4, 16, 1))])
+    with pytest.raises(pkg.MismatchError):                       # same bytes, other element width
+        plan.bind([tv(pkg, 0x1000, [100], dtype=(2, 32, 1)), tv(pkg, 0x2000, [32], dtype=(2, 32, 1))])
+    # a destination view with other strides but the same shape is fine
+    plan.bind([tv(pkg, 0x1000, [100], dtype=(0, 32, 1)),
+               tv(pkg, 0x2000, [8, 8], strides=[16, 1], dtype=(2, 16, 1))])
+    assert [s["mode"] for s in plan.segments()] == [0, 2]
+
+
+# ------------------------------------------------------------------ DLPack and devices
+
+def test_dlpack_extract_numpy(pkg):
+    a = np.arange(24, dtype=np.float32).reshape(4, 6)
+    v = pkg.extract(a[:, 1:4])
+    assert v.device_type == 1 and v.dtype == (2, 32, 1) and v.shape == (4, 3)
+    assert v.strides == (6, 1) and v.data + v.byte_offset == a[:, 1:4].ctypes.data
+    assert v.nbytes == 48
+    with pytest.raises(TypeError):
+        pkg.extract(object())
+
+
+def test_dlpack_export_single_consume(pkg):
+    released = []
+    src = np.arange(40, dtype=np.int32)
+    exp = pkg.DLPackExport(src.ctypes.data, (5, 8), (0, 32, 1), 1, 0, release=lambda: released.append(1))
+    assert exp.__dlpack_device__() == (1, 0)
+    out = np.from_dlpack(exp)
+    assert out.shape == (5, 8) and out.dtype == np.int32 and np.array_equal(out.reshape(-1), src)
+    with pytest.raises(RuntimeError):
+        exp.__dlpack__()
+    del out
+    import gc
+    gc.collect()
+    assert released == [1]
+    # never consumed: released when dropped
+    exp2 = pkg.DLPackExport(src.ctypes.data, 160, (1, 8, 1), 1, 0, release=lambda: released.append(2))
+    del exp2
+    gc.collect()
+    assert released == [1, 2]
+
+
+def test_device_objects(pkg):
+    d = pkg.rocm(3)
+    assert d.get_type() == pkg.DeviceType.ROCM and d.get_type_string() == "rocm"
+    assert d.get_context_handle() == 3 and repr(d) == "RocmDevice(device_id=3)"
+    assert d.clone().device_id == 3
+    c = pkg.cpu(numa_node=1)
+    assert c.get_type_string() == "cpu" and c.get_context_handle() is None
+    assert isinstance(pkg.auto_detect(), pkg.Device)
+
+
+# ------------------------------------------------------------------ no device: fail loudly
+
+def test_no_silent_cpu_fallback_without_gpu(pkg):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    assert pkg.device_count() == 0
+    assert isinstance(pkg.auto_detect(), pkg.CpuDevice)
+    src = np.arange(64, dtype=np.uint8)
+    plan = pkg.BundlePlan.create([src], align=1)
+    host_payload = np.zeros(64, np.uint8)
+    with pytest.raises(pkg.AxonRocmError):          # host tensors still move through HIP copies
+        plan.pack(host_payload.ctypes.data, 64)
+    assert not host_payload.any()
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.DevicePool(device=0)
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.RocmMemoryResourceManager().allocate(3, 1024)
+    with pytest.raises(pkg.AxonRocmError):
+        with pkg.rocm(0).activate():
+            pass
+
+
+def test_missing_library_is_an_import_error(pkg, monkeypatch):
+    monkeypatch.setattr(pkg._capi, "_lib", None)
+    monkeypatch.setattr(pkg._capi, "LIBRARY_PATH", "/nonexistent/libaxon_rocm.so")
+    with pytest.raises(ImportError):
+        pkg._capi.load()
