@@ -7,11 +7,12 @@ nothing here computes on the CPU.
 """
 from . import _capi
 from ._capi import (AxonRocmError, HeaderError, LengthError, MismatchError, NoDeviceError,
-                    UnsupportedMemoryError)
+                    NoMessageError, NotImplementedForEager, UnsupportedMemoryError)
 from .bundle import BundlePlan, PackedBundle, TensorMeta, pack_bundle, unpack_bundle
 from .device import (CpuDevice, Device, DeviceType, RocmDevice, auto_detect, cpu, device_count,
                      rocm)
 from .dlpack import DLPackExport, TensorView, extract, extract_many
+from .loopback import AmMessage, LoopbackAmContext
 from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager
 
 __version__ = "0.1.0"

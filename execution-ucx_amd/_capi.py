@@ -73,12 +73,22 @@ class NoDeviceError(AxonRocmError):
     """No usable ROCm device."""
 
 
+class NoMessageError(AxonRocmError, LookupError):
+    """Unknown receive key (UCS_ERR_NO_MESSAGE, ucx_am_context.hpp:1570-1574)."""
+
+
+class NotImplementedForEager(AxonRocmError, NotImplementedError):
+    """recv_buffer on an eager message (UCS_ERR_NOT_IMPLEMENTED, :1643-1651)."""
+
+
 _ERROR_TYPES = {
     AXR_ERR_LENGTH: LengthError,
     AXR_ERR_UNSUPPORTED: UnsupportedMemoryError,
     AXR_ERR_HEADER: HeaderError,
     AXR_ERR_MISMATCH: MismatchError,
     AXR_ERR_NO_DEVICE: NoDeviceError,
+    AXR_ERR_NO_MESSAGE: NoMessageError,
+    AXR_ERR_NOT_IMPLEMENTED: NotImplementedForEager,
 }
 
 # ---------------------------------------------------------------- structures
@@ -147,6 +157,25 @@ class SegmentInfo(C.Structure):
     ]
 
 
+class AmData(C.Structure):
+    """axr_am_data_t == ucx_am_data_t."""
+
+    _fields_ = [("header", Buffer), ("buffer", Buffer), ("buffer_type", C.c_int), ("mem_h", C.c_void_p)]
+
+
+class AmIovec(C.Structure):
+    """axr_am_iovec_t == ucx_am_iovec_t."""
+
+    _fields_ = [("header", Buffer), ("buffer_vec", C.POINTER(Buffer)), ("buffer_count", C.c_size_t),
+                ("buffer_type", C.c_int), ("mem_h", C.c_void_p)]
+
+
+class AmMessage(C.Structure):
+    _fields_ = [("key", C.c_uint64), ("conn_id", C.c_uint64), ("header", Buffer),
+                ("data_length", C.c_uint64), ("is_rndv", C.c_int), ("buffer_type", C.c_int),
+                ("eager_data", Buffer)]
+
+
 REGISTER_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p))
 UNREGISTER_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)
 
@@ -213,6 +242,17 @@ PROTOTYPES = {
     "axr_plan_segments": (C.c_int, [_vp, C.POINTER(SegmentInfo), _sz, C.POINTER(_sz)]),
     "axr_tune_set": (C.c_int, [C.c_char_p, C.c_int64]),
     "axr_tune_get": (C.c_int, [C.c_char_p, _i64p]),
+    "axr_am_context_create": (C.c_int, [C.c_char_p, _sz, _vpp]),
+    "axr_am_context_destroy": (C.c_int, [_vp]),
+    "axr_am_connect": (C.c_int, [_vp, _vp, _u64p]),
+    "axr_am_send": (C.c_int, [_vp, C.c_uint64, C.POINTER(AmData), _vp, _u64p]),
+    "axr_am_send_iov": (C.c_int, [_vp, C.c_uint64, C.POINTER(AmIovec), _vp, _u64p]),
+    "axr_am_request_test": (C.c_int, [_vp, C.c_uint64, _intp]),
+    "axr_am_recv_header": (C.c_int, [_vp, C.POINTER(AmMessage)]),
+    "axr_am_recv_buffer": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
+    "axr_am_recv_buffer_iov": (C.c_int, [_vp, C.c_uint64, C.c_int, C.POINTER(Buffer), _sz, _vp]),
+    "axr_am_message_release": (C.c_int, [_vp, C.c_uint64]),
+    "axr_am_pending": (C.c_int, [_vp, C.POINTER(_sz)]),
     "axr_divide_by_two": (C.c_int, [_vp, _sz, _vp]),
     "axr_compare": (C.c_int, [_vp, _vp, _sz, _u64p]),
     "axr_checksum": (C.c_int, [_vp, _sz, C.c_uint64, _u64p]),

@@ -1,0 +1,297 @@
+// Loopback active-message context: the AM-bundle surface of the reference's
+// ucx_am_context for one process without UCX.  Semantics and reference lines
+// are given with the declarations in axon_rocm.h.
+#include <hip/hip_runtime_api.h>
+
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <new>
+
+#include "axr_internal.h"
+
+using namespace axr;
+
+namespace {
+
+struct Piece {
+  const void* data;
+  size_t size;
+};
+
+struct Request {
+  std::atomic<int> done{0};
+};
+
+struct Message {
+  uint64_t key = 0;
+  uint64_t conn_id = 0;
+  std::vector<uint8_t> header;
+  std::vector<uint8_t> eager;
+  std::vector<Piece> pieces;       // rendezvous: the sender's buffers
+  uint64_t data_length = 0;
+  bool rndv = false;
+  int buffer_type = AXR_MEM_HOST;
+  std::shared_ptr<Request> request;
+};
+
+bool host_type(int t) { return t == AXR_MEM_HOST || t == AXR_MEM_ROCM_MANAGED; }
+bool known_type(int t) { return host_type(t) || t == AXR_MEM_ROCM; }
+
+std::atomic<uint64_t> g_next_id{1};
+
+}  // namespace
+
+struct axr_am_context {
+  std::string name;
+  size_t zcopy_thresh = 4096;
+  std::mutex mu;
+  std::deque<std::unique_ptr<Message>> arrived;          // not yet seen by recv_header
+  std::map<uint64_t, std::unique_ptr<Message>> parked;   // handed out, awaiting fetch/release
+  std::map<uint64_t, axr_am_context*> endpoints;         // conn id -> peer
+  std::map<uint64_t, std::shared_ptr<Request>> requests;
+};
+
+namespace {
+
+size_t env_zcopy_thresh() {
+  const char* val = std::getenv("UCX_ZCOPY_THRESH");
+  if (!val) return 4096;
+  char* end = nullptr;
+  const long long v = std::strtoll(val, &end, 10);
+  if (end == val || v <= 0) return 4096;
+  return static_cast<size_t>(v);
+}
+
+int copy_piece(int dst_type, void* dst, int src_type, const void* src, size_t n, hipStream_t s) {
+  if (n == 0) return AXR_OK;
+  if (host_type(dst_type) && host_type(src_type)) {
+    std::memcpy(dst, src, n);
+    return AXR_OK;
+  }
+  return check_hip(hipMemcpyAsync(dst, src, n, hipMemcpyDefault, s), "hipMemcpyAsync(loopback)");
+}
+
+int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, uint64_t* request) {
+  axr_am_context* peer = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto it = ctx->endpoints.find(conn_id);
+    if (it == ctx->endpoints.end()) return fail(AXR_ERR_INVALID, "unknown connection id");
+    peer = it->second;
+    const uint64_t rid = g_next_id++;
+    ctx->requests[rid] = m->request;
+    if (request) *request = rid;
+  }
+  m->key = g_next_id++;
+  m->conn_id = conn_id;
+  std::lock_guard<std::mutex> lock(peer->mu);
+  peer->arrived.push_back(std::move(m));
+  return AXR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_t** ctx) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_context_create: null result");
+  axr_am_context* c = new (std::nothrow) axr_am_context();
+  if (!c) return fail(AXR_ERR_NOMEM, "axr_am_context_create: out of host memory");
+  c->name = name ? name : "";
+  c->zcopy_thresh = zcopy_thresh ? zcopy_thresh : env_zcopy_thresh();
+  *ctx = c;
+  return AXR_OK;
+}
+
+int axr_am_context_destroy(axr_am_context_t* ctx) {
+  if (!ctx) return AXR_OK;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    for (auto& m : ctx->arrived) m->request->done.store(-1);
+    for (auto& kv : ctx->parked) kv.second->request->done.store(-1);
+  }
+  delete ctx;
+  return AXR_OK;
+}
+
+int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_id) {
+  if (!from || !to || !conn_id) return fail(AXR_ERR_INVALID, "axr_am_connect: null argument");
+  const uint64_t id = g_next_id++;
+  std::lock_guard<std::mutex> lock(from->mu);
+  from->endpoints[id] = to;
+  *conn_id = id;
+  return AXR_OK;
+}
+
+int axr_am_send(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* d, void* stream,
+                uint64_t* request) {
+  if (!ctx || !d) return fail(AXR_ERR_INVALID, "axr_am_send: null argument");
+  if (!d->header.data || d->header.size == 0)
+    return fail(AXR_ERR_INVALID, "axr_am_send: the header must not be empty");
+  if ((d->buffer.data == nullptr) != (d->buffer.size == 0))
+    return fail(AXR_ERR_INVALID, "axr_am_send: buffer pointer and size disagree");
+  if (!known_type(d->buffer_type)) return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
+  std::unique_ptr<Message> m(new Message());
+  m->request = std::make_shared<Request>();
+  const uint8_t* h = static_cast<const uint8_t*>(d->header.data);
+  m->header.assign(h, h + d->header.size);
+  m->data_length = d->buffer.size;
+  m->buffer_type = d->buffer_type;
+  // a zero-length rendezvous is treated as eager (ucx_am_context.hpp:1955-1958)
+  m->rndv = d->buffer.size >= ctx->zcopy_thresh && d->buffer.size > 0;
+  if (m->rndv) {
+    m->pieces.push_back({d->buffer.data, d->buffer.size});
+  } else {
+    m->eager.resize(d->buffer.size);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc = copy_piece(AXR_MEM_HOST, m->eager.data(), d->buffer_type, d->buffer.data,
+                        d->buffer.size, s);
+    if (rc) return rc;
+    if (!host_type(d->buffer_type) && d->buffer.size) {
+      rc = check_hip(hipStreamSynchronize(s), "hipStreamSynchronize");
+      if (rc) return rc;
+    }
+    m->request->done.store(1);   // eager: the sender's buffer is free again
+  }
+  return deliver(ctx, conn_id, std::move(m), request);
+}
+
+int axr_am_send_iov(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* d, void* /*stream*/,
+                    uint64_t* request) {
+  if (!ctx || !d) return fail(AXR_ERR_INVALID, "axr_am_send_iov: null argument");
+  if (!d->header.data || d->header.size == 0)
+    return fail(AXR_ERR_INVALID, "axr_am_send_iov: the header must not be empty");
+  if ((d->buffer_vec == nullptr) != (d->buffer_count == 0))
+    return fail(AXR_ERR_INVALID, "axr_am_send_iov: buffer vector and count disagree");
+  if (!known_type(d->buffer_type)) return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
+  std::unique_ptr<Message> m(new Message());
+  m->request = std::make_shared<Request>();
+  const uint8_t* h = static_cast<const uint8_t*>(d->header.data);
+  m->header.assign(h, h + d->header.size);
+  m->buffer_type = d->buffer_type;
+  for (size_t i = 0; i < d->buffer_count; ++i) {
+    if (d->buffer_vec[i].size && !d->buffer_vec[i].data)
+      return fail(AXR_ERR_INVALID, "axr_am_send_iov: null entry with a size");
+    m->pieces.push_back({d->buffer_vec[i].data, d->buffer_vec[i].size});
+    m->data_length += d->buffer_vec[i].size;
+  }
+  m->rndv = m->data_length > 0;   // always rendezvous; nothing to fetch when empty
+  if (!m->rndv) m->request->done.store(1);
+  return deliver(ctx, conn_id, std::move(m), request);
+}
+
+int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done) {
+  if (!ctx || !done) return fail(AXR_ERR_INVALID, "axr_am_request_test: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto it = ctx->requests.find(request);
+  if (it == ctx->requests.end()) return fail(AXR_ERR_INVALID, "axr_am_request_test: unknown request");
+  const int st = it->second->done.load();
+  *done = st;
+  if (st != 0) ctx->requests.erase(it);
+  return AXR_OK;
+}
+
+int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* out) {
+  if (!ctx || !out) return fail(AXR_ERR_INVALID, "axr_am_recv_header: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (ctx->arrived.empty()) return fail(AXR_ERR_NO_MESSAGE, "no message queued");
+  std::unique_ptr<Message> m = std::move(ctx->arrived.front());
+  ctx->arrived.pop_front();
+  std::memset(out, 0, sizeof(*out));
+  out->key = m->key;
+  out->conn_id = m->conn_id;
+  out->header = axr_buffer_t{m->header.data(), m->header.size()};
+  out->data_length = m->data_length;
+  out->is_rndv = m->rndv ? 1 : 0;
+  out->buffer_type = m->buffer_type;
+  if (!m->rndv) out->eager_data = axr_buffer_t{m->eager.empty() ? nullptr : m->eager.data(), m->eager.size()};
+  const uint64_t key = m->key;
+  ctx->parked[key] = std::move(m);
+  return AXR_OK;
+}
+
+static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_buffer_t* vec,
+                 size_t count, void* stream) {
+  if (!known_type(dst_type)) return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
+  std::unique_ptr<Message> m;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto it = ctx->parked.find(key);
+    if (it == ctx->parked.end()) return fail(AXR_ERR_NO_MESSAGE, "no message with this key");
+    if (!it->second->rndv)
+      return fail(AXR_ERR_NOT_IMPLEMENTED, "message was eager: its data came with the header");
+    uint64_t room = 0;
+    for (size_t i = 0; i < count; ++i) room += vec[i].size;
+    if (room < it->second->data_length)
+      return fail(AXR_ERR_LENGTH, "receive buffer is smaller than the message");
+    m = std::move(it->second);
+    ctx->parked.erase(it);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // stream the sender's pieces, in order, into the receiver's entries, in order
+  size_t di = 0, doff = 0;
+  int rc = AXR_OK;
+  bool device_copy = false;
+  for (const Piece& p : m->pieces) {
+    size_t poff = 0;
+    while (poff < p.size && rc == AXR_OK) {
+      while (doff == vec[di].size) {
+        ++di;
+        doff = 0;
+      }
+      const size_t n = std::min(p.size - poff, vec[di].size - doff);
+      rc = copy_piece(dst_type, static_cast<uint8_t*>(vec[di].data) + doff, m->buffer_type,
+                      static_cast<const uint8_t*>(p.data) + poff, n, s);
+      device_copy = device_copy || !(host_type(dst_type) && host_type(m->buffer_type));
+      poff += n;
+      doff += n;
+    }
+    if (rc) break;
+  }
+  if (rc == AXR_OK && device_copy) rc = check_hip(hipStreamSynchronize(s), "hipStreamSynchronize");
+  m->request->done.store(rc == AXR_OK ? 1 : -1);
+  return rc;
+}
+
+int axr_am_recv_buffer(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst, size_t dst_bytes,
+                       void* stream) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null context");
+  if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null buffer");
+  axr_buffer_t one{dst, dst_bytes};
+  return fetch(ctx, key, dst_type, &one, 1, stream);
+}
+
+int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,
+                           const axr_buffer_t* buffer_vec, size_t buffer_count, void* stream) {
+  if (!ctx || !buffer_vec || buffer_count == 0)
+    return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_iov: null or empty buffer vector");
+  for (size_t i = 0; i < buffer_count; ++i) {
+    if (!buffer_vec[i].data || buffer_vec[i].size == 0)
+      return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_iov: every entry must be allocated and non-empty");
+  }
+  return fetch(ctx, key, dst_type, buffer_vec, buffer_count, stream);
+}
+
+int axr_am_message_release(axr_am_context_t* ctx, uint64_t key) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_message_release: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto it = ctx->parked.find(key);
+  if (it == ctx->parked.end()) return AXR_OK;   // already fetched: nothing left to drop
+  if (it->second->rndv) it->second->request->done.store(-1);
+  ctx->parked.erase(it);
+  return AXR_OK;
+}
+
+int axr_am_pending(axr_am_context_t* ctx, size_t* count) {
+  if (!ctx || !count) return fail(AXR_ERR_INVALID, "axr_am_pending: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  *count = ctx->arrived.size();
+  return AXR_OK;
+}
+
+}  // extern "C"

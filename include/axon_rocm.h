@@ -313,6 +313,87 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
 AXR_API int axr_tune_set(const char* key, int64_t value);
 AXR_API int axr_tune_get(const char* key, int64_t* value);
 
+/* ------------------------------------------------ loopback active messages */
+
+/* In-process stand-in for the reference's ucx_am_context, for machines without
+ * UCX: two contexts in one process joined by a loopback endpoint, the topology
+ * of test_code/test_cuda_connection.cpp:256-297.  It keeps the observable
+ * behaviour of connection_send / connection_recv_header / connection_recv_buffer
+ * (ucx_context/ucx_context_concept.hpp:247-470):
+ *   - a send needs a non-empty header; the payload may be empty
+ *     (ucx_am_context.hpp:2275-2284);
+ *   - a contiguous payload below the zcopy threshold (UCX_ZCOPY_THRESH, default
+ *     4096; ucx_connection.cpp:45,113-124) is eager: header and payload are copied
+ *     to host memory at send time and the send is complete; otherwise, and always
+ *     for an iov payload (ucx_connection.cpp:417-419), it is a rendezvous: only
+ *     the header is copied, the receiver fetches the payload with
+ *     axr_am_recv_buffer*, and the send completes then;
+ *   - messages are delivered in FIFO order per receiving context;
+ *   - an iov payload received into a contiguous buffer is the concatenation of
+ *     its entries in order (ucx_am_connection_test.cpp:1051-1108).
+ * Payload bytes move with device copies on `stream` (one per iov entry), which
+ * is also what UCX's rocm_copy transport would do for the reference's iov send. */
+
+typedef struct axr_am_context axr_am_context_t;
+
+/* == ucx_am_data_t / ucx_am_iovec_t (ucx_context/ucx_context_def.h:80-129) */
+typedef struct axr_am_data {
+  axr_buffer_t header;
+  axr_buffer_t buffer;
+  int buffer_type;   /* axr_memory_type_t */
+  void* mem_h;
+} axr_am_data_t;
+typedef struct axr_am_iovec {
+  axr_buffer_t header;
+  axr_buffer_t* buffer_vec;
+  size_t buffer_count;
+  int buffer_type;
+  void* mem_h;
+} axr_am_iovec_t;
+
+/* What connection_recv_header yields: for a rendezvous message the key under
+ * which the payload is parked, for an eager one the payload itself (host
+ * memory).  header / eager_data stay valid until axr_am_message_release. */
+typedef struct axr_am_message {
+  uint64_t key;
+  uint64_t conn_id;       /* reply connection, learned from the sender        */
+  axr_buffer_t header;    /* host copy of the AM header                       */
+  uint64_t data_length;
+  int is_rndv;
+  int buffer_type;        /* memory type of the sender's payload              */
+  axr_buffer_t eager_data;
+} axr_am_message_t;
+
+/* zcopy_thresh 0 reads UCX_ZCOPY_THRESH, else 4096. */
+AXR_API int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_t** ctx);
+AXR_API int axr_am_context_destroy(axr_am_context_t* ctx);
+/* Endpoint from `from` to `to`; *conn_id names it in axr_am_send*. */
+AXR_API int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_id);
+/* *request identifies the send for axr_am_request_test. */
+AXR_API int axr_am_send(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* data,
+                        void* stream, uint64_t* request);
+AXR_API int axr_am_send_iov(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* data,
+                            void* stream, uint64_t* request);
+AXR_API int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done);
+/* Next message in arrival order; AXR_ERR_NO_MESSAGE when none is queued. */
+AXR_API int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* message);
+/* Fetch a rendezvous payload into one contiguous buffer of memory type
+ * dst_type (blocking on `stream`).  Unknown key -> AXR_ERR_NO_MESSAGE; eager
+ * message -> AXR_ERR_NOT_IMPLEMENTED (ucx_am_context.hpp:1570-1574, 1643-1651);
+ * dst_bytes below data_length -> AXR_ERR_LENGTH. */
+AXR_API int axr_am_recv_buffer(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
+                               size_t dst_bytes, void* stream);
+/* Same into an iov: entries must be non-null and non-empty and add up to at
+ * least data_length (ucx_am_context.hpp:1808-1818); filled in order. */
+AXR_API int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,
+                                   const axr_buffer_t* buffer_vec, size_t buffer_count,
+                                   void* stream);
+/* Drop a message's host copies (and, for an unfetched rendezvous, complete the
+ * sender's request as cancelled). */
+AXR_API int axr_am_message_release(axr_am_context_t* ctx, uint64_t key);
+/* Messages queued and not yet taken by axr_am_recv_header. */
+AXR_API int axr_am_pending(axr_am_context_t* ctx, size_t* count);
+
 /* -------------------------------------------------- verification utilities */
 
 /* data[i] /= 2.0f in place; the device-side "process" step of the reference's

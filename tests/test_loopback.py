@@ -1,0 +1,228 @@
+"""The loopback AM context against the behaviour the reference's tests pin
+(ucx_am_connection_test.cpp, ucx_am_context_test.cpp).  Host-memory cases run
+without a GPU; the device cases are marked gpu."""
+import numpy as np
+import pytest
+
+HOST, ROCM = 0, 3
+
+
+def pattern(n, start=0):
+    return ((np.arange(n, dtype=np.uint64) + start) % 256).astype(np.uint8)
+
+
+@pytest.fixture
+def pair(pkg):
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    yield client, server, conn
+    client.close()
+    server.close()
+
+
+def test_header_is_required_and_payload_may_be_empty(pkg, pair):
+    client, server, conn = pair
+    with pytest.raises(pkg.AxonRocmError):
+        client.send(conn, b"", 0, 0, memory_type=HOST)
+    with pytest.raises(pkg.AxonRocmError):
+        client.send(conn + 12345, b"h", 0, 0, memory_type=HOST)      # unknown connection
+    req = client.send(conn, b"only header", 0, 0, memory_type=HOST)
+    assert client.test(req)
+    m = server.recv_header()
+    assert m.header == b"only header" and m.data_length == 0 and not m.is_rndv and m.eager_data == b""
+    assert m.conn_id == conn
+    assert server.recv_header() is None
+
+
+def test_eager_below_threshold_rendezvous_above(pkg):
+    # UCX_ZCOPY_THRESH default 4096 (ucx_connection.cpp:45); tests force 8192 (ucx_am_context_test.cpp:131)
+    client, server = pkg.LoopbackAmContext("c", zcopy_thresh=8192), pkg.LoopbackAmContext("s")
+    conn = client.connect(server)
+    src = pattern(8192)
+    r_small = client.send(conn, b"\x01", src.ctypes.data, 8191, memory_type=HOST)
+    r_big = client.send(conn, b"\x02", src.ctypes.data, 8192, memory_type=HOST)
+    assert client.test(r_small) and not client.test(r_big)
+    small = server.recv_header(release_eager=False)
+    assert not small.is_rndv and small.eager_data == src[:8191].tobytes()
+    dst = np.zeros(8192, np.uint8)
+    with pytest.raises(pkg.NotImplementedForEager):          # UCS_ERR_NOT_IMPLEMENTED
+        server.recv_into(small, dst.ctypes.data, 8192, memory_type=HOST)
+    server.release(small)
+    big = server.recv_header()
+    assert big.is_rndv and big.data_length == 8192 and big.eager_data is None
+    with pytest.raises(pkg.LengthError):
+        server.recv_into(big, dst.ctypes.data, 100, memory_type=HOST)
+    server.recv_into(big, dst.ctypes.data, 8192, memory_type=HOST)
+    assert np.array_equal(dst, src) and client.test(r_big)
+    with pytest.raises(pkg.NoMessageError):                  # UCS_ERR_NO_MESSAGE
+        server.recv_into(big, dst.ctypes.data, 8192, memory_type=HOST)
+
+
+@pytest.mark.parametrize("lens", [(256, 512, 300), (512 * 1024, 256 * 1024, 800 * 1024)])
+def test_iov_send_contiguous_and_iov_receive_kat(pkg, pair, lens):
+    """ucx_am_connection_test.cpp:933-1108: iov -> contiguous equals the flat
+    pattern; iov -> iov of the same lengths equals the segments; header echoed."""
+    client, server, conn = pair
+    segs, cursor = [], 0
+    for n in lens:
+        segs.append(pattern(n, cursor))
+        cursor += n
+    bufs = [(s.ctypes.data, s.size) for s in segs]
+    r1 = client.send_iov(conn, bytes([1, 2, 3, 4]), bufs, memory_type=HOST)
+    r2 = client.send_iov(conn, bytes([1, 2, 3, 4]), bufs, memory_type=HOST)
+    assert not client.test(r1)                               # iov is always rendezvous
+    m = server.recv_header()
+    assert m.header == bytes([1, 2, 3, 4]) and m.is_rndv and m.data_length == sum(lens)
+    flat = np.zeros(sum(lens), np.uint8)
+    server.recv_into(m, flat.ctypes.data, flat.size, memory_type=HOST)
+    assert np.array_equal(flat, pattern(sum(lens)))
+    m2 = server.recv_header()
+    outs = [np.zeros(n, np.uint8) for n in lens]
+    server.recv_buffer_iov(m2, [(o.ctypes.data, o.size) for o in outs], memory_type=HOST)
+    for o, s in zip(outs, segs):
+        assert np.array_equal(o, s)
+    assert client.test(r1) and client.test(r2)
+
+
+def test_iov_receive_needs_allocated_entries(pkg, pair):
+    client, server, conn = pair
+    src = pattern(100)
+    client.send_iov(conn, b"h", [(src.ctypes.data, 100)], memory_type=HOST)
+    m = server.recv_header()
+    dst = np.zeros(100, np.uint8)
+    with pytest.raises(pkg.AxonRocmError):
+        server.recv_buffer_iov(m, [(dst.ctypes.data, 50), (0, 50)], memory_type=HOST)
+    with pytest.raises(pkg.AxonRocmError):
+        server.recv_buffer_iov(m, [(dst.ctypes.data, 100), (dst.ctypes.data, 0)], memory_type=HOST)
+    server.recv_buffer_iov(m, [(dst.ctypes.data, 40), (dst.ctypes.data + 40, 60)], memory_type=HOST)
+    assert np.array_equal(dst, src)
+
+
+def test_fifo_order_and_cancel(pkg, pair):
+    client, server, conn = pair
+    src = pattern(10000)
+    reqs = [client.send(conn, bytes([i]), src.ctypes.data + i, 5000, memory_type=HOST) for i in range(5)]
+    assert server.pending() == 5
+    for i in range(5):
+        m = server.recv_header()
+        assert m.header == bytes([i])
+        if i == 2:
+            server.release(m)                                # receiver drops the descriptor
+            with pytest.raises(pkg.AxonRocmError):
+                client.test(reqs[i])
+            continue
+        dst = np.zeros(5000, np.uint8)
+        server.recv_into(m, dst.ctypes.data, 5000, memory_type=HOST)
+        assert np.array_equal(dst, src[i:i + 5000]) and client.test(reqs[i])
+
+
+def test_unsupported_memory_type(pkg, pair):
+    client, server, conn = pair
+    src = pattern(10)
+    with pytest.raises(pkg.UnsupportedMemoryError):
+        client.send(conn, b"h", src.ctypes.data, 10, memory_type=1)      # ucx_memory_type::CUDA
+
+
+# ------------------------------------------------------------------ device cases
+
+@pytest.mark.gpu
+def test_c1_host_bundle_end_to_end(pkg, orc, gpu):
+    """BASELINE config 1: 64 fp32 host tensors -> one packed buffer + header ->
+    loopback AM -> unpack -> byte-for-byte."""
+    import torch
+    from execution_ucx_amd import workloads
+    srcs = workloads.host_bundle_c1(seed=0)
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    stream = torch.cuda.current_stream().cuda_stream
+    packed = pkg.pack_bundle(srcs, align=1, stream=stream)
+    req = client.send_bundle(conn, packed, stream=stream)
+    msg = server.recv_header()
+    assert msg.is_rndv and msg.data_length == 4 << 20 and msg.buffer_type == ROCM
+    assert msg.header == packed.header
+    recv = server.recv_buffer(msg, stream=stream)            # allocates from the pool
+    assert client.test(req)
+    host = np.zeros(4 << 20, np.uint8)
+    pkg.RocmMemoryResourceManager().memcpy(HOST, host.ctypes.data, ROCM, recv.data, host.size)
+    assert np.array_equal(host, orc.pack([s.view(np.uint8) for s in srcs], 1))
+    outs = [np.zeros_like(s) for s in srcs]
+    plan = pkg.unpack_bundle(msg.header, recv, out=outs, stream=stream)
+    torch.cuda.synchronize()
+    plan.close()
+    for a, b in zip(srcs, outs):
+        assert a.tobytes() == b.tobytes()
+    recv.release()
+    packed.payload.release()
+
+
+@pytest.mark.gpu
+def test_device_iov_equals_packed_bundle(pkg, orc, gpu):
+    """The reference's way (one iov entry per tensor, gathered by the transport)
+    and this build's way (one pack kernel, one contiguous send) deliver the same
+    bytes for the tight layout."""
+    import torch
+    rng = np.random.default_rng(3)
+    tensors = [torch.from_numpy(rng.integers(0, 256, size=int(n), dtype=np.uint8)).to(gpu)
+               for n in rng.integers(1, 300000, size=40)]
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    stream = torch.cuda.current_stream().cuda_stream
+    packed = pkg.pack_bundle(tensors, align=1, stream=stream)
+    r_iov = client.send_iov(conn, packed.header, [(t.data_ptr(), t.numel()) for t in tensors], ROCM,
+                            stream=stream, keep=tensors)
+    r_one = client.send_bundle(conn, packed, stream=stream)
+    m_iov, m_one = server.recv_header(), server.recv_header()
+    assert m_iov.data_length == m_one.data_length == packed.payload_bytes
+    b_iov = server.recv_buffer(m_iov, stream=stream)
+    b_one = server.recv_buffer(m_one, stream=stream)
+    assert client.test(r_iov) and client.test(r_one)
+    n = packed.payload_bytes
+    got_iov = torch.empty(n, dtype=torch.uint8, device=gpu)
+    got_one = torch.empty(n, dtype=torch.uint8, device=gpu)
+    mr = pkg.RocmMemoryResourceManager()
+    mr.memcpy(ROCM, got_iov.data_ptr(), ROCM, b_iov.data, n)
+    mr.memcpy(ROCM, got_one.data_ptr(), ROCM, b_one.data, n)
+    assert torch.equal(got_iov, got_one)
+    want = orc.pack([t.cpu().numpy() for t in tensors], 1)
+    assert np.array_equal(got_one.cpu().numpy(), want)
+    # zero-copy receive: views over the received buffer, typed from the header
+    outs = pkg.unpack_bundle(m_one.header, b_one, from_dlpack_fn=torch.from_dlpack)
+    for t, o in zip(tensors, outs):
+        assert torch.equal(t, o)
+
+
+@pytest.mark.gpu
+def test_device_eager_and_process_reply(pkg, gpu):
+    """Small device payload goes eager through host memory; the send -> process ->
+    reply round trip of ucx_am_context_test.cpp:1893-1944 with the halving kernel."""
+    import ctypes as C
+    import torch
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    c2s, s2c = client.connect(server), server.connect(client)
+    lib = pkg._capi.load()
+    for n in (32, 1 << 20):
+        x = torch.from_numpy((np.arange(n) % 256).astype(np.float32)).to(gpu)
+        torch.cuda.synchronize()
+        req = client.send(c2s, b"req", x.data_ptr(), 4 * n, ROCM, keep=x)
+        m = server.recv_header()
+        if 4 * n < 4096:
+            assert not m.is_rndv
+            y = torch.from_numpy(np.frombuffer(m.eager_data, dtype=np.float32).copy()).to(gpu)
+        else:
+            buf = server.recv_buffer(m)
+            y = torch.empty(n, dtype=torch.float32, device=gpu)
+            pkg.RocmMemoryResourceManager().memcpy(ROCM, y.data_ptr(), ROCM, buf.data, 4 * n)
+            buf.release()
+        assert client.test(req)
+        pkg._capi.check(lib.axr_divide_by_two(y.data_ptr(), n, None))
+        torch.cuda.synchronize()
+        rep = server.send(s2c, b"rep", y.data_ptr(), 4 * n, ROCM, keep=y)
+        r = client.recv_header()
+        if r.is_rndv:
+            z = torch.empty(n, dtype=torch.float32, device=gpu)
+            client.recv_into(r, z.data_ptr(), 4 * n, ROCM)
+            got = z.cpu().numpy()
+        else:
+            got = np.frombuffer(r.eager_data, dtype=np.float32)
+        assert server.test(rep)
+        assert np.array_equal(got, (np.arange(n) % 256).astype(np.float32) / 2)
