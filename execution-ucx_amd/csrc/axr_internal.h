@@ -73,7 +73,7 @@ struct LaunchConfig {
   uint32_t tiles_per_wave = 0;
   uint32_t tile_rows = 2;
   uint32_t threads = 256;   // per workgroup, a multiple of 64
-  bool nontemporal = true;
+  uint32_t nontemporal = 3;   // bit 0: tensor-side accesses, bit 1: payload-side accesses
   bool elements = false;   // some segment uses kModeElements
   bool xcd_remap = false;  // give each die a contiguous share of the wave index space
 };
@@ -90,7 +90,13 @@ struct Tunables {
   int64_t max_tiles = 1 << 17;
   int64_t max_waves = 1 << 20;    // beyond this many tiles a wave takes several
   int64_t threads = 256;          // workgroup size
-  int64_t nontemporal = 1;        // non-temporal loads/stores in the copy loops
+  // Non-temporal hint: bit 0 tensor-side accesses, bit 1 payload-side accesses;
+  // -1 = automatic: tensors always stream (read or written once), the payload
+  // streams only when it is larger than payload_cache_bytes.  A smaller payload
+  // is written with ordinary stores so that it is still in the 256 MB
+  // last-level cache when the consumer (unpack, or the transport's copy) reads it.
+  int64_t nontemporal = -1;
+  int64_t payload_cache_bytes = 256ll << 20;
   int64_t gather_run_bytes = 512; // strided runs shorter than this use element mode
   int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
 };

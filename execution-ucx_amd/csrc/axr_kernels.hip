@@ -65,13 +65,13 @@ __device__ __forceinline__ gbytes as_global(uint64_t address) {
 // Wave-cooperative copy of one tile.  src, dst and the length are
 // wave-uniform, lane_off is lane * 16.  A full tile is ROWS loads then ROWS
 // stores per lane.
-template <uint32_t ROWS, bool NT>
+template <uint32_t ROWS, bool NTL, bool NTS>
 __device__ __forceinline__ void wave_copy_full(gcbytes src, gbytes dst, uint32_t lane_off) {
   u32x4 v[ROWS];
 #pragma unroll
-  for (uint32_t k = 0; k < ROWS; ++k) v[k] = load16<NT>(src + lane_off + k * kRowBytes);
+  for (uint32_t k = 0; k < ROWS; ++k) v[k] = load16<NTL>(src + lane_off + k * kRowBytes);
 #pragma unroll
-  for (uint32_t k = 0; k < ROWS; ++k) store16<NT>(dst + lane_off + k * kRowBytes, v[k]);
+  for (uint32_t k = 0; k < ROWS; ++k) store16<NTS>(dst + lane_off + k * kRowBytes, v[k]);
 }
 
 // A partial tile (n < ROWS KiB) keeps the same shape: slot j (= lane + 64 k)
@@ -79,7 +79,7 @@ __device__ __forceinline__ void wave_copy_full(gcbytes src, gbytes dst, uint32_t
 // slot past the last whole vector moves the final 16 bytes [n - 16, n), which
 // overlap the previous slot with identical data.  No byte loops, no second
 // memory round trip; only ranges under 16 bytes are moved bytewise.
-template <uint32_t ROWS, bool NT>
+template <uint32_t ROWS, bool NTL, bool NTS>
 __device__ __forceinline__ void wave_copy_partial(gcbytes src, gbytes dst, uint32_t n,
                                                   uint32_t lane, uint32_t lane_off) {
   if (n < kVecBytes) {
@@ -93,7 +93,7 @@ __device__ __forceinline__ void wave_copy_partial(gcbytes src, gbytes dst, uint3
 #pragma unroll
   for (uint32_t k = 0; k < ROWS; ++k) {
     const uint32_t o = lane_off + k * kRowBytes;
-    v[k] = load16<NT>(src + (o < body ? o : last));   // unconditional: all loads in flight together
+    v[k] = load16<NTL>(src + (o < body ? o : last));   // unconditional: all loads in flight together
   }
   // Pin every loaded value here: it keeps the compiler from sinking a load into
   // the masked store that uses it (load -> wait -> store per slot), and it puts
@@ -104,19 +104,19 @@ __device__ __forceinline__ void wave_copy_partial(gcbytes src, gbytes dst, uint3
 #pragma unroll
   for (uint32_t k = 0; k < ROWS; ++k) {
     const uint32_t o = lane_off + k * kRowBytes;
-    if (o < limit) store16<NT>(dst + (o < body ? o : last), v[k]);
+    if (o < limit) store16<NTS>(dst + (o < body ? o : last), v[k]);
   }
 }
 
 // `left` bytes remain in the run from this tile's start; the tile takes at
 // most ROWS KiB of them.
-template <uint32_t ROWS, bool NT>
+template <uint32_t ROWS, bool NTL, bool NTS>
 __device__ __forceinline__ void wave_copy(gcbytes src, gbytes dst, uint64_t left, uint32_t lane,
                                           uint32_t lane_off) {
   if (left >= ROWS * kRowBytes) {
-    wave_copy_full<ROWS, NT>(src, dst, lane_off);
+    wave_copy_full<ROWS, NTL, NTS>(src, dst, lane_off);
   } else {
-    wave_copy_partial<ROWS, NT>(src, dst, static_cast<uint32_t>(left), lane, lane_off);
+    wave_copy_partial<ROWS, NTL, NTS>(src, dst, static_cast<uint32_t>(left), lane, lane_off);
   }
 }
 
@@ -214,8 +214,20 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   }
 }
 
-template <bool PACK, uint32_t ROWS, bool NT, bool ELEMENTS>
-__global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(KernelArgs a) {
+template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
+__global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
+    const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
+    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap) {
+  // Scalar arguments (not one struct) so that the compiler can preload them
+  // into SGPRs at dispatch instead of fetching the kernarg segment first.
+  KernelArgs a;
+  a.segs = segs_arg;
+  a.dims = dims_arg;
+  a.wave_seg = wave_seg_arg;
+  a.payload = payload_arg;
+  a.ntiles = ntiles;
+  a.tiles_per_wave = tiles_per_wave;
+  a.xcd_remap = xcd_remap;
   constexpr uint32_t kTile = ROWS * kRowBytes;
   const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
   const uint32_t lane_off = lane * kVecBytes;
@@ -262,10 +274,10 @@ __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(KernelA
       const uint64_t left = seg_run - boff;
       gbytes ten = as_global(seg_ptr) + boff;
       if constexpr (PACK) {
-        wave_copy<ROWS, NT>(ten, pay + boff, left, lane, lane_off);
+        wave_copy<ROWS, NTT, NTP>(ten, pay + boff, left, lane, lane_off);
         if (last && pad) wave_zero(pay + seg_run, pad, lane);
       } else {
-        wave_copy<ROWS, NT>(pay + boff, ten, left, lane, lane_off);
+        wave_copy<ROWS, NTP, NTT>(pay + boff, ten, left, lane, lane_off);
       }
     } else if (dsel == kSegFillOnly) {
       if constexpr (PACK) wave_zero(pay, pad, lane);
@@ -280,9 +292,9 @@ __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(KernelA
         gbytes ten = as_global(seg_ptr) + run_offset(dm, run) + boff;
         gbytes p = pay + static_cast<uint64_t>(run) * seg_run + boff;
         if constexpr (PACK) {
-          wave_copy<ROWS, NT>(ten, p, left, lane, lane_off);
+          wave_copy<ROWS, NTT, NTP>(ten, p, left, lane, lane_off);
         } else {
-          wave_copy<ROWS, NT>(p, ten, left, lane, lane_off);
+          wave_copy<ROWS, NTP, NTT>(p, ten, left, lane, lane_off);
         }
       } else if constexpr (ELEMENTS) {
         element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
@@ -350,14 +362,22 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
 template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap
+#define AXR_LAUNCH(NTT, NTP, EL) \
+  hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, 0, stream, AXR_ARGS)
   if (cfg.elements) {
     // strided tensors with short runs are present: the general kernel
-    hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, false, true>), grid, block, 0, stream, args);
-  } else if (cfg.nontemporal) {
-    hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, true, false>), grid, block, 0, stream, args);
+    AXR_LAUNCH(false, false, true);
   } else {
-    hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, false, false>), grid, block, 0, stream, args);
+    switch (cfg.nontemporal) {   // bit 0: tensor side, bit 1: payload side
+      case 0: AXR_LAUNCH(false, false, false); break;
+      case 1: AXR_LAUNCH(true, false, false); break;
+      case 2: AXR_LAUNCH(false, true, false); break;
+      default: AXR_LAUNCH(true, true, false); break;
+    }
   }
+#undef AXR_LAUNCH
+#undef AXR_ARGS
   return check_hip(hipGetLastError(), "bundle kernel launch");
 }
 

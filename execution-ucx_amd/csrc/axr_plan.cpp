@@ -419,7 +419,11 @@ int build_tables(axr_plan* p) {
   p->cfg.xcd_remap = tn.xcd_remap != 0 && p->cfg.workgroups >= 4 * kXcds;
   if (p->cfg.xcd_remap) p->cfg.workgroups = (p->cfg.workgroups + kXcds - 1) / kXcds * kXcds;
   p->cfg.tile_rows = rows;
-  p->cfg.nontemporal = tn.nontemporal != 0;
+  if (tn.nontemporal < 0) {
+    p->cfg.nontemporal = p->payload_bytes > static_cast<uint64_t>(tn.payload_cache_bytes) ? 3u : 1u;
+  } else {
+    p->cfg.nontemporal = static_cast<uint32_t>(tn.nontemporal) & 3u;
+  }
   p->cfg.elements = false;
   for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode == kModeElements;
 

@@ -293,7 +293,11 @@ int axr_tune_set(const char* key, int64_t value) {
     if (value < 1 || value > (1ll << 30)) return fail(AXR_ERR_INVALID, "max_waves must be in [1, 2^30]");
     t.max_waves = value;
   } else if (k == "nontemporal") {
-    t.nontemporal = value ? 1 : 0;
+    if (value < -1 || value > 3) return fail(AXR_ERR_INVALID, "nontemporal must be -1 (auto) or 0..3");
+    t.nontemporal = value;
+  } else if (k == "payload_cache_bytes") {
+    if (value < 0) return fail(AXR_ERR_INVALID, "payload_cache_bytes must not be negative");
+    t.payload_cache_bytes = value;
   } else if (k == "gather_run_bytes") {
     if (value < 1 || value > (1 << 20))
       return fail(AXR_ERR_INVALID, "gather_run_bytes must be in [1, 2^20]");
@@ -318,6 +322,7 @@ int axr_tune_get(const char* key, int64_t* value) {
   else if (k == "max_tiles") *value = t.max_tiles;
   else if (k == "max_waves") *value = t.max_waves;
   else if (k == "nontemporal") *value = t.nontemporal;
+  else if (k == "payload_cache_bytes") *value = t.payload_cache_bytes;
   else if (k == "gather_run_bytes") *value = t.gather_run_bytes;
   else if (k == "threads") *value = t.threads;
   else if (k == "xcd_remap") *value = t.xcd_remap;

@@ -308,7 +308,8 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
 
 /* Tuning knobs (process-wide, read when a plan builds its device tables):
  * "tile_rows" (KiB per wavefront tile: 0 auto, 1, 2, 4, 8, 16), "max_tiles",
- * "max_waves", "threads" (workgroup size), "nontemporal", "gather_run_bytes",
+ * "max_waves", "threads" (workgroup size), "nontemporal" (-1 auto, or bit 0
+ * tensor side / bit 1 payload side), "payload_cache_bytes", "gather_run_bytes",
  * "xcd_remap".  Unknown key -> AXR_ERR_INVALID. */
 AXR_API int axr_tune_set(const char* key, int64_t value);
 AXR_API int axr_tune_get(const char* key, int64_t* value);

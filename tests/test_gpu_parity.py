@@ -242,7 +242,7 @@ def test_every_kernel_instantiation(pkg, orc, gpu, rows, threads):
     tensors += [mat[::2, 16:2064], mat.t()[5:9]]           # run tiles and element mode
     chunks = [tbytes(t) for t in tensors]
     try:
-        for nt, max_waves in ((1, 1 << 20), (0, 1 << 20), (1, 7)):
+        for nt, max_waves in ((3, 1 << 20), (0, 1 << 20), (1, 7), (2, 1 << 20)):
             pkg.tune(tile_rows=rows, threads=threads, nontemporal=nt, max_waves=max_waves)
             for align in (1, 256):
                 got, plan, buf = run_pack(pkg, tensors, align, gpu)
@@ -255,7 +255,7 @@ def test_every_kernel_instantiation(pkg, orc, gpu, rows, threads):
                 for o, c in zip(outs, chunks):
                     assert np.array_equal(tbytes(o), c), (nt, max_waves, align)
     finally:
-        pkg.tune(tile_rows=0, threads=256, nontemporal=1, max_waves=1 << 20)
+        pkg.tune(tile_rows=0, threads=256, nontemporal=-1, max_waves=1 << 20)
 
 
 # ------------------------------------------------------------------ strided views
