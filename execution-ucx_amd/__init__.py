@@ -14,6 +14,7 @@ from .device import (CpuDevice, Device, DeviceType, RocmDevice, auto_detect, cpu
 from .dlpack import DLPackExport, TensorView, extract, extract_many
 from .loopback import AmMessage, LoopbackAmContext
 from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager
+from .pipeline import StreamedTransfer
 
 __version__ = "0.1.0"
 

@@ -250,6 +250,7 @@ PROTOTYPES = {
     "axr_am_request_test": (C.c_int, [_vp, C.c_uint64, _intp]),
     "axr_am_recv_header": (C.c_int, [_vp, C.POINTER(AmMessage)]),
     "axr_am_recv_buffer": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
+    "axr_am_recv_buffer_async": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
     "axr_am_recv_buffer_iov": (C.c_int, [_vp, C.c_uint64, C.c_int, C.POINTER(Buffer), _sz, _vp]),
     "axr_am_message_release": (C.c_int, [_vp, C.c_uint64]),
     "axr_am_pending": (C.c_int, [_vp, C.POINTER(_sz)]),

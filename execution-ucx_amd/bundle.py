@@ -60,8 +60,11 @@ class BundlePlan:
         """Sender side: ``tensors`` are DLPack producers (or TensorViews), laid
         out in argument order.  ``align=1`` is the reference's tight layout."""
         lib = _capi.load()
-        views = extract_many(tensors)
-        arr = TensorArray(views)
+        if isinstance(tensors, TensorArray):      # descriptors prepared once, reused per call
+            arr, views = tensors, tensors.views
+        else:
+            views = extract_many(tensors)
+            arr = TensorArray(views)
         h = C.c_void_p()
         _capi.check(lib.axr_plan_create(arr.pointer(), arr.count, align, 0, C.byref(h)))
         return cls(h.value, keepalive=views)
@@ -75,8 +78,11 @@ class BundlePlan:
         return cls(h.value)
 
     def bind(self, tensors: Sequence[Any]) -> "BundlePlan":
-        views = extract_many(tensors)
-        arr = TensorArray(views)
+        if isinstance(tensors, TensorArray):
+            arr, views = tensors, tensors.views
+        else:
+            views = extract_many(tensors)
+            arr = TensorArray(views)
         _capi.check(self._lib.axr_plan_bind(self._h, arr.pointer(), arr.count))
         self._keep = views
         return self

@@ -60,12 +60,13 @@ static_assert(sizeof(Dims) == 96, "Dims layout");
 struct KernelArgs {
   const Seg* segs;            // nseg + 1 entries, last is a sentinel with tile_begin == ntiles
   const Dims* dims;
-  const uint32_t* wave_seg;   // first segment of each wavefront's tile range
+  const uint32_t* wave_seg;   // segment holding tile (k << seg_shift), for every k
   uint8_t* payload;
   uint32_t nseg;
   uint32_t ntiles;
   uint32_t tiles_per_wave;
   uint32_t xcd_remap;         // 0 or the number of workgroups per die
+  uint32_t seg_shift;         // log2 of the tile-block size of wave_seg
 };
 
 struct LaunchConfig {
@@ -73,6 +74,7 @@ struct LaunchConfig {
   uint32_t tiles_per_wave = 0;
   uint32_t tile_rows = 2;
   uint32_t threads = 256;   // per workgroup, a multiple of 64
+  uint32_t seg_shift = 0;   // wave_seg has one entry per 2^seg_shift tiles
   uint32_t nontemporal = 3;   // bit 0: tensor-side accesses, bit 1: payload-side accesses
   bool elements = false;   // some segment uses kModeElements
   bool xcd_remap = false;  // give each die a contiguous share of the wave index space

@@ -217,7 +217,7 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
 template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
     const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
-    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap) {
+    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift) {
   // Scalar arguments (not one struct) so that the compiler can preload them
   // into SGPRs at dispatch instead of fetching the kernarg segment first.
   KernelArgs a;
@@ -228,6 +228,7 @@ __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
   a.ntiles = ntiles;
   a.tiles_per_wave = tiles_per_wave;
   a.xcd_remap = xcd_remap;
+  a.seg_shift = seg_shift;
   constexpr uint32_t kTile = ROWS * kRowBytes;
   const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
   const uint32_t lane_off = lane * kVecBytes;
@@ -247,7 +248,10 @@ __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
   const AXR_CONST uint32_t* wave_seg =
       reinterpret_cast<const AXR_CONST uint32_t*>(reinterpret_cast<uintptr_t>(a.wave_seg));
   gbytes payload = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(a.payload));
-  uint32_t s = wave_seg[wave];
+  // The index has one entry per block of 2^seg_shift tiles (the planner sizes
+  // blocks so that they rarely hold more than one segment); the loop below
+  // walks forward from there to the segment of this wave's first tile.
+  uint32_t s = wave_seg[t >> a.seg_shift];
   uint64_t seg_ptr = segs[s].ptr, seg_off = segs[s].off, seg_run = segs[s].run_bytes;
   uint32_t seg_begin = segs[s].tile_begin, seg_meta = segs[s].meta;
   uint32_t seg_end = segs[s + 1].tile_begin;
@@ -362,7 +366,7 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
 template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
-#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift
 #define AXR_LAUNCH(NTT, NTP, EL) \
   hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, 0, stream, AXR_ARGS)
   if (cfg.elements) {

@@ -24,7 +24,12 @@ struct Piece {
 };
 
 struct Request {
-  std::atomic<int> done{0};
+  std::atomic<int> done{0};        // 1 complete, -1 cancelled or failed
+  hipEvent_t event = nullptr;      // set by an asynchronous fetch: done once it has fired
+  std::mutex mu;
+  ~Request() {
+    if (event) (void)hipEventDestroy(event);
+  }
 };
 
 struct Message {
@@ -190,7 +195,16 @@ int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->requests.find(request);
   if (it == ctx->requests.end()) return fail(AXR_ERR_INVALID, "axr_am_request_test: unknown request");
-  const int st = it->second->done.load();
+  int st = it->second->done.load();
+  if (st == 0) {
+    std::lock_guard<std::mutex> rl(it->second->mu);
+    if (it->second->event) {
+      const hipError_t q = hipEventQuery(it->second->event);
+      if (q == hipSuccess) st = 1;
+      else if (q != hipErrorNotReady) st = -1;
+      if (st != 0) it->second->done.store(st);
+    }
+  }
   *done = st;
   if (st != 0) ctx->requests.erase(it);
   return AXR_OK;
@@ -216,7 +230,7 @@ int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* out) {
 }
 
 static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_buffer_t* vec,
-                 size_t count, void* stream) {
+                 size_t count, void* stream, bool wait = true) {
   if (!known_type(dst_type)) return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
   std::unique_ptr<Message> m;
   {
@@ -253,6 +267,14 @@ static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_bu
     }
     if (rc) break;
   }
+  if (rc == AXR_OK && device_copy && !wait) {
+    // completion of the send = completion of the copies just enqueued
+    std::lock_guard<std::mutex> lock(m->request->mu);
+    rc = check_hip(hipEventCreateWithFlags(&m->request->event, hipEventDisableTiming), "hipEventCreate");
+    if (rc == AXR_OK) rc = check_hip(hipEventRecord(m->request->event, s), "hipEventRecord");
+    if (rc != AXR_OK) m->request->done.store(-1);
+    return rc;
+  }
   if (rc == AXR_OK && device_copy) rc = check_hip(hipStreamSynchronize(s), "hipStreamSynchronize");
   m->request->done.store(rc == AXR_OK ? 1 : -1);
   return rc;
@@ -264,6 +286,14 @@ int axr_am_recv_buffer(axr_am_context_t* ctx, uint64_t key, int dst_type, void* 
   if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null buffer");
   axr_buffer_t one{dst, dst_bytes};
   return fetch(ctx, key, dst_type, &one, 1, stream);
+}
+
+int axr_am_recv_buffer_async(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
+                             size_t dst_bytes, void* stream) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_async: null context");
+  if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_async: null buffer");
+  axr_buffer_t one{dst, dst_bytes};
+  return fetch(ctx, key, dst_type, &one, 1, stream, /*wait=*/false);
 }
 
 int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,

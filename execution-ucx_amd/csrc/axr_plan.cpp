@@ -427,15 +427,22 @@ int build_tables(axr_plan* p) {
   p->cfg.elements = false;
   for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode == kModeElements;
 
-  const size_t nwaves = static_cast<size_t>(p->cfg.workgroups) * waves_per_wg;
-  p->wave_seg.assign(nwaves, 0);
-  size_t s = 0;
+  // Tile-block index: entry k = segment that holds tile k << seg_shift.  Blocks
+  // are sized to about one segment each (a power of two, at most 256 tiles), so
+  // a bundle of few large tensors gets a tiny index and a bundle of many small
+  // ones one entry per few tiles; a wave walks at most a segment or two forward.
   const size_t nseg = p->segs.size() - 1;
-  for (size_t w = 0; w < nwaves; ++w) {
-    const uint64_t t0 = static_cast<uint64_t>(w) * tpw;
+  uint32_t shift = 0;
+  while (shift < 8 && (static_cast<uint64_t>(nseg) << (shift + 1)) <= p->ntiles) ++shift;
+  p->cfg.seg_shift = shift;
+  const size_t nblocks = (static_cast<size_t>(p->ntiles) >> shift) + 1;
+  p->wave_seg.assign(nblocks, 0);
+  size_t s = 0;
+  for (size_t k = 0; k < nblocks; ++k) {
+    const uint64_t t0 = static_cast<uint64_t>(k) << shift;
     if (t0 >= p->ntiles) break;
     while (s + 1 < nseg && p->segs[s + 1].tile_begin <= t0) ++s;
-    p->wave_seg[w] = static_cast<uint32_t>(s);
+    p->wave_seg[k] = static_cast<uint32_t>(s);
   }
 
   p->dims_at = align_up(p->segs.size() * sizeof(Seg), 16);
@@ -516,6 +523,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   a.ntiles = p->ntiles;
   a.tiles_per_wave = p->cfg.tiles_per_wave;
   a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
+  a.seg_shift = p->cfg.seg_shift;
   rc = launch_bundle_kernel(pack, a, p->cfg, stream);
   if (rc) return rc;
   if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())

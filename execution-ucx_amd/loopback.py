@@ -130,9 +130,11 @@ class LoopbackAmContext:
         return dst
 
     def recv_into(self, message: AmMessage, ptr: int, nbytes: int, memory_type: int = ROCM,
-                  stream=None) -> None:
-        _capi.check(self._lib.axr_am_recv_buffer(self._h, message.key, memory_type, ptr, nbytes,
-                                                 _stream_handle(stream)))
+                  stream=None, wait: bool = True) -> None:
+        """Fetch into caller memory.  ``wait=False`` only enqueues the copies on
+        ``stream`` (work ordered after them on that stream sees the data)."""
+        fn = self._lib.axr_am_recv_buffer if wait else self._lib.axr_am_recv_buffer_async
+        _capi.check(fn(self._h, message.key, memory_type, ptr, nbytes, _stream_handle(stream)))
 
     def recv_buffer_iov(self, message: AmMessage, buffers: Sequence[Tuple[int, int]],
                         memory_type: int = ROCM, stream=None) -> None:

@@ -384,6 +384,11 @@ AXR_API int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* message)
  * dst_bytes below data_length -> AXR_ERR_LENGTH. */
 AXR_API int axr_am_recv_buffer(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
                                size_t dst_bytes, void* stream);
+/* Same, but only enqueues the copies on `stream`: the data is in place for work
+ * ordered after them on that stream, and the sender's request completes when
+ * they have run (for pipelines that must not block the host). */
+AXR_API int axr_am_recv_buffer_async(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
+                                     size_t dst_bytes, void* stream);
 /* Same into an iov: entries must be non-null and non-empty and add up to at
  * least data_length (ucx_am_context.hpp:1808-1818); filled in order. */
 AXR_API int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,

@@ -434,6 +434,32 @@ def test_c5_pitched_chunk(pkg, orc, gpu):
         assert int(twin[:, :, spec.cols:].view(torch.int16).ne(0).sum()) == 0     # pitch gap untouched
 
 
+def test_c5_streamed_pipeline(pkg, gpu):
+    """Double-buffered pack -> loopback send -> unpack over two streams: small
+    chunks (eager and rendezvous sizes) and four full 256 MiB chunks."""
+    import torch
+    from execution_ucx_amd import workloads
+    for spec, chunks in ((workloads.pitched_chunk(views=3, rows=4, cols=64), 7),
+                         (workloads.pitched_chunk(views=5, rows=64, cols=256), 9),
+                         (workloads.pitched_chunk(), 4)):
+        src = torch.empty(chunks, spec.views, spec.rows, spec.pitch, dtype=torch.bfloat16, device=gpu)
+        src.view(torch.int16).random_(-32768, 32767)
+        dst = torch.zeros_like(src)
+        torch.cuda.synchronize()
+        slot = (spec.view_bytes + 255) // 256 * 256 * spec.views
+        st = pkg.StreamedTransfer(slot_bytes=slot)
+        per_chunk = spec.views * spec.parent_elems * 2
+        for k in range(chunks):
+            st.submit(workloads.pitched_views(src.data_ptr() + k * per_chunk, spec),
+                      workloads.pitched_views(dst.data_ptr() + k * per_chunk, spec))
+        st.finish()
+        s16, d16 = src.view(torch.int16), dst.view(torch.int16)
+        assert torch.equal(d16[..., :spec.cols], s16[..., :spec.cols])
+        assert int(d16[..., spec.cols:].ne(0).sum()) == 0
+        st.close()
+        assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+
+
 # ------------------------------------------------------------------ checksums, compare
 
 def test_checksum_of_checksums(pkg, orc, gpu):
