@@ -2,7 +2,7 @@
 """Benchmark of the tensor-bundle pack+unpack path on one MI355X.
 
 A step is one pack plus one unpack of the 4,096-tensor mixed bundle
-(BASELINE.json configs[1]); inputs are resident in HBM before the timed region.
+(4096 1-D tensors of 256 B-64 KiB in five dtypes); inputs are resident in HBM before the timed region.
 `value` = 4 * P / t  (P = sum of tensor bytes; pack reads P and writes P, unpack
 reads P and writes P), in GB/s, timed with HIP events on the stream the kernels
 are launched on.  By default the steps rotate over several independent copies of
@@ -274,6 +274,32 @@ def stream_c5(h, chunks=32):
             "overlap_speedup": round(out[1] / out[2], 3)}
 
 
+def host_bundle_c1(h, reps=30):
+    """64 fp32 host tensors (4 MiB) -> device payload -> host tensors: every byte
+    crosses PCIe twice, so this is a transfer figure, not an HBM one."""
+    import numpy as np
+    from execution_ucx_amd import workloads
+    srcs = workloads.host_bundle_c1(seed=0)
+    outs = [np.zeros_like(s) for s in srcs]
+    plan = h.pkg.BundlePlan.create(srcs, align=1)
+    nbytes = plan.payload_bytes
+    payload = h.torch.empty(nbytes, dtype=h.torch.uint8, device="cuda")
+    rplan = h.pkg.BundlePlan.from_header(plan.header).bind(outs)
+    times = []
+    for _ in range(reps + 3):
+        h.sync()
+        t0 = time.perf_counter()
+        plan.pack(payload.data_ptr(), nbytes, h.stream)
+        rplan.unpack(payload.data_ptr(), nbytes, h.stream)
+        h.capi.check(h.lib.axr_stream_synchronize(h.stream))
+        times.append(time.perf_counter() - t0)
+    if any(a.tobytes() != b.tobytes() for a, b in zip(srcs, outs)):
+        raise SystemExit("bench.py: host bundle round trip differs")
+    t = sorted(times[3:])[reps // 2]
+    return {"payload_bytes_P": nbytes, "round_trip_us": round(t * 1e6, 1),
+            "GBps_pcie_inclusive_4P": round(4.0 * nbytes / t / 1e9, 2)}
+
+
 def cpu_baseline(spec, seed=0):
     """Reference host path on this box's cores: memcpy concat + split of the same bundle."""
     import numpy as np
@@ -409,6 +435,7 @@ def main():
                                       "payload_bytes_P": c5[0].data_bytes, "steps": k5}
         del c5
         torch.cuda.empty_cache()
+        extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["c5_streamed_8GiB"] = stream_c5(h)
         torch.cuda.empty_cache()
         c4 = make_c4_set(h)

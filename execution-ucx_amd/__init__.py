@@ -15,6 +15,7 @@ from .dlpack import DLPackExport, TensorView, extract, extract_many
 from .loopback import AmMessage, LoopbackAmContext
 from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager
 from .pipeline import StreamedTransfer
+from .transfer import recv_tensors, send_tensors
 
 __version__ = "0.1.0"
 

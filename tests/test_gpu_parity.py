@@ -509,6 +509,27 @@ def test_dlpack_rocm_capsules_and_zero_copy_receive(pkg, gpu):
     assert [o.data_ptr() - base for o in outs] == packed.plan.layout()[0]   # views, not copies
 
 
+def test_pinned_host_destination(pkg, orc, gpu):
+    """Scatter a device payload straight into pinned host tensors (the staging a
+    checkpoint writer needs) and gather from them: the kernel addresses pinned
+    memory like device memory."""
+    import torch
+    rng = np.random.default_rng(8)
+    srcs = [rand_bytes_tensor(rng, n, gpu) for n in (70000, 33, 4096, 123457)]
+    got, plan, buf = run_pack(pkg, srcs, 256, gpu)
+    pinned = [torch.zeros(t.numel(), dtype=torch.uint8).pin_memory() for t in srcs]
+    views = [pkg.TensorView(data=p.data_ptr(), device_type=11, device_id=0, dtype=(1, 8, 1),
+                            shape=(p.numel(),), strides=None, owner=p) for p in pinned]
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(views)
+    assert rplan.launch_info()["host_copies"] == 0           # no staged copies: one kernel
+    rplan.unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    for p, t in zip(pinned, srcs):
+        assert np.array_equal(p.numpy(), t.cpu().numpy())
+    got2, plan2, _ = run_pack(pkg, views, 256, gpu)          # and back: pinned sources
+    assert np.array_equal(got2, got)
+
+
 # ------------------------------------------------------------------ plan reuse, streams, errors
 
 def test_plan_reuse_rebind_and_streams(pkg, orc, gpu):

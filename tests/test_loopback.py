@@ -127,7 +127,7 @@ def test_unsupported_memory_type(pkg, pair):
 
 @pytest.mark.gpu
 def test_c1_host_bundle_end_to_end(pkg, orc, gpu):
-    """BASELINE config 1: 64 fp32 host tensors -> one packed buffer + header ->
+    """The host-memory bundle: 64 fp32 host tensors -> one packed buffer + header ->
     loopback AM -> unpack -> byte-for-byte."""
     import torch
     from execution_ucx_amd import workloads
@@ -226,3 +226,43 @@ def test_device_eager_and_process_reply(pkg, gpu):
             got = np.frombuffer(r.eager_data, dtype=np.float32)
         assert server.test(rep)
         assert np.array_equal(got, (np.arange(n) % 256).astype(np.float32) / 2)
+
+
+@pytest.mark.gpu
+def test_send_recv_tensors_with_memory_policy(pkg, gpu):
+    """Receive side of the memory-policy contract: the policy sees the metas, its
+    own tensors come back filled; without a policy the result is zero-copy views;
+    a tiny bundle goes the eager way through host memory."""
+    import torch
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    stream = torch.cuda.current_stream().cuda_stream
+    big = [torch.randn(5000, device=gpu), torch.randn(33, 77, device=gpu).to(torch.bfloat16),
+           torch.arange(1000, device=gpu, dtype=torch.int32)]
+    tiny = [torch.arange(10, device=gpu, dtype=torch.int32), torch.ones(3, device=gpu)]
+    for tensors, rndv in ((big, True), (tiny, False)):
+        seen = {}
+
+        def policy(metas):
+            seen["metas"] = metas
+            seen["outs"] = [torch.zeros(m.shape, dtype=t.dtype, device=gpu) for m, t in zip(metas, tensors)]
+            return seen["outs"]
+
+        req, bundle = pkg.send_tensors(client, conn, tensors, stream=stream)
+        assert server.pending() == 1
+        got = pkg.recv_tensors(server, memory_policy=policy, stream=stream)
+        assert client.test(req)
+        assert [m.shape for m in seen["metas"]] == [tuple(t.shape) for t in tensors]
+        assert all(g is o for g, o in zip(got, seen["outs"]))         # the policy's own objects
+        for a, b in zip(tensors, got):
+            assert torch.equal(a, b)
+        req, bundle2 = pkg.send_tensors(client, conn, tensors, stream=stream)
+        views = pkg.recv_tensors(server, from_dlpack_fn=torch.from_dlpack, stream=stream)
+        assert client.test(req)
+        for a, b in zip(tensors, views):
+            assert torch.equal(a, b) and b.device.type == "cuda"
+        with pytest.raises(RuntimeError):
+            pkg.send_tensors(client, conn, tensors, stream=stream)
+            pkg.recv_tensors(server, memory_policy=lambda metas: [torch.zeros(1, device=gpu)], stream=stream)
+        assert (bundle.payload_bytes >= 4096) == rndv
+    assert pkg.recv_tensors(server) is None
