@@ -73,7 +73,7 @@ struct LaunchConfig {
   uint32_t workgroups = 0;
   uint32_t tiles_per_wave = 0;
   uint32_t tile_rows = 2;
-  uint32_t threads = 256;   // per workgroup, a multiple of 64
+  uint32_t threads = 128;   // per workgroup, a multiple of 64
   uint32_t seg_shift = 0;   // wave_seg has one entry per 2^seg_shift tiles
   uint32_t nontemporal = 3;   // bit 0: tensor-side accesses, bit 1: payload-side accesses
   bool elements = false;   // some segment uses kModeElements
@@ -84,14 +84,15 @@ struct LaunchConfig {
 
 struct Tunables {
   // Tile = tile_rows KiB moved by one wavefront.  0 picks the smallest of
-  // 2, 4, 8, 16 that keeps the bundle within max_tiles tiles: small tiles and a
-  // grid of one tile per wave measured fastest on MI355X (the hardware
-  // dispatcher balances the load), larger tiles bound the per-wave index table
-  // and the host time to fill it for multi-GiB bundles.
+  // 2, 4, 8, 16 that keeps the bundle within max_tiles tiles (and one tile per
+  // run for bundles of short strided runs): small tiles and a grid of one tile
+  // per wave measured fastest on MI355X (the hardware dispatcher balances the
+  // load); larger tiles only bound the grid for multi-GiB bundles.
   int64_t tile_rows = 0;
-  int64_t max_tiles = 1 << 17;
+  int64_t max_tiles = 1 << 20;
   int64_t max_waves = 1 << 20;    // beyond this many tiles a wave takes several
-  int64_t threads = 256;          // workgroup size
+  int64_t threads = 0;            // workgroup size; 0 = 256 below 65,536 tiles (fewer dispatches
+                                  // for short kernels), 128 above (finer balance at the tail)
   // Non-temporal hint: bit 0 tensor-side accesses, bit 1 payload-side accesses;
   // -1 = automatic: tensors always stream (read or written once), the payload
   // streams only when it is larger than payload_cache_bytes.  A smaller payload

@@ -148,6 +148,8 @@ typedef const AXR_CONST Dims* dims_table;
 __device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
   int64_t off = 0;
   const uint32_t nd = dm->ndim;
+  if (nd == 1)   // one strided dimension (pitched rows, cache blocks): no division
+    return static_cast<int64_t>(run) * dm->stride[kMaxOuterDims - 1];
 #pragma unroll
   for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
     if (static_cast<uint32_t>(d) + nd >= kMaxOuterDims) {
@@ -289,7 +291,8 @@ __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
       dims_table dm = dims + (dsel - 1);
       if (dm->mode == kModeRunTiles) {
         const uint32_t tpr = dm->tiles_per_run;
-        const uint32_t run = q / tpr;
+        const uint32_t tpr_log2 = dm->granule;   // run-tile mode: 1 + log2(tpr) when a power of two
+        const uint32_t run = tpr_log2 ? q >> (tpr_log2 - 1) : q / tpr;
         const uint32_t piece = q - run * tpr;
         const uint64_t boff = static_cast<uint64_t>(piece) * kTile;
         const uint64_t left = seg_run - boff;

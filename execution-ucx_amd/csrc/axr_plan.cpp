@@ -316,6 +316,9 @@ struct Builder {
       if (tpr > 0xffffffffull || runs > 0xffffffffull)
         return fail(AXR_ERR_UNSUPPORTED, "strided tensor has too many runs");
       dm.tiles_per_run = static_cast<uint32_t>(tpr);
+      // granule is unused in this mode: it carries 1 + log2(tiles per run) when
+      // that is a power of two, so the kernel can shift instead of divide
+      dm.granule = (tpr & (tpr - 1)) == 0 ? 1u + static_cast<uint32_t>(__builtin_ctzll(tpr)) : 0u;
       ntile = runs * tpr;
     } else {
       dm.mode = kModeElements;
@@ -359,6 +362,23 @@ int build_tables(axr_plan* p) {
   uint32_t rows = static_cast<uint32_t>(tn.tile_rows);
   if (rows == 0) {
     rows = 2;
+    // A bundle made only of strided views with one short run length (pitched
+    // rows, small cache blocks) gets one tile per run: fewer waves, no split runs.
+    uint64_t common_run = 0;
+    bool uniform_runs = !p->tensors.empty();
+    for (const TensorRec& t : p->tensors) {
+      if (t.nbytes == 0) continue;
+      const uint64_t item = (static_cast<uint64_t>(t.bits) + 7) / 8;
+      const Collapsed c = collapse(t, p->shape_of(t), p->strides_of(t), item);
+      if (c.extent.empty() || (common_run && c.run_bytes != common_run)) {
+        uniform_runs = false;
+        break;
+      }
+      common_run = c.run_bytes;
+    }
+    if (uniform_runs && common_run >= 2 * kRowBytes && common_run <= kMaxTileRows * kRowBytes) {
+      while (rows < kMaxTileRows && rows * kRowBytes < common_run) rows *= 2;
+    }
     while (rows < kMaxTileRows &&
            p->payload_bytes / (static_cast<uint64_t>(rows) * kRowBytes) >
                static_cast<uint64_t>(tn.max_tiles))
@@ -411,7 +431,7 @@ int build_tables(axr_plan* p) {
   uint64_t tpw = (p->ntiles + static_cast<uint64_t>(tn.max_waves) - 1) /
                  static_cast<uint64_t>(tn.max_waves);
   if (tpw == 0) tpw = 1;
-  p->cfg.threads = static_cast<uint32_t>(tn.threads);
+  p->cfg.threads = tn.threads ? static_cast<uint32_t>(tn.threads) : (p->ntiles < 65536 ? 256u : 128u);
   const uint32_t waves_per_wg = p->cfg.threads / kWaveLanes;
   const uint64_t per_wg = tpw * waves_per_wg;
   p->cfg.tiles_per_wave = static_cast<uint32_t>(tpw);

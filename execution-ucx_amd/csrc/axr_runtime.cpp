@@ -303,8 +303,8 @@ int axr_tune_set(const char* key, int64_t value) {
       return fail(AXR_ERR_INVALID, "gather_run_bytes must be in [1, 2^20]");
     t.gather_run_bytes = value;
   } else if (k == "threads") {
-    if (value < 64 || value > 1024 || value % 64)
-      return fail(AXR_ERR_INVALID, "threads must be a multiple of 64 in [64, 1024]");
+    if (value != 0 && (value < 64 || value > 1024 || value % 64))
+      return fail(AXR_ERR_INVALID, "threads must be 0 (auto) or a multiple of 64 in [64, 1024]");
     t.threads = value;
   } else if (k == "xcd_remap") {
     t.xcd_remap = value ? 1 : 0;

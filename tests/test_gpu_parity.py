@@ -255,7 +255,7 @@ def test_every_kernel_instantiation(pkg, orc, gpu, rows, threads):
                 for o, c in zip(outs, chunks):
                     assert np.array_equal(tbytes(o), c), (nt, max_waves, align)
     finally:
-        pkg.tune(tile_rows=0, threads=256, nontemporal=-1, max_waves=1 << 20)
+        pkg.tune(tile_rows=0, threads=0, nontemporal=-1, max_waves=1 << 20)
 
 
 # ------------------------------------------------------------------ strided views

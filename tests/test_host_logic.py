@@ -223,10 +223,12 @@ def test_pitched_view_rows(pkg):
     from execution_ucx_amd import workloads
     spec = workloads.pitched_chunk()
     v = workloads.pitched_views(0x7f00_0000_0000, spec)[1]
-    segs, _ = seg_of(pkg, v)
+    segs, info = seg_of(pkg, v)
     s = segs[0]
     assert (s["mode"], s["run_bytes"], s["shape"], s["stride_bytes"]) == (1, 4096, (1024,), (6144,))
-    assert s["tiles"] == 1024 * 2
+    assert s["tiles"] == 1024 and info["tile_bytes"] == 4096       # one tile per 4 KiB row
+    segs, info = seg_of(pkg, v, tile_rows=2)
+    assert segs[0]["tiles"] == 2048 and info["tile_bytes"] == 2048
 
 
 def test_short_runs_use_element_mode(pkg):
