@@ -53,13 +53,6 @@ struct HostCopy {
 };
 
 template <typename T>
-void put(std::vector<uint8_t>& v, T x) {
-  uint8_t b[sizeof(T)];
-  std::memcpy(b, &x, sizeof(T));   // build targets are little-endian (x86-64, gfx950)
-  v.insert(v.end(), b, b + sizeof(T));
-}
-
-template <typename T>
 T get(const uint8_t* p) {
   T x;
   std::memcpy(&x, p, sizeof(T));
@@ -146,26 +139,35 @@ void compute_layout(axr_plan* p) {
 }
 
 void encode_header(axr_plan* p) {
+  size_t total = kFixedHeader;
+  for (const auto& t : p->tensors) total += kTensorHeader + 8 * static_cast<size_t>(t.ndim);
   std::vector<uint8_t>& h = p->header;
-  h.clear();
-  put<uint32_t>(h, kMagic);
-  put<uint16_t>(h, kVersion);
-  put<uint16_t>(h, 0);
-  put<uint32_t>(h, static_cast<uint32_t>(p->tensors.size()));
-  put<uint32_t>(h, p->align);
-  put<uint64_t>(h, p->payload_bytes);
+  h.resize(total);
+  uint8_t* w = h.data();
+  auto emit = [&w](const void* src, size_t n) {   // targets are little-endian (x86-64, gfx950)
+    std::memcpy(w, src, n);
+    w += n;
+  };
+  const uint32_t magic = kMagic, n = static_cast<uint32_t>(p->tensors.size()), align = p->align;
+  const uint16_t version = kVersion, flags = 0;
+  emit(&magic, 4);
+  emit(&version, 2);
+  emit(&flags, 2);
+  emit(&n, 4);
+  emit(&align, 4);
+  emit(&p->payload_bytes, 8);
+  const uint64_t zero = 0;   // byte_offset: the packed copy starts at its offset
   for (const auto& t : p->tensors) {
-    put<uint64_t>(h, t.offset);
-    put<uint64_t>(h, t.nbytes);
-    put<int32_t>(h, t.device_type);
-    put<int32_t>(h, t.device_id);
-    put<int32_t>(h, t.ndim);
-    put<uint8_t>(h, t.code);
-    put<uint8_t>(h, t.bits);
-    put<uint16_t>(h, t.lanes);
-    put<uint64_t>(h, 0);   // byte_offset: the packed copy starts at its offset
-    const int64_t* shape = p->shape_of(t);
-    for (int32_t d = 0; d < t.ndim; ++d) put<int64_t>(h, shape[d]);
+    emit(&t.offset, 8);
+    emit(&t.nbytes, 8);
+    emit(&t.device_type, 4);
+    emit(&t.device_id, 4);
+    emit(&t.ndim, 4);
+    emit(&t.code, 1);
+    emit(&t.bits, 1);
+    emit(&t.lanes, 2);
+    emit(&zero, 8);
+    if (t.ndim) emit(p->shape_of(t), 8 * static_cast<size_t>(t.ndim));
   }
 }
 
@@ -205,55 +207,52 @@ void quiesce(axr_plan* p) {
 
 // ------------------------------------------------------------ table building
 
+// Outer (strided) dimensions and the contiguous inner run of one tensor, in
+// fixed storage: planning a bundle of thousands of tensors must not allocate
+// per tensor.
 struct Collapsed {
-  std::vector<uint64_t> extent;   // outer dims, outermost first
-  std::vector<int64_t> stride;    // bytes
+  uint64_t extent[kMaxNdim];   // outer dims, outermost first
+  int64_t stride[kMaxNdim];    // bytes
+  size_t nd = 0;
   uint64_t run_bytes = 0;
 };
 
 // Reduce (shape, element strides) to the fewest strided outer dimensions plus
 // one contiguous inner run.  Extent-1 dims vanish; adjacent dims that together
 // address a regular span merge.
-Collapsed collapse(const TensorRec& t, const int64_t* shape, const int64_t* strides,
-                   uint64_t item) {
-  Collapsed c;
-  std::vector<uint64_t> ext;
-  std::vector<int64_t> str;
-  int64_t dense = static_cast<int64_t>(item);
-  std::vector<int64_t> row_major(t.ndim);
+void collapse(const TensorRec& t, const int64_t* shape, const int64_t* strides, uint64_t item,
+              Collapsed* c) {
+  c->nd = 0;
+  // merged dims, innermost first
+  uint64_t me[kMaxNdim];
+  int64_t ms[kMaxNdim];
+  size_t nm = 0;
+  int64_t dense = static_cast<int64_t>(item);   // row-major stride of the current dim
   for (int32_t d = t.ndim - 1; d >= 0; --d) {
-    row_major[d] = dense;
+    const int64_t row_major = dense;
     dense *= shape[d];
-  }
-  for (int32_t d = 0; d < t.ndim; ++d) {
     if (shape[d] == 1) continue;
-    ext.push_back(static_cast<uint64_t>(shape[d]));
-    str.push_back(strides ? strides[d] * static_cast<int64_t>(item) : row_major[d]);
-  }
-  // merge from the inside out
-  std::vector<uint64_t> me;
-  std::vector<int64_t> ms;
-  for (size_t i = ext.size(); i-- > 0;) {
-    if (!me.empty() && str[i] == ms.back() * static_cast<int64_t>(me.back())) {
-      me.back() *= ext[i];   // outer dim continues the inner one
+    const int64_t st = strides ? strides[d] * static_cast<int64_t>(item) : row_major;
+    if (nm && st == ms[nm - 1] * static_cast<int64_t>(me[nm - 1])) {
+      me[nm - 1] *= static_cast<uint64_t>(shape[d]);   // this dim continues the inner one
     } else {
-      me.push_back(ext[i]);
-      ms.push_back(str[i]);
+      me[nm] = static_cast<uint64_t>(shape[d]);
+      ms[nm] = st;
+      ++nm;
     }
   }
-  // me/ms are innermost first
   size_t first_outer = 0;
-  if (!me.empty() && ms[0] == static_cast<int64_t>(item)) {
-    c.run_bytes = me[0] * item;
+  if (nm && ms[0] == static_cast<int64_t>(item)) {
+    c->run_bytes = me[0] * item;
     first_outer = 1;
   } else {
-    c.run_bytes = item;
+    c->run_bytes = item;
   }
-  for (size_t i = me.size(); i-- > first_outer;) {
-    c.extent.push_back(me[i]);
-    c.stride.push_back(ms[i]);
+  for (size_t i = nm; i-- > first_outer;) {
+    c->extent[c->nd] = me[i];
+    c->stride[c->nd] = ms[i];
+    ++c->nd;
   }
-  return c;
 }
 
 struct Builder {
@@ -369,8 +368,9 @@ int build_tables(axr_plan* p) {
     for (const TensorRec& t : p->tensors) {
       if (t.nbytes == 0) continue;
       const uint64_t item = (static_cast<uint64_t>(t.bits) + 7) / 8;
-      const Collapsed c = collapse(t, p->shape_of(t), p->strides_of(t), item);
-      if (c.extent.empty() || (common_run && c.run_bytes != common_run)) {
+      Collapsed c;
+      collapse(t, p->shape_of(t), p->strides_of(t), item, &c);
+      if (c.nd == 0 || (common_run && c.run_bytes != common_run)) {
         uniform_runs = false;
         break;
       }
@@ -385,6 +385,8 @@ int build_tables(axr_plan* p) {
       rows *= 2;
   }
   Builder b{p, rows * kRowBytes};
+  p->segs.reserve(p->tensors.size() + 1);
+  p->seg_tensor.reserve(p->tensors.size());
 
   for (size_t i = 0; i < p->tensors.size(); ++i) {
     const TensorRec& t = p->tensors[i];
@@ -398,17 +400,17 @@ int build_tables(axr_plan* p) {
       for (int32_t d = 0; d < t.ndim; ++d)
         if (strides[d] == 0 && shape[d] > 1) p->overlapping_dst = true;
     }
-    Collapsed c = collapse(t, shape, strides, item);
-    const size_t first = p->segs.size();
+    Collapsed c;
+    collapse(t, shape, strides, item, &c);
     int rc;
     if (t.device_type == kDLROCM || t.device_type == kDLROCMHost) {
-      rc = b.add_strided(static_cast<uint32_t>(i), t.address, t.offset, c.extent.data(),
-                         c.stride.data(), c.extent.size(), c.run_bytes);
+      rc = b.add_strided(static_cast<uint32_t>(i), t.address, t.offset, c.extent, c.stride, c.nd,
+                         c.run_bytes);
       if (rc) return rc;
       if (pad) p->segs.back().meta |= static_cast<uint32_t>(pad);
     } else if (t.device_type == kDLCPU) {
-      rc = b.add_host(static_cast<uint32_t>(i), t.address, t.offset, c.extent.data(),
-                      c.stride.data(), c.extent.size(), c.run_bytes);
+      rc = b.add_host(static_cast<uint32_t>(i), t.address, t.offset, c.extent, c.stride, c.nd,
+                      c.run_bytes);
       if (rc) return rc;
       if (pad) {
         rc = b.add_seg(static_cast<uint32_t>(i), 0, end, 0, 1, kSegFillOnly);
@@ -419,7 +421,6 @@ int build_tables(axr_plan* p) {
       return fail(AXR_ERR_UNSUPPORTED,
                   "Unsupported memory type: DLPack device " + std::to_string(t.device_type));
     }
-    (void)first;
   }
   p->ntiles = static_cast<uint32_t>(b.tiles);
   Seg sentinel;
@@ -594,6 +595,10 @@ int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align, uint3
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_create: out of host memory");
   p->align = align;
   p->tensors.resize(n);
+  size_t ndims = 0;
+  for (size_t i = 0; i < n; ++i)
+    if (tensors[i].ndim > 0 && tensors[i].ndim <= kMaxNdim) ndims += 2 * static_cast<size_t>(tensors[i].ndim);
+  p->dims64.reserve(ndims);
   for (size_t i = 0; i < n; ++i) {
     rc = store_tensor(p, tensors[i], &p->tensors[i]);
     if (rc) {
