@@ -605,6 +605,70 @@ def test_error_paths(pkg, gpu):
     zero.pack(0, 0)
 
 
+def test_tensor_larger_than_4_gib(pkg, gpu):
+    """64-bit offsets end to end: one 5 GiB tensor next to small ones."""
+    import torch
+    n = 5 * (1 << 30) + 12345
+    big = torch.empty(n, dtype=torch.uint8, device=gpu)
+    big[: n // 8 * 8].view(torch.int64).random_()
+    big[n - 12345:] = 7
+    small = torch.arange(1000, device=gpu, dtype=torch.int32)
+    plan = pkg.BundlePlan.create([small, big, small], align=256)
+    info = plan.launch_info()
+    assert info["tiles"] * info["tile_bytes"] >= n and info["tile_bytes"] > 2048
+    payload = torch.empty(plan.payload_bytes, dtype=torch.uint8, device=gpu)
+    plan.pack(payload.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    offs, sizes = plan.layout()
+    assert sizes[1] == n and offs[2] == offs[1] + (n + 255) // 256 * 256
+    assert torch.equal(payload[offs[1]:offs[1] + n], big)
+    assert torch.equal(payload[offs[2]:offs[2] + 4000].view(torch.int32), small)
+    out_big = torch.zeros_like(big)
+    outs = [torch.zeros_like(small), out_big, torch.zeros_like(small)]
+    pkg.BundlePlan.from_header(plan.header).bind(outs).unpack(payload.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    assert torch.equal(out_big, big) and torch.equal(outs[0], small) and torch.equal(outs[2], small)
+
+
+def test_concurrent_host_threads(pkg, orc, gpu):
+    """Plans, packs and pool traffic from several host threads at once (the UCX
+    worker thread, thread-pool threads and Python threads all use one manager)."""
+    import threading
+    import torch
+    lib = pkg._capi.load()
+    errors = []
+
+    def worker(seed):
+        try:
+            rng = np.random.default_rng(seed)
+            s = C.c_void_p()
+            pkg._capi.check(lib.axr_stream_create(C.byref(s)))
+            for it in range(25):
+                sizes = [int(x) for x in rng.integers(1, 50000, size=30)]
+                host = [rng.integers(0, 256, size=n, dtype=np.uint8) for n in sizes]
+                with torch.cuda.stream(torch.cuda.ExternalStream(s.value)):
+                    tensors = [torch.from_numpy(a).to(gpu, non_blocking=False) for a in host]
+                packed = pkg.pack_bundle(tensors, align=256, stream=s.value)
+                pkg._capi.check(lib.axr_stream_synchronize(s))
+                back = np.zeros(packed.payload_bytes, np.uint8)
+                pkg._capi.check(lib.axr_memcpy(0, back.ctypes.data, 3, packed.payload.data, back.size))
+                if not np.array_equal(back, orc.pack(host, 256)):
+                    errors.append(f"thread {seed} iteration {it}: payload differs")
+                packed.plan.close()
+                packed.payload.release()
+            pkg._capi.check(lib.axr_stream_destroy(s))
+        except Exception as ex:   # noqa: BLE001
+            errors.append(repr(ex))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]
+    assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+
+
 # ------------------------------------------------------------------ memory resource
 
 def test_pool_and_copy_table(pkg, gpu):
