@@ -26,6 +26,7 @@ constexpr uint32_t kVecBytes = 16;                           // one dwordx4 per 
 constexpr uint32_t kRowBytes = kWaveLanes * kVecBytes;       // 1 KiB per wave-wide access
 constexpr uint32_t kMaxTileRows = 16;
 constexpr uint32_t kMaxThreadsPerWorkgroup = 1024;
+constexpr uint32_t kMaxElementThreads = 256;   // kernels that decode elements or transpose: more registers
 constexpr uint32_t kXcds = 8;   // accelerator dies; workgroup i is dispatched to die i % 8
 constexpr uint32_t kMaxOuterDims = 6;
 
@@ -45,17 +46,34 @@ static_assert(sizeof(Seg) == 32, "Seg layout");
 
 constexpr uint32_t kModeRunTiles = 0;   // every tile is a piece of one contiguous run
 constexpr uint32_t kModeElements = 1;   // tile covers packed bytes; lanes decode granules
+constexpr uint32_t kModeTranspose = 2;  // tile is a square block transposed through LDS
 
-struct Dims {             // 96 bytes, one per strided segment
+// Transposed tiles are T x T elements with T = kTransposeRowBytes / element size,
+// so that a tile row is 128 bytes (eight 16-byte vectors) on both sides.
+constexpr uint32_t kTransposeRowBytes = 128;
+constexpr uint32_t kTransposeLdsPitch = kTransposeRowBytes + 4;   // one dword of padding per row
+constexpr uint32_t kMaxBatchDims = 4;
+
+struct Dims {             // 160 bytes, one per strided segment
   uint32_t mode;
-  uint32_t ndim;          // outer (non-run) dimensions after collapsing, <= kMaxOuterDims
+  uint32_t ndim;          // outer (non-run) dimensions after collapsing, <= kMaxOuterDims;
+                          // kModeTranspose: batch dimensions (<= kMaxBatchDims)
   uint32_t tiles_per_run; // kModeRunTiles
-  uint32_t granule;       // kModeElements: bytes moved per lane access (1,2,4,8,16)
+  uint32_t granule;       // kModeElements: bytes moved per lane access (1,2,4,8,16);
+                          // kModeRunTiles: 1 + log2(tiles_per_run) when a power of two;
+                          // kModeTranspose: element size
   uint64_t nbytes;        // bytes of the whole segment
   uint32_t shape[kMaxOuterDims];
-  int64_t stride[kMaxOuterDims];   // bytes, outermost first
+  int64_t stride[kMaxOuterDims];   // bytes, outermost first, right-aligned
+  // kModeTranspose: A is the innermost packed dimension (strided in the tensor), B the
+  // dimension that is contiguous in the tensor; the rest are batch dimensions.
+  uint64_t pstride[kMaxBatchDims]; // packed byte strides of the batch dims (aligned with shape[2..5])
+  int64_t stride_a;                // tensor byte stride of A
+  uint64_t pstride_b;              // packed byte stride of B
+  uint32_t ext_a, ext_b;
+  uint32_t tiles_a, tiles_b;
 };
-static_assert(sizeof(Dims) == 96, "Dims layout");
+static_assert(sizeof(Dims) == 160, "Dims layout");
 
 struct KernelArgs {
   const Seg* segs;            // nseg + 1 entries, last is a sentinel with tile_begin == ntiles
@@ -76,7 +94,8 @@ struct LaunchConfig {
   uint32_t threads = 128;   // per workgroup, a multiple of 64
   uint32_t seg_shift = 0;   // wave_seg has one entry per 2^seg_shift tiles
   uint32_t nontemporal = 3;   // bit 0: tensor-side accesses, bit 1: payload-side accesses
-  bool elements = false;   // some segment uses kModeElements
+  bool elements = false;   // some segment uses kModeElements or kModeTranspose
+  uint32_t lds_per_wave = 0;   // bytes of LDS each wavefront needs (transposed tiles only)
   bool xcd_remap = false;  // give each die a contiguous share of the wave index space
 };
 
@@ -102,6 +121,7 @@ struct Tunables {
   int64_t payload_cache_bytes = 256ll << 20;
   int64_t gather_run_bytes = 512; // strided runs shorter than this use element mode
   int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
+  int64_t transpose = 1;          // move transposed views as square blocks through LDS
 };
 Tunables& tunables();
 

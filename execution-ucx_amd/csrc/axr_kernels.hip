@@ -166,48 +166,78 @@ __device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
 // Element mode: the tile covers kTile packed bytes of a strided segment whose
 // contiguous runs are short; each lane decodes the tensor address of its own
 // granules.  Only kernels instantiated with ELEMENTS carry this code, so the
-// streaming kernels keep a small register footprint.
+// streaming kernels keep a small register footprint.  The planner keeps every
+// extent and the run count below 2^31, so the per-granule arithmetic is 32-bit;
+// the tile's first run is decoded once (wave-uniform) and each lane only
+// propagates the carry of its own distance from it, stopping at the first
+// dimension where no lane carries further.
 template <bool PACK, uint32_t ROWS>
 __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_bytes, dims_table dm,
                                           gbytes pay, uint32_t q, uint32_t lane) {
   constexpr uint32_t kTile = ROWS * kRowBytes;
   const uint32_t g = dm->granule;
-  const uint32_t gpr = static_cast<uint32_t>(run_bytes / g);
+  const uint32_t gs = static_cast<uint32_t>(__builtin_ctz(g));
+  const uint32_t gpr = static_cast<uint32_t>(run_bytes >> gs);
+  const uint32_t nd = dm->ndim;
   const uint64_t b0 = static_cast<uint64_t>(q) * kTile;
   const uint64_t left = dm->nbytes - b0;
   const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
-  const uint64_t e0 = b0 / g;
-  const uint64_t run0 = e0 / gpr;
-  const uint32_t w0 = static_cast<uint32_t>(e0 - run0 * gpr);
+  const uint64_t e0 = b0 >> gs;
+  uint32_t run0, w0;
+  if ((e0 >> 32) == 0) {
+    const uint32_t e32 = static_cast<uint32_t>(e0);
+    run0 = e32 / gpr;
+    w0 = e32 - run0 * gpr;
+  } else {
+    run0 = static_cast<uint32_t>(e0 / gpr);
+    w0 = static_cast<uint32_t>(e0 - static_cast<uint64_t>(run0) * gpr);
+  }
   uint32_t idx0[kMaxOuterDims];
+  int64_t base = 0;
   {
-    uint64_t r = run0;
+    uint32_t r = run0;
 #pragma unroll
     for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
-      const uint32_t extent = dm->shape[d];
-      const uint64_t next = r / extent;
-      idx0[d] = static_cast<uint32_t>(r - next * extent);
-      r = next;
+      idx0[d] = 0;
+      if (static_cast<uint32_t>(d) + nd >= kMaxOuterDims) {
+        const uint32_t extent = dm->shape[d];
+        const uint32_t next = r / extent;
+        idx0[d] = r - next * extent;
+        base += static_cast<int64_t>(idx0[d]) * dm->stride[d];
+        r = next;
+      }
     }
   }
-  const uint32_t ng = n / g;
-  gbytes tbase = as_global(seg_ptr);
+  const uint32_t ng = n >> gs;
+  gbytes tbase = as_global(seg_ptr) + base;
   gbytes pbase = pay + b0;
   for (uint32_t e = lane; e < ng; e += kWaveLanes) {
     uint32_t w = w0 + e;
-    uint32_t carry = w / gpr;
-    w -= carry * gpr;
-    int64_t toff = static_cast<int64_t>(w) * g;
+    uint32_t carry;
+    if (gpr == 1) {
+      carry = w;
+      w = 0;
+    } else {
+      carry = w / gpr;
+      w -= carry * gpr;
+    }
+    int64_t toff = static_cast<int64_t>(w << gs);
 #pragma unroll
     for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
-      const uint32_t extent = dm->shape[d];
-      const uint64_t v = static_cast<uint64_t>(idx0[d]) + carry;
-      const uint32_t c = static_cast<uint32_t>(v / extent);
-      const uint32_t i = static_cast<uint32_t>(v - static_cast<uint64_t>(c) * extent);
-      toff += static_cast<int64_t>(i) * dm->stride[d];
-      carry = c;
+      if (static_cast<uint32_t>(d) + nd >= kMaxOuterDims) {
+        if (__builtin_amdgcn_ballot_w64(carry != 0) == 0) break;   // wave-uniform
+        const uint32_t extent = dm->shape[d];
+        uint32_t v = idx0[d] + carry;
+        uint32_t c = 0;
+        if (__builtin_amdgcn_ballot_w64(v >= extent) != 0) {
+          c = v / extent;
+          v -= c * extent;
+        }
+        toff += static_cast<int64_t>(static_cast<int32_t>(v - idx0[d])) * dm->stride[d];
+        carry = c;
+      }
     }
-    gbytes pp = pbase + static_cast<uint64_t>(e) * g;
+    gbytes pp = pbase + (static_cast<uint64_t>(e) << gs);
     if constexpr (PACK) {
       move_granule_dyn(g, tbase + toff, pp);
     } else {
@@ -216,10 +246,218 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   }
 }
 
+// ---------------------------------------------------------------- transposed tiles
+//
+// A view whose innermost packed dimension (A) is strided in the tensor while
+// another dimension (B) is contiguous there is a transposition: rows that are
+// contiguous on one side are columns on the other.  A wavefront moves one
+// T x T block (T = 128 bytes / element size) through its own slice of LDS:
+// rows are read from global memory as eight 16-byte vectors each (eight rows per
+// instruction), parked in LDS in the same orientation with a one-dword pad per
+// row, gathered back column-wise, and written as 16-byte vectors along the
+// other side's contiguous direction.  Both global sides therefore see whole
+// 128-byte lines.  LDS traffic of one wavefront is processed in issue order,
+// so no workgroup barrier is involved (waves never share a slice).
+#define AXR_LDS __attribute__((address_space(3)))
+typedef AXR_LDS uint8_t* lbytes;
+
+template <uint32_t E> struct unit_of;
+template <> struct unit_of<1> { typedef uint8_t type; };
+template <> struct unit_of<2> { typedef uint16_t type; };
+template <> struct unit_of<4> { typedef uint32_t type; };
+template <> struct unit_of<8> { typedef uint64_t type; };
+template <> struct unit_of<16> { typedef u32x4 type; };
+
+template <uint32_t E>
+__device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gbytes wr,
+                                               int64_t wr_pitch, lbytes lds, uint32_t lane) {
+  constexpr uint32_t T = kTransposeRowBytes / E, NK = T / 8, EV = kVecBytes / E;
+  typedef typename unit_of<E>::type U;
+  typedef U __attribute__((aligned(E < 4 ? E : 4))) lds_unit;
+  const uint32_t r8 = lane >> 3, v = lane & 7;
+  u32x4 x[NK];
+#pragma unroll
+  for (uint32_t k = 0; k < NK; ++k)
+    x[k] = load16<false>(rd + static_cast<int64_t>(k * 8 + r8) * rd_pitch + v * kVecBytes);
+#pragma unroll
+  for (uint32_t k = 0; k < NK; ++k) {
+    AXR_LDS uint32_t* w =
+        reinterpret_cast<AXR_LDS uint32_t*>(lds + (k * 8 + r8) * kTransposeLdsPitch + v * kVecBytes);
+    w[0] = x[k].x;
+    w[1] = x[k].y;
+    w[2] = x[k].z;
+    w[3] = x[k].w;
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (uint32_t k = 0; k < NK; ++k) {
+    const uint32_t c = k * 8 + r8;
+    U e[EV];
+#pragma unroll
+    for (uint32_t i = 0; i < EV; ++i)
+      e[i] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + (v * EV + i) * kTransposeLdsPitch + c * E);
+    u32x4 out;
+    __builtin_memcpy(&out, e, kVecBytes);
+    store16<false>(wr + static_cast<int64_t>(c) * wr_pitch + v * kVecBytes, out);
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+__device__ __forceinline__ void lds_put(uint32_t E, gcbytes src, lbytes dst) {
+  switch (E) {
+    case 16: {
+      typedef u32x4 __attribute__((aligned(1))) gl;
+      const u32x4 x = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
+      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(dst);
+      w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
+      break;
+    }
+    case 8: {
+      typedef uint64_t __attribute__((aligned(1))) gl;
+      typedef uint64_t __attribute__((aligned(4))) ll;
+      *reinterpret_cast<AXR_LDS ll*>(dst) = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
+      break;
+    }
+    case 4: {
+      typedef uint32_t __attribute__((aligned(1))) gl;
+      *reinterpret_cast<AXR_LDS uint32_t*>(dst) = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
+      break;
+    }
+    case 2: {
+      typedef uint16_t __attribute__((aligned(1))) gl;
+      *reinterpret_cast<AXR_LDS uint16_t*>(dst) = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
+      break;
+    }
+    default: *dst = *src; break;
+  }
+}
+
+__device__ __forceinline__ void lds_get(uint32_t E, const AXR_LDS uint8_t* src, gbytes dst) {
+  switch (E) {
+    case 16: {
+      typedef u32x4 __attribute__((aligned(1))) gl;
+      const AXR_LDS uint32_t* r = reinterpret_cast<const AXR_LDS uint32_t*>(src);
+      const u32x4 x = {r[0], r[1], r[2], r[3]};
+      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = x;
+      break;
+    }
+    case 8: {
+      typedef uint64_t __attribute__((aligned(1))) gl;
+      typedef uint64_t __attribute__((aligned(4))) ll;
+      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = *reinterpret_cast<const AXR_LDS ll*>(src);
+      break;
+    }
+    case 4: {
+      typedef uint32_t __attribute__((aligned(1))) gl;
+      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = *reinterpret_cast<const AXR_LDS uint32_t*>(src);
+      break;
+    }
+    case 2: {
+      typedef uint16_t __attribute__((aligned(1))) gl;
+      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = *reinterpret_cast<const AXR_LDS uint16_t*>(src);
+      break;
+    }
+    default: *dst = *src; break;
+  }
+}
+
+// Quotient idx / d for idx < 2^14, d <= 128, by multiplication (exact in that range).
+__device__ __forceinline__ uint32_t small_div(uint32_t idx, uint32_t d, uint32_t magic) {
+  return d == 1 ? idx : __umulhi(idx, magic);
+}
+
+// Partial or misaligned block: the same two phases one element per lane.  Both
+// global sides still see consecutive lanes on consecutive elements.
+__device__ __forceinline__ void transpose_edge(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
+                                               int64_t wr_pitch, uint32_t nr, uint32_t nc,
+                                               lbytes lds, uint32_t lane) {
+  const uint32_t total = nr * nc;
+  const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
+  const uint32_t mc = 0xffffffffu / nc + 1u, mr = 0xffffffffu / nr + 1u;
+  for (uint32_t i = lane; i < total; i += kWaveLanes) {
+    const uint32_t r = small_div(i, nc, mc);
+    const uint32_t c = i - r * nc;
+    lds_put(E, rd + static_cast<int64_t>(r) * rd_pitch + (c << es),
+            lds + r * kTransposeLdsPitch + (c << es));
+  }
+  __builtin_amdgcn_wave_barrier();
+  for (uint32_t i = lane; i < total; i += kWaveLanes) {
+    const uint32_t c = small_div(i, nr, mr);
+    const uint32_t r = i - c * nr;
+    lds_get(E, lds + r * kTransposeLdsPitch + (c << es),
+            wr + static_cast<int64_t>(c) * wr_pitch + (r << es));
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+// Reads nr rows of nc elements (rows rd_pitch bytes apart) and writes nc rows of
+// nr elements (rows wr_pitch bytes apart).
+__device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
+                                                int64_t wr_pitch, uint32_t nr, uint32_t nc,
+                                                lbytes lds, uint32_t lane) {
+  const uint32_t T = kTransposeRowBytes >> __builtin_ctz(E);
+  const uint64_t bits = reinterpret_cast<uintptr_t>(rd) | static_cast<uint64_t>(rd_pitch) |
+                        reinterpret_cast<uintptr_t>(wr) | static_cast<uint64_t>(wr_pitch);
+  if (nr == T && nc == T && (bits & 15u) == 0) {
+    switch (E) {
+      case 1: transpose_full<1>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
+      case 2: transpose_full<2>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
+      case 4: transpose_full<4>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
+      case 8: transpose_full<8>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
+      default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
+    }
+  } else {
+    transpose_edge(E, rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane);
+  }
+}
+
+// Tile q of a transposed segment: batch index (outer dims), then block (ia, ib).
+template <bool PACK>
+__device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, gbytes pay,
+                                               uint32_t q, lbytes lds, uint32_t lane) {
+  const uint32_t E = dm->granule;
+  const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
+  const uint32_t T = kTransposeRowBytes >> es;
+  const uint32_t ta = dm->tiles_a, tb = dm->tiles_b;
+  const uint32_t per_batch = ta * tb;
+  uint32_t o = q / per_batch;
+  const uint32_t rem = q - o * per_batch;
+  const uint32_t ia = rem / tb;
+  const uint32_t ib = rem - ia * tb;
+  int64_t toff = 0;
+  uint64_t poff = 0;
+  const uint32_t nbatch = dm->ndim;
+#pragma unroll
+  for (int d = static_cast<int>(kMaxBatchDims) - 1; d >= 0; --d) {
+    if (static_cast<uint32_t>(d) + nbatch >= kMaxBatchDims) {
+      const uint32_t extent = dm->shape[kMaxOuterDims - kMaxBatchDims + d];
+      const uint32_t next = o / extent;
+      const uint32_t idx = o - next * extent;
+      toff += static_cast<int64_t>(idx) * dm->stride[kMaxOuterDims - kMaxBatchDims + d];
+      poff += static_cast<uint64_t>(idx) * dm->pstride[d];
+      o = next;
+    }
+  }
+  const uint32_t a0 = ia * T, b0 = ib * T;
+  const uint32_t ra = dm->ext_a - a0, rb = dm->ext_b - b0;
+  const uint32_t na = ra < T ? ra : T, nb = rb < T ? rb : T;
+  const int64_t stride_a = dm->stride_a;
+  const uint64_t pstride_b = dm->pstride_b;
+  gbytes ten = as_global(seg_ptr) + toff + static_cast<int64_t>(a0) * stride_a +
+               (static_cast<uint64_t>(b0) << es);
+  gbytes pp = pay + poff + static_cast<uint64_t>(b0) * pstride_b + (static_cast<uint64_t>(a0) << es);
+  if constexpr (PACK) {
+    transpose_block(E, ten, stride_a, pp, static_cast<int64_t>(pstride_b), na, nb, lds, lane);
+  } else {
+    transpose_block(E, pp, static_cast<int64_t>(pstride_b), ten, stride_a, nb, na, lds, lane);
+  }
+}
+
 template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
-__global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
+__global__ __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
     const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
-    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift) {
+    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
+    uint32_t lds_per_wave) {
   // Scalar arguments (not one struct) so that the compiler can preload them
   // into SGPRs at dispatch instead of fetching the kernarg segment first.
   KernelArgs a;
@@ -304,7 +542,13 @@ __global__ __launch_bounds__(kMaxThreadsPerWorkgroup) void bundle_kernel(
           wave_copy<ROWS, NTP, NTT>(p, ten, left, lane, lane_off);
         }
       } else if constexpr (ELEMENTS) {
-        element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
+        if (dm->mode == kModeTranspose) {
+          extern __shared__ uint8_t lds_slices[];   // lds_per_wave bytes for each wavefront
+          lbytes lds = (lbytes)lds_slices + (threadIdx.x >> 6) * lds_per_wave;
+          transpose_tile<PACK>(seg_ptr, dm, pay, q, lds, lane);
+        } else {
+          element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
+        }
       }
       if constexpr (PACK) {
         if (last && pad) wave_zero(pay + dm->nbytes, pad, lane);
@@ -369,9 +613,10 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
 template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
-#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift
+  const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * (cfg.threads / kWaveLanes) : 0u;
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave
 #define AXR_LAUNCH(NTT, NTP, EL) \
-  hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, 0, stream, AXR_ARGS)
+  hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, lds_bytes, stream, AXR_ARGS)
   if (cfg.elements) {
     // strided tensors with short runs are present: the general kernel
     AXR_LAUNCH(false, false, true);
@@ -416,6 +661,10 @@ int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& 
     return fail(AXR_ERR_INVALID, "workgroup size must be a multiple of 64 up to 1024");
   if (args.xcd_remap && (cfg.workgroups % kXcds || args.xcd_remap != cfg.workgroups / kXcds))
     return fail(AXR_ERR_INVALID, "die remapping needs a grid that is a multiple of 8");
+  if (cfg.elements && cfg.threads > kMaxElementThreads)
+    return fail(AXR_ERR_INVALID, "bundles with short strided runs need workgroups of at most 256");
+  if (static_cast<uint64_t>(cfg.lds_per_wave) * (cfg.threads / kWaveLanes) > 64u * 1024u)
+    return fail(AXR_ERR_INVALID, "workgroup needs more than 64 KiB of LDS");
   const uint64_t covered = static_cast<uint64_t>(cfg.workgroups) * (cfg.threads / kWaveLanes) *
                            cfg.tiles_per_wave;
   if (covered < args.ntiles || args.tiles_per_wave != cfg.tiles_per_wave) {

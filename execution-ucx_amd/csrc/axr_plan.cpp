@@ -188,6 +188,7 @@ void invalidate_tables(axr_plan* p) {
   p->host_copy_tensor.clear();
   p->overlapping_dst = false;
   p->ntiles = 0;
+  p->cfg.lds_per_wave = 0;
 }
 
 // Wait until the device no longer reads the plan's tables.  No event is
@@ -309,7 +310,58 @@ struct Builder {
       dm.stride[kMaxOuterDims - nd + d] = str[d];
     }
     uint64_t ntile;
-    if (run_bytes >= static_cast<uint64_t>(tunables().gather_run_bytes)) {
+    // A transposition: no contiguous inner run beyond one element, but some outer
+    // dimension (B) is contiguous in the tensor.  Blocks of A x B go through LDS.
+    size_t dim_b = nd;
+    if (nd >= 2 && run_bytes <= kVecBytes && (run_bytes & (run_bytes - 1)) == 0 &&
+        tunables().transpose != 0 && ext[nd - 1] >= 8) {
+      for (size_t d = 0; d + 1 < nd; ++d) {
+        if (str[d] == static_cast<int64_t>(run_bytes) && ext[d] >= 8) {
+          dim_b = d;
+          break;
+        }
+      }
+    }
+    if (dim_b < nd) {
+      const uint32_t e = static_cast<uint32_t>(run_bytes);
+      const uint32_t t = kTransposeRowBytes / e;
+      const size_t dim_a = nd - 1;
+      dm.mode = kModeTranspose;
+      dm.granule = e;
+      dm.ndim = static_cast<uint32_t>(nd - 2);
+      for (uint32_t d = 0; d < kMaxOuterDims; ++d) {
+        dm.shape[d] = 1;
+        dm.stride[d] = 0;
+      }
+      // packed byte stride of dim d = element size * product of the inner extents
+      uint64_t packed[kMaxOuterDims];
+      uint64_t acc = e;
+      for (size_t d = nd; d-- > 0;) {
+        packed[d] = acc;
+        acc *= ext[d];
+      }
+      uint64_t batches = 1;
+      size_t slot = kMaxBatchDims;
+      for (size_t d = nd; d-- > 0;) {
+        if (d == dim_a || d == dim_b) continue;
+        --slot;
+        dm.shape[kMaxOuterDims - kMaxBatchDims + slot] = static_cast<uint32_t>(ext[d]);
+        dm.stride[kMaxOuterDims - kMaxBatchDims + slot] = str[d];
+        dm.pstride[slot] = packed[d];
+        batches *= ext[d];
+      }
+      dm.stride_a = str[dim_a];
+      dm.pstride_b = packed[dim_b];
+      dm.ext_a = static_cast<uint32_t>(ext[dim_a]);
+      dm.ext_b = static_cast<uint32_t>(ext[dim_b]);
+      dm.tiles_a = (dm.ext_a + t - 1) / t;
+      dm.tiles_b = (dm.ext_b + t - 1) / t;
+      const uint64_t per_batch = static_cast<uint64_t>(dm.tiles_a) * dm.tiles_b;
+      if (per_batch > 0xffffffffull || batches > 0xffffffffull / per_batch)
+        return fail(AXR_ERR_UNSUPPORTED, "transposed tensor has too many blocks");
+      ntile = batches * per_batch;
+      p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, t * kTransposeLdsPitch);
+    } else if (run_bytes >= static_cast<uint64_t>(tunables().gather_run_bytes)) {
       dm.mode = kModeRunTiles;
       const uint64_t tpr = (run_bytes + tile_bytes - 1) / tile_bytes;
       if (tpr > 0xffffffffull || runs > 0xffffffffull)
@@ -321,6 +373,8 @@ struct Builder {
       ntile = runs * tpr;
     } else {
       dm.mode = kModeElements;
+      // the kernel's per-granule index arithmetic is 32-bit
+      if (runs > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "strided tensor has too many runs");
       uint32_t g = 16;
       while (g > 1 && (run_bytes % g) != 0) g >>= 1;
       dm.granule = g;
@@ -433,6 +487,14 @@ int build_tables(axr_plan* p) {
                  static_cast<uint64_t>(tn.max_waves);
   if (tpw == 0) tpw = 1;
   p->cfg.threads = tn.threads ? static_cast<uint32_t>(tn.threads) : (p->ntiles < 65536 ? 256u : 128u);
+  p->cfg.elements = false;
+  for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode != kModeRunTiles;
+  if (p->cfg.elements) p->cfg.threads = std::min(p->cfg.threads, kMaxElementThreads);
+  if (p->cfg.lds_per_wave) {
+    // transposed blocks: every wave of a workgroup owns a slice of at most 64 KiB of LDS
+    const uint32_t fit = (64u * 1024u / p->cfg.lds_per_wave) * kWaveLanes;
+    p->cfg.threads = std::min(p->cfg.threads, fit);
+  }
   const uint32_t waves_per_wg = p->cfg.threads / kWaveLanes;
   const uint64_t per_wg = tpw * waves_per_wg;
   p->cfg.tiles_per_wave = static_cast<uint32_t>(tpw);
@@ -445,8 +507,6 @@ int build_tables(axr_plan* p) {
   } else {
     p->cfg.nontemporal = static_cast<uint32_t>(tn.nontemporal) & 3u;
   }
-  p->cfg.elements = false;
-  for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode == kModeElements;
 
   // Tile-block index: entry k = segment that holds tile k << seg_shift.  Blocks
   // are sized to about one segment each (a power of two, at most 256 tiles), so
@@ -847,13 +907,20 @@ int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity
       o.mode = 3;
     } else {
       const Dims& dm = plan->dims[dsel - 1];
-      o.mode = dm.mode == kModeRunTiles ? 1 : 2;
+      o.mode = dm.mode == kModeRunTiles ? 1 : (dm.mode == kModeElements ? 2 : 5);
       o.nbytes = dm.nbytes;
       o.ndim = dm.ndim;
       o.granule = dm.granule;
       for (uint32_t d = 0; d < dm.ndim; ++d) {
         o.shape[d] = dm.shape[kMaxOuterDims - dm.ndim + d];
         o.stride_bytes[d] = dm.stride[kMaxOuterDims - dm.ndim + d];
+      }
+      if (dm.mode == kModeTranspose) {   // batch dims, then B (contiguous in the tensor), then A
+        o.shape[o.ndim] = dm.ext_b;
+        o.stride_bytes[o.ndim] = dm.granule;
+        o.shape[o.ndim + 1] = dm.ext_a;
+        o.stride_bytes[o.ndim + 1] = dm.stride_a;
+        o.ndim += 2;
       }
     }
   }

@@ -308,6 +308,8 @@ int axr_tune_set(const char* key, int64_t value) {
     t.threads = value;
   } else if (k == "xcd_remap") {
     t.xcd_remap = value ? 1 : 0;
+  } else if (k == "transpose") {
+    t.transpose = value ? 1 : 0;
   } else {
     return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   }
@@ -326,6 +328,7 @@ int axr_tune_get(const char* key, int64_t* value) {
   else if (k == "gather_run_bytes") *value = t.gather_run_bytes;
   else if (k == "threads") *value = t.threads;
   else if (k == "xcd_remap") *value = t.xcd_remap;
+  else if (k == "transpose") *value = t.transpose;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

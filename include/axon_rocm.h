@@ -288,14 +288,16 @@ AXR_API int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info);
 typedef struct axr_segment_info {
   uint32_t tensor;        /* index of the tensor the segment belongs to       */
   uint32_t mode;          /* 0 one run, 1 strided run tiles, 2 strided
-                             elements, 3 zero fill only, 4 host copy          */
+                             elements, 3 zero fill only, 4 host copy,
+                             5 transposed blocks (dims listed as batch...,
+                             the tensor-contiguous dim, the packed-inner dim) */
   uint64_t address;       /* tensor-side address of the first element         */
   uint64_t offset;        /* payload offset                                   */
   uint64_t run_bytes;     /* contiguous bytes per run                         */
   uint64_t nbytes;        /* bytes of the whole segment                       */
   uint32_t pad;           /* zero bytes written after the segment by pack     */
   uint32_t ndim;          /* strided outer dimensions (<= 6)                  */
-  uint32_t granule;       /* mode 2: bytes per lane access                    */
+  uint32_t granule;       /* mode 2: bytes per lane access; mode 5: element   */
   uint32_t tiles;
   uint32_t shape[6];
   int64_t stride_bytes[6];
@@ -310,7 +312,8 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "tile_rows" (KiB per wavefront tile: 0 auto, 1, 2, 4, 8, 16), "max_tiles",
  * "max_waves", "threads" (workgroup size), "nontemporal" (-1 auto, or bit 0
  * tensor side / bit 1 payload side), "payload_cache_bytes", "gather_run_bytes",
- * "xcd_remap".  Unknown key -> AXR_ERR_INVALID. */
+ * "xcd_remap", "transpose" (1: transposed views move as square blocks through
+ * LDS; 0: element by element).  Unknown key -> AXR_ERR_INVALID. */
 AXR_API int axr_tune_set(const char* key, int64_t value);
 AXR_API int axr_tune_get(const char* key, int64_t* value);
 

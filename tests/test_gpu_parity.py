@@ -319,6 +319,93 @@ def test_strided_gather_scatter_random(pkg, orc, gpu, dtype_name):
             assert len(metas) == len(views) - 1
 
 
+@pytest.mark.parametrize("dtype_name", ["uint8", "bfloat16", "float32", "float64", "complex128"])
+def test_transposed_views(pkg, orc, gpu, dtype_name):
+    """Views whose packed-inner dimension is strided while another dimension is
+    contiguous in the tensor move as square blocks through LDS: whole aligned
+    blocks, ragged edges, misaligned bases and batched permutations, against the
+    oracle's element-by-element gather and scatter."""
+    import torch
+    dt = getattr(torch, dtype_name)
+    item = torch.empty((), dtype=dt).element_size()
+    t = 128 // item                                            # block edge in elements
+    rng = np.random.default_rng(100 + item)
+
+    def parent_of(shape):
+        nbytes = int(np.prod(shape)) * item
+        return rand_bytes_tensor(rng, nbytes, gpu).view(dt).reshape(shape)
+
+    m2 = parent_of([2 * t, 3 * t])
+    m3 = parent_of([t + 5, 2 * t + 3])
+    m4 = parent_of([3, 20, 2, 24])
+    m5 = parent_of([2, 9, 70])
+    cases = [
+        (m2, m2.t()),                                          # whole aligned blocks only
+        (m3, m3.t()),                                          # ragged in both directions
+        (m3, m3[1:, 3:].t()),                                  # base off the 16-byte grid
+        (m3, m3[::2, 1::3].t()),                               # strided on both sides: element mode
+        (m4, m4.permute(2, 0, 3, 1)),                          # two batch dims around the block
+        (m4, m4[:, 2:19].permute(0, 2, 3, 1)),
+        (m5, m5.permute(2, 0, 1)),                             # [70, 2*9] after merging
+        (m5, m5.permute(1, 2, 0)),
+    ]
+    views = [v for _, v in cases]
+    plan = pkg.BundlePlan.create(views, align=256)
+    modes = [s["mode"] for s in plan.segments()]
+    assert modes.count(5) >= 5, modes
+    chunks = []
+    for parent, v in cases:
+        host_parent = parent.reshape(-1).view(torch.uint8).cpu().numpy()
+        chunks.append(orc.gather_strided(host_parent, v.data_ptr() - parent.data_ptr(),
+                                         tuple(v.shape), tuple(v.stride()), item))
+    for align in (256, 1):
+        got, plan, buf = run_pack(pkg, views, align, gpu)
+        assert np.array_equal(got, orc.pack(chunks, align)), align
+        # scatter back through the same views of poisoned twins
+        twins, tviews, expects = [], [], []
+        for (parent, v), c in zip(cases, chunks):
+            twin = device_bytes(parent.numel() * item, gpu, fill=0x77).view(dt).reshape(parent.shape)
+            twins.append(twin)
+            tviews.append(twin.as_strided(v.shape, v.stride(), v.storage_offset()))
+            e = np.full(parent.numel() * item, 0x77, np.uint8)
+            orc.scatter_strided(c, e, v.data_ptr() - parent.data_ptr(), tuple(v.shape),
+                                tuple(v.stride()), item)
+            expects.append(e)
+        pkg.BundlePlan.from_header(plan.header).bind(tviews).unpack(buf.data_ptr(), plan.payload_bytes)
+        torch.cuda.synchronize()
+        for i, (twin, e) in enumerate(zip(twins, expects)):
+            assert np.array_equal(twin.reshape(-1).view(torch.uint8).cpu().numpy(), e), (align, i)
+    # the element-by-element path gives the same bytes
+    pkg.tune(transpose=0)
+    try:
+        got0, plan0, _ = run_pack(pkg, views, 256, gpu)
+        assert 5 not in {s["mode"] for s in plan0.segments()}
+        assert np.array_equal(got0, orc.pack(chunks, 256))
+    finally:
+        pkg.tune(transpose=1)
+
+
+def test_transposed_large_matrix_round_trip(pkg, gpu):
+    """A 4096 x 4096 bf16 transposition (32 MiB) against torch's own
+    contiguous copy, and back into a transposed destination."""
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    x = torch.randint(-2 ** 15, 2 ** 15, (4096, 4096), device="cuda", generator=g,
+                      dtype=torch.int16).view(torch.bfloat16)
+    plan = pkg.BundlePlan.create([x.t()], align=256)
+    assert [s["mode"] for s in plan.segments()] == [5]
+    buf = device_bytes(plan.payload_bytes, gpu)
+    plan.pack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    want = x.t().contiguous().view(torch.int16).reshape(-1)
+    assert torch.equal(buf[:want.numel() * 2].view(torch.int16), want)
+    y = torch.zeros_like(x)
+    pkg.BundlePlan.from_header(plan.header).bind([y.t()]).unpack(buf.data_ptr(), plan.payload_bytes)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), x.view(torch.int16))
+
+
 def test_strided_many_dims_and_long_runs(pkg, orc, gpu):
     """More strided outer dimensions than the device table holds (peeled on the
     host), runs that span several tiles, and a transposed matrix."""
@@ -334,7 +421,7 @@ def test_strided_many_dims_and_long_runs(pkg, orc, gpu):
     chunks = [tbytes(v) for v in views]
     plan = pkg.BundlePlan.create(views, align=256)
     modes = {s["mode"] for s in plan.segments()}
-    assert {1, 2} <= modes                                      # run tiles and element mode both used
+    assert {1, 2, 5} <= modes                  # run tiles, element mode and transposed blocks all used
     got, plan, buf = run_pack(pkg, views, 256, gpu)
     assert np.array_equal(got, orc.pack(chunks, 256))
     outs = [torch.zeros_like(v, memory_format=torch.contiguous_format) for v in views]

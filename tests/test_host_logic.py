@@ -196,7 +196,7 @@ def seg_of(pkg, view, align=256, **tune):
         return plan.segments(), plan.launch_info()
     finally:
         if tune:
-            pkg.tune(tile_rows=0, gather_run_bytes=512)
+            pkg.tune(tile_rows=0, gather_run_bytes=512, transpose=1)
 
 
 def test_compact_tensor_is_one_run(pkg):
@@ -233,7 +233,7 @@ def test_pitched_view_rows(pkg):
 
 def test_short_runs_use_element_mode(pkg):
     # transposed matrix: no contiguous inner run
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(4, 16, 1)))
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(4, 16, 1)), transpose=0)
     s = segs[0]
     assert (s["mode"], s["run_bytes"], s["granule"]) == (2, 2, 2)
     assert s["shape"] == (30, 20) and s["stride_bytes"] == (2, 60)
@@ -247,6 +247,31 @@ def test_short_runs_use_element_mode(pkg):
     assert segs[0]["mode"] == 1
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=400)
     assert segs[0]["mode"] == 2 and segs[0]["granule"] == 4
+
+
+def test_transposed_views_use_square_blocks(pkg):
+    # fp16 [300, 200] transposed: B (contiguous in the tensor) = 300, A (packed inner) = 200
+    segs, info = seg_of(pkg, tv(pkg, 0x10000, [300, 200], strides=[1, 300], dtype=(4, 16, 1)))
+    s = segs[0]
+    assert (s["mode"], s["granule"], s["nbytes"]) == (5, 2, 120000)
+    assert s["shape"] == (300, 200) and s["stride_bytes"] == (2, 600)
+    assert s["tiles"] == 5 * 4                      # 64 x 64 element blocks
+    assert info["threads_per_workgroup"] <= 256
+    # fp32 [B, H, S, D] -> permute(2, 0, 3, 1): H becomes the innermost packed dim
+    b, h, sq, d = 2, 40, 3, 50
+    v = tv(pkg, 0x10000, [sq, b, d, h], strides=[d, h * sq * d, 1, sq * d], dtype=(2, 32, 1))
+    s = seg_of(pkg, v)[0][0]
+    assert (s["mode"], s["granule"]) == (5, 4)
+    # batch dims (sq, b), then the tensor-contiguous dim d, then the packed-inner dim h
+    assert s["shape"] == (sq, b, d, h)
+    assert s["stride_bytes"] == (4 * d, 4 * h * sq * d, 4, 4 * sq * d)
+    assert s["tiles"] == b * sq * 2 * 2             # 32 x 32 element blocks
+    # tiny extents and odd element sizes stay in element mode
+    assert seg_of(pkg, tv(pkg, 0x10000, [30, 4], strides=[1, 30]))[0][0]["mode"] == 2
+    assert seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(2, 96, 1)))[0][0]["mode"] == 2
+    # 16-byte elements transpose as 8 x 8 blocks
+    s = seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(2, 128, 1)))[0][0]
+    assert (s["mode"], s["granule"], s["tiles"]) == (5, 16, 4 * 3)
 
 
 def test_negative_and_many_strides(pkg):
