@@ -119,7 +119,7 @@ struct Tunables {
   // last-level cache when the consumer (unpack, or the transport's copy) reads it.
   int64_t nontemporal = -1;
   int64_t payload_cache_bytes = 256ll << 20;
-  int64_t gather_run_bytes = 512; // strided runs shorter than this use element mode
+  int64_t gather_run_bytes = 1024; // strided runs shorter than this use element mode (measured crossover)
   int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
   int64_t transpose = 1;          // move transposed views as square blocks through LDS
 };

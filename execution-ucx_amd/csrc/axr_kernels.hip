@@ -209,18 +209,14 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
     }
   }
   const uint32_t ng = n >> gs;
+  const uint32_t gpr_magic = 0xffffffffu / gpr + 1u;
   gbytes tbase = as_global(seg_ptr) + base;
   gbytes pbase = pay + b0;
   for (uint32_t e = lane; e < ng; e += kWaveLanes) {
     uint32_t w = w0 + e;
-    uint32_t carry;
-    if (gpr == 1) {
-      carry = w;
-      w = 0;
-    } else {
-      carry = w / gpr;
-      w -= carry * gpr;
-    }
+    // w < gpr + tile / g: for gpr <= 2^15, w * gpr < 2^32 and the multiply-high quotient is exact
+    uint32_t carry = gpr == 1 ? w : (gpr <= 32768u ? __umulhi(w, gpr_magic) : w / gpr);
+    w -= carry * gpr;
     int64_t toff = static_cast<int64_t>(w << gs);
 #pragma unroll
     for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {

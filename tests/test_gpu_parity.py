@@ -237,23 +237,33 @@ def test_every_kernel_instantiation(pkg, orc, gpu, rows, threads):
     rng = np.random.default_rng(rows * 1000 + threads)
     sizes = [0, 5, 16, 17, 1000, 1024, 1025, 2048, 4097, 16384, 16400, 70001, 3 * 16384 + 100]
     sizes += [int(x) for x in rng.integers(1, 60000, size=20)]
-    tensors = [rand_bytes_tensor(rng, n, gpu) for n in sizes]
+    streaming = [rand_bytes_tensor(rng, n, gpu) for n in sizes]
     mat = rand_bytes_tensor(rng, 200 * 3000, gpu).reshape(200, 3000)
-    tensors += [mat[::2, 16:2064], mat.t()[5:9]]           # run tiles and element mode
-    chunks = [tbytes(t) for t in tensors]
+    streaming += [mat[::2, 16:2064]]                        # run tiles
+    # short runs and a transposition select the kernels that decode elements
+    # (their workgroups hold at most 256 threads)
+    general = streaming + [mat.t()[5:9], mat[:, 7:107], mat.t()]
     try:
-        for nt, max_waves in ((3, 1 << 20), (0, 1 << 20), (1, 7), (2, 1 << 20)):
-            pkg.tune(tile_rows=rows, threads=threads, nontemporal=nt, max_waves=max_waves)
-            for align in (1, 256):
-                got, plan, buf = run_pack(pkg, tensors, align, gpu)
-                info = plan.launch_info()
-                assert info["tile_bytes"] == rows * 1024 and info["threads_per_workgroup"] == threads
-                assert np.array_equal(got, orc.pack(chunks, align)), (nt, max_waves, align)
-                outs = [torch.zeros_like(t, memory_format=torch.contiguous_format) for t in tensors]
-                pkg.BundlePlan.from_header(plan.header).bind(outs).unpack(buf.data_ptr(), plan.payload_bytes)
-                torch.cuda.synchronize()
-                for o, c in zip(outs, chunks):
-                    assert np.array_equal(tbytes(o), c), (nt, max_waves, align)
+        for tensors, thread_cap in ((streaming, 1024), (general, 256)):
+            chunks = [tbytes(t) for t in tensors]
+            for nt, max_waves in ((3, 1 << 20), (0, 1 << 20), (1, 7), (2, 1 << 20)):
+                pkg.tune(tile_rows=rows, threads=threads, nontemporal=nt, max_waves=max_waves)
+                for align in (1, 256):
+                    got, plan, buf = run_pack(pkg, tensors, align, gpu)
+                    info = plan.launch_info()
+                    assert info["tile_bytes"] == rows * 1024
+                    got_threads = info["threads_per_workgroup"]
+                    if tensors is streaming:
+                        assert got_threads == threads
+                    else:                       # also bounded by the LDS the byte transposition needs
+                        assert got_threads in (min(threads, 192), min(threads, thread_cap))
+                    assert np.array_equal(got, orc.pack(chunks, align)), (nt, max_waves, align)
+                    outs = [torch.zeros_like(t, memory_format=torch.contiguous_format) for t in tensors]
+                    pkg.BundlePlan.from_header(plan.header).bind(outs).unpack(buf.data_ptr(),
+                                                                               plan.payload_bytes)
+                    torch.cuda.synchronize()
+                    for o, c in zip(outs, chunks):
+                        assert np.array_equal(tbytes(o), c), (nt, max_waves, align)
     finally:
         pkg.tune(tile_rows=0, threads=0, nontemporal=-1, max_waves=1 << 20)
 

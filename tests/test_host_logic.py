@@ -196,7 +196,7 @@ def seg_of(pkg, view, align=256, **tune):
         return plan.segments(), plan.launch_info()
     finally:
         if tune:
-            pkg.tune(tile_rows=0, gather_run_bytes=512, transpose=1)
+            pkg.tune(tile_rows=0, gather_run_bytes=1024, transpose=1)
 
 
 def test_compact_tensor_is_one_run(pkg):
@@ -275,18 +275,18 @@ def test_transposed_views_use_square_blocks(pkg):
 
 
 def test_negative_and_many_strides(pkg):
-    segs, _ = seg_of(pkg, tv(pkg, 0x20000, [4, 600], strides=[-1000, 1]))
-    assert segs[0]["stride_bytes"] == (-1000,) and segs[0]["mode"] == 1
+    segs, _ = seg_of(pkg, tv(pkg, 0x20000, [4, 1200], strides=[-2000, 1]))
+    assert segs[0]["stride_bytes"] == (-2000,) and segs[0]["mode"] == 1
     # 8 strided outer dims: the two outermost are peeled on the host
-    shape = [2, 3, 2, 2, 2, 2, 2, 2, 600]
-    strides, acc = [], 700
+    shape = [2, 3, 2, 2, 2, 2, 2, 2, 1200]
+    strides, acc = [], 1400
     for n in reversed(shape[:-1]):
         strides.insert(0, acc)
         acc *= n + 1                       # leave gaps so nothing merges
     strides.append(1)
     segs, _ = seg_of(pkg, tv(pkg, 0x100000, shape, strides=strides))
     assert len(segs) == 6 and all(s["ndim"] == 6 and s["mode"] == 1 for s in segs)
-    assert [s["offset"] for s in segs] == [i * 64 * 600 for i in range(6)]
+    assert [s["offset"] for s in segs] == [i * 64 * 1200 for i in range(6)]
     assert segs[1]["address"] - segs[0]["address"] == strides[1]
     assert segs[3]["address"] - segs[0]["address"] == strides[0]
 
