@@ -34,7 +34,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--rotate", type=int, default=4,
                     help="independent bundle copies cycled through by the steps (1 = cache resident)")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "transposed"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--tune", default="", help="comma separated key=value kernel tunables")
@@ -173,6 +173,26 @@ def make_c5_sets(h, count):
             workloads.pitched_views(dst.data_ptr(), spec), 256, (src, dst),
             check=lambda s=src, d=dst, c=spec.cols: bool(h.torch.equal(
                 s.view(h.torch.int16)[:, :, :c], d.view(h.torch.int16)[:, :, :c]))))
+    return sets
+
+
+def make_transposed_sets(h, count, seed=0, n=8, edge=4096):
+    """n transposed [edge, edge] bf16 matrices per bundle (x.t() views), scattered
+    back through the same transposition."""
+    import torch
+    from execution_ucx_amd import workloads
+    sets = []
+    for k in range(count):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed + k)
+        src = [torch.randint(-2 ** 15, 2 ** 15, (edge, edge), device="cuda", generator=g,
+                             dtype=torch.int16).view(torch.bfloat16) for _ in range(n)]
+        dst = [torch.zeros_like(x) for x in src]
+        sets.append(BundleSet(
+            h, workloads.views_of_torch([x.t() for x in src]),
+            workloads.views_of_torch([y.t() for y in dst]), 256, (src, dst),
+            check=lambda src=src, dst=dst: all(bool(torch.equal(x.view(torch.int16), y.view(torch.int16)))
+                                               for x, y in zip(src, dst))))
     return sets
 
 
@@ -361,6 +381,9 @@ def main():
     elif args.workload == "c4":
         sets = [make_c4_set(h)]
         name = "C4 strided KV-cache block gather/scatter, 512 blocks x 32 layers"
+    elif args.workload == "transposed":
+        sets = make_transposed_sets(h, max(1, min(args.rotate, 2)))
+        name = "8 transposed 4096 x 4096 bf16 matrices (x.t() views), 256 MiB"
     else:
         sets = make_c5_sets(h, max(1, min(args.rotate, 2)))
         name = "C5 chunk: 64 pitched 2-D views, 256 MiB"
@@ -434,6 +457,13 @@ def main():
         extras["c5_pitched_chunk"] = {"GBps": round(rate(c5[0].data_bytes, ms5, k5), 1),
                                       "payload_bytes_P": c5[0].data_bytes, "steps": k5}
         del c5
+        torch.cuda.empty_cache()
+        tr = make_transposed_sets(h, 2)
+        verify_set(h, tr[0])
+        mst = run_sets(h, tr, k5, 5)
+        extras["transposed_views"] = {"GBps": round(rate(tr[0].data_bytes, mst, k5), 1),
+                                      "payload_bytes_P": tr[0].data_bytes, "steps": k5}
+        del tr
         torch.cuda.empty_cache()
         extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["c5_streamed_8GiB"] = stream_c5(h)
