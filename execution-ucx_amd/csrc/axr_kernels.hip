@@ -266,15 +266,27 @@ template <> struct unit_of<16> { typedef u32x4 type; };
 
 template <uint32_t E>
 __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gbytes wr,
-                                               int64_t wr_pitch, lbytes lds, uint32_t lane) {
+                                               int64_t wr_pitch, lbytes lds, uint32_t lane,
+                                               bool nt_rd, bool nt_wr) {
   constexpr uint32_t T = kTransposeRowBytes / E, NK = T / 8, EV = kVecBytes / E;
   typedef typename unit_of<E>::type U;
   typedef U __attribute__((aligned(E < 4 ? E : 4))) lds_unit;
   const uint32_t r8 = lane >> 3, v = lane & 7;
   u32x4 x[NK];
+  // The cache hints are wave-uniform: one branch around each phase, not per access.
+  // The empty asm statements keep the two arms distinct: without them the optimizer
+  // merges the arms' identical accesses and the hint is lost.
+  if (nt_rd) {
+    asm volatile("");
 #pragma unroll
-  for (uint32_t k = 0; k < NK; ++k)
-    x[k] = load16<false>(rd + static_cast<int64_t>(k * 8 + r8) * rd_pitch + v * kVecBytes);
+    for (uint32_t k = 0; k < NK; ++k)
+      x[k] = load16<true>(rd + static_cast<int64_t>(k * 8 + r8) * rd_pitch + v * kVecBytes);
+    asm volatile("");
+  } else {
+#pragma unroll
+    for (uint32_t k = 0; k < NK; ++k)
+      x[k] = load16<false>(rd + static_cast<int64_t>(k * 8 + r8) * rd_pitch + v * kVecBytes);
+  }
 #pragma unroll
   for (uint32_t k = 0; k < NK; ++k) {
     AXR_LDS uint32_t* w =
@@ -285,6 +297,7 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
     w[3] = x[k].w;
   }
   __builtin_amdgcn_wave_barrier();
+  u32x4 out[NK];
 #pragma unroll
   for (uint32_t k = 0; k < NK; ++k) {
     const uint32_t c = k * 8 + r8;
@@ -292,9 +305,18 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
 #pragma unroll
     for (uint32_t i = 0; i < EV; ++i)
       e[i] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + (v * EV + i) * kTransposeLdsPitch + c * E);
-    u32x4 out;
-    __builtin_memcpy(&out, e, kVecBytes);
-    store16<false>(wr + static_cast<int64_t>(c) * wr_pitch + v * kVecBytes, out);
+    __builtin_memcpy(&out[k], e, kVecBytes);
+  }
+  if (nt_wr) {
+    asm volatile("");
+#pragma unroll
+    for (uint32_t k = 0; k < NK; ++k)
+      store16<true>(wr + static_cast<int64_t>(k * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
+    asm volatile("");
+  } else {
+#pragma unroll
+    for (uint32_t k = 0; k < NK; ++k)
+      store16<false>(wr + static_cast<int64_t>(k * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
   }
   __builtin_amdgcn_wave_barrier();
 }
@@ -390,17 +412,17 @@ __device__ __forceinline__ void transpose_edge(uint32_t E, gcbytes rd, int64_t r
 // nr elements (rows wr_pitch bytes apart).
 __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
                                                 int64_t wr_pitch, uint32_t nr, uint32_t nc,
-                                                lbytes lds, uint32_t lane) {
+                                                lbytes lds, uint32_t lane, bool nt_rd, bool nt_wr) {
   const uint32_t T = kTransposeRowBytes >> __builtin_ctz(E);
   const uint64_t bits = reinterpret_cast<uintptr_t>(rd) | static_cast<uint64_t>(rd_pitch) |
                         reinterpret_cast<uintptr_t>(wr) | static_cast<uint64_t>(wr_pitch);
   if (nr == T && nc == T && (bits & 15u) == 0) {
     switch (E) {
-      case 1: transpose_full<1>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
-      case 2: transpose_full<2>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
-      case 4: transpose_full<4>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
-      case 8: transpose_full<8>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
-      default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane); break;
+      case 1: transpose_full<1>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
+      case 2: transpose_full<2>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
+      case 4: transpose_full<4>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
+      case 8: transpose_full<8>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
+      default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
     }
   } else {
     transpose_edge(E, rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane);
@@ -410,7 +432,8 @@ __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t 
 // Tile q of a transposed segment: batch index (outer dims), then block (ia, ib).
 template <bool PACK>
 __device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, gbytes pay,
-                                               uint32_t q, lbytes lds, uint32_t lane) {
+                                               uint32_t q, lbytes lds, uint32_t lane,
+                                               uint32_t nt_bits) {
   const uint32_t E = dm->granule;
   const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
   const uint32_t T = kTransposeRowBytes >> es;
@@ -443,9 +466,11 @@ __device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, 
                (static_cast<uint64_t>(b0) << es);
   gbytes pp = pay + poff + static_cast<uint64_t>(b0) * pstride_b + (static_cast<uint64_t>(a0) << es);
   if constexpr (PACK) {
-    transpose_block(E, ten, stride_a, pp, static_cast<int64_t>(pstride_b), na, nb, lds, lane);
+    transpose_block(E, ten, stride_a, pp, static_cast<int64_t>(pstride_b), na, nb, lds, lane,
+                    (nt_bits & 1u) != 0, (nt_bits & 2u) != 0);
   } else {
-    transpose_block(E, pp, static_cast<int64_t>(pstride_b), ten, stride_a, nb, na, lds, lane);
+    transpose_block(E, pp, static_cast<int64_t>(pstride_b), ten, stride_a, nb, na, lds, lane,
+                    (nt_bits & 2u) != 0, (nt_bits & 1u) != 0);
   }
 }
 
@@ -453,7 +478,7 @@ template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
     const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
     uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
-    uint32_t lds_per_wave) {
+    uint32_t lds_per_wave, uint32_t nt_bits) {
   // Scalar arguments (not one struct) so that the compiler can preload them
   // into SGPRs at dispatch instead of fetching the kernarg segment first.
   KernelArgs a;
@@ -541,7 +566,7 @@ __global__ __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkg
         if (dm->mode == kModeTranspose) {
           extern __shared__ uint8_t lds_slices[];   // lds_per_wave bytes for each wavefront
           lbytes lds = (lbytes)lds_slices + (threadIdx.x >> 6) * lds_per_wave;
-          transpose_tile<PACK>(seg_ptr, dm, pay, q, lds, lane);
+          transpose_tile<PACK>(seg_ptr, dm, pay, q, lds, lane, nt_bits);
         } else {
           element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
         }
@@ -610,19 +635,19 @@ template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
   const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * (cfg.threads / kWaveLanes) : 0u;
-#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave, cfg.nontemporal
 #define AXR_LAUNCH(NTT, NTP, EL) \
   hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, lds_bytes, stream, AXR_ARGS)
-  if (cfg.elements) {
-    // strided tensors with short runs are present: the general kernel
-    AXR_LAUNCH(false, false, true);
-  } else {
-    switch (cfg.nontemporal) {   // bit 0: tensor side, bit 1: payload side
-      case 0: AXR_LAUNCH(false, false, false); break;
-      case 1: AXR_LAUNCH(true, false, false); break;
-      case 2: AXR_LAUNCH(false, true, false); break;
-      default: AXR_LAUNCH(true, true, false); break;
-    }
+  // cfg.elements: strided tensors with short runs or transpositions are present
+  switch ((cfg.elements ? 4u : 0u) | (cfg.nontemporal & 3u)) {   // bit 0: tensor side, bit 1: payload side
+    case 0: AXR_LAUNCH(false, false, false); break;
+    case 1: AXR_LAUNCH(true, false, false); break;
+    case 2: AXR_LAUNCH(false, true, false); break;
+    case 3: AXR_LAUNCH(true, true, false); break;
+    case 4: AXR_LAUNCH(false, false, true); break;
+    case 5: AXR_LAUNCH(true, false, true); break;
+    case 6: AXR_LAUNCH(false, true, true); break;
+    default: AXR_LAUNCH(true, true, true); break;
   }
 #undef AXR_LAUNCH
 #undef AXR_ARGS
