@@ -53,6 +53,7 @@ constexpr uint32_t kModeTranspose = 2;  // tile is a square block transposed thr
 constexpr uint32_t kTransposeRowBytes = 128;
 constexpr uint32_t kTransposeLdsPitch = kTransposeRowBytes + 4;   // one dword of padding per row
 constexpr uint32_t kMaxBatchDims = 4;
+constexpr uint32_t kMinElementTileBytes = 8192;   // element-mode work unit (measured: 8 KiB beats 2, 4 and 16)
 
 struct Dims {             // 160 bytes, one per strided segment
   uint32_t mode;
@@ -119,7 +120,9 @@ struct Tunables {
   // last-level cache when the consumer (unpack, or the transport's copy) reads it.
   int64_t nontemporal = -1;
   int64_t payload_cache_bytes = 256ll << 20;
-  int64_t gather_run_bytes = 1024; // strided runs shorter than this use element mode (measured crossover)
+  // Strided runs shorter than this use element mode when they are multiples of
+  // 16 bytes, shorter than an eighth of it otherwise (measured crossovers).
+  int64_t gather_run_bytes = 2048;
   int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
   int64_t transpose = 1;          // move transposed views as square blocks through LDS
 };

@@ -163,6 +163,37 @@ __device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
   return off;
 }
 
+// Moves the ng granules (type T) of one element-mode tile, U per lane at a
+// time: addresses first, then all loads, then all stores, so a lane keeps U
+// accesses in flight instead of a load-wait-store chain per granule.
+template <bool PACK, typename T, uint32_t U, typename DECODE>
+__device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32_t ng,
+                                              uint32_t lane, DECODE decode) {
+  typedef T __attribute__((aligned(1))) loose;   // no alignment promise on either side
+  for (uint32_t e0 = lane; e0 < ng; e0 += U * kWaveLanes) {
+    gbytes tp[U], pp[U];
+    T val[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t e = e0 + u * kWaveLanes;
+      const uint32_t ec = e < ng ? e : ng - 1u;   // slots past the end repeat the last granule's load
+      tp[u] = tbase + decode(ec);
+      pp[u] = pbase + static_cast<uint64_t>(ec) * sizeof(T);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u)
+      val[u] = *reinterpret_cast<const AXR_GLOBAL loose*>(PACK ? tp[u] : pp[u]);
+    if constexpr (sizeof(T) == 16) {
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u) asm volatile("" : "+v"(val[u])::"memory");
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      if (e0 + u * kWaveLanes < ng) *reinterpret_cast<AXR_GLOBAL loose*>(PACK ? pp[u] : tp[u]) = val[u];
+    }
+  }
+}
+
 // Element mode: the tile covers kTile packed bytes of a strided segment whose
 // contiguous runs are short; each lane decodes the tensor address of its own
 // granules.  Only kernels instantiated with ELEMENTS carry this code, so the
@@ -174,7 +205,8 @@ __device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
 template <bool PACK, uint32_t ROWS>
 __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_bytes, dims_table dm,
                                           gbytes pay, uint32_t q, uint32_t lane) {
-  constexpr uint32_t kTile = ROWS * kRowBytes;
+  // element-mode tiles are at least 8 KiB: the per-tile decode is amortised over more bytes
+  constexpr uint32_t kTile = ROWS * kRowBytes < kMinElementTileBytes ? kMinElementTileBytes : ROWS * kRowBytes;
   const uint32_t g = dm->granule;
   const uint32_t gs = static_cast<uint32_t>(__builtin_ctz(g));
   const uint32_t gpr = static_cast<uint32_t>(run_bytes >> gs);
@@ -212,7 +244,8 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   const uint32_t gpr_magic = 0xffffffffu / gpr + 1u;
   gbytes tbase = as_global(seg_ptr) + base;
   gbytes pbase = pay + b0;
-  for (uint32_t e = lane; e < ng; e += kWaveLanes) {
+  // tensor-side byte offset (relative to the tile's first run) of granule e of the tile
+  auto decode = [&](uint32_t e) -> int64_t {
     uint32_t w = w0 + e;
     // w < gpr + tile / g: for gpr <= 2^15, w * gpr < 2^32 and the multiply-high quotient is exact
     uint32_t carry = gpr == 1 ? w : (gpr <= 32768u ? __umulhi(w, gpr_magic) : w / gpr);
@@ -233,12 +266,16 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
         carry = c;
       }
     }
-    gbytes pp = pbase + (static_cast<uint64_t>(e) << gs);
-    if constexpr (PACK) {
-      move_granule_dyn(g, tbase + toff, pp);
-    } else {
-      move_granule_dyn(g, pp, tbase + toff);
-    }
+    return toff;
+  };
+  // Accesses per lane and round.  16-byte granules measured fastest one at a time
+  // (a 2 KiB tile is two rounds); narrow granules gain from four in flight.
+  switch (g) {
+    case 16: element_moves<PACK, u32x4, 1>(tbase, pbase, ng, lane, decode); break;
+    case 8: element_moves<PACK, uint64_t, 2>(tbase, pbase, ng, lane, decode); break;
+    case 4: element_moves<PACK, uint32_t, 4>(tbase, pbase, ng, lane, decode); break;
+    case 2: element_moves<PACK, uint16_t, 4>(tbase, pbase, ng, lane, decode); break;
+    default: element_moves<PACK, uint8_t, 4>(tbase, pbase, ng, lane, decode); break;
   }
 }
 
@@ -271,52 +308,60 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
   constexpr uint32_t T = kTransposeRowBytes / E, NK = T / 8, EV = kVecBytes / E;
   typedef typename unit_of<E>::type U;
   typedef U __attribute__((aligned(E < 4 ? E : 4))) lds_unit;
+  // at most eight vectors per lane in flight: a block of bytes (128 rows) moves in two halves
+  constexpr uint32_t B = NK < 8 ? NK : 8;
   const uint32_t r8 = lane >> 3, v = lane & 7;
-  u32x4 x[NK];
-  // The cache hints are wave-uniform: one branch around each phase, not per access.
+  // The cache hints are wave-uniform: one branch around each batch, not per access.
   // The empty asm statements keep the two arms distinct: without them the optimizer
   // merges the arms' identical accesses and the hint is lost.
-  if (nt_rd) {
-    asm volatile("");
 #pragma unroll
-    for (uint32_t k = 0; k < NK; ++k)
-      x[k] = load16<true>(rd + static_cast<int64_t>(k * 8 + r8) * rd_pitch + v * kVecBytes);
-    asm volatile("");
-  } else {
+  for (uint32_t kb = 0; kb < NK; kb += B) {
+    u32x4 x[B];
+    if (nt_rd) {
+      asm volatile("");
 #pragma unroll
-    for (uint32_t k = 0; k < NK; ++k)
-      x[k] = load16<false>(rd + static_cast<int64_t>(k * 8 + r8) * rd_pitch + v * kVecBytes);
-  }
+      for (uint32_t k = 0; k < B; ++k)
+        x[k] = load16<true>(rd + static_cast<int64_t>((kb + k) * 8 + r8) * rd_pitch + v * kVecBytes);
+      asm volatile("");
+    } else {
 #pragma unroll
-  for (uint32_t k = 0; k < NK; ++k) {
-    AXR_LDS uint32_t* w =
-        reinterpret_cast<AXR_LDS uint32_t*>(lds + (k * 8 + r8) * kTransposeLdsPitch + v * kVecBytes);
-    w[0] = x[k].x;
-    w[1] = x[k].y;
-    w[2] = x[k].z;
-    w[3] = x[k].w;
+      for (uint32_t k = 0; k < B; ++k)
+        x[k] = load16<false>(rd + static_cast<int64_t>((kb + k) * 8 + r8) * rd_pitch + v * kVecBytes);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < B; ++k) {
+      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(
+          lds + ((kb + k) * 8 + r8) * kTransposeLdsPitch + v * kVecBytes);
+      w[0] = x[k].x;
+      w[1] = x[k].y;
+      w[2] = x[k].z;
+      w[3] = x[k].w;
+    }
   }
   __builtin_amdgcn_wave_barrier();
-  u32x4 out[NK];
 #pragma unroll
-  for (uint32_t k = 0; k < NK; ++k) {
-    const uint32_t c = k * 8 + r8;
-    U e[EV];
+  for (uint32_t kb = 0; kb < NK; kb += B) {
+    u32x4 out[B];
 #pragma unroll
-    for (uint32_t i = 0; i < EV; ++i)
-      e[i] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + (v * EV + i) * kTransposeLdsPitch + c * E);
-    __builtin_memcpy(&out[k], e, kVecBytes);
-  }
-  if (nt_wr) {
-    asm volatile("");
+    for (uint32_t k = 0; k < B; ++k) {
+      const uint32_t c = (kb + k) * 8 + r8;
+      U e[EV];
 #pragma unroll
-    for (uint32_t k = 0; k < NK; ++k)
-      store16<true>(wr + static_cast<int64_t>(k * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
-    asm volatile("");
-  } else {
+      for (uint32_t i = 0; i < EV; ++i)
+        e[i] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + (v * EV + i) * kTransposeLdsPitch + c * E);
+      __builtin_memcpy(&out[k], e, kVecBytes);
+    }
+    if (nt_wr) {
+      asm volatile("");
 #pragma unroll
-    for (uint32_t k = 0; k < NK; ++k)
-      store16<false>(wr + static_cast<int64_t>(k * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
+      for (uint32_t k = 0; k < B; ++k)
+        store16<true>(wr + static_cast<int64_t>((kb + k) * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
+      asm volatile("");
+    } else {
+#pragma unroll
+      for (uint32_t k = 0; k < B; ++k)
+        store16<false>(wr + static_cast<int64_t>((kb + k) * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
+    }
   }
   __builtin_amdgcn_wave_barrier();
 }

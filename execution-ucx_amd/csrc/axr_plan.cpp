@@ -256,6 +256,21 @@ void collapse(const TensorRec& t, const int64_t* shape, const int64_t* strides, 
   }
 }
 
+// Largest power of two up to 16 that divides the run length.
+uint32_t granule_of(uint64_t run_bytes) {
+  uint32_t g = 16;
+  while (g > 1 && (run_bytes % g) != 0) g >>= 1;
+  return g;
+}
+
+// Runs shorter than this move in element mode.  With 16-byte granules element
+// mode matches run tiles up to about 2 KiB runs; narrower granules move fewer
+// bytes per access and lose to the (length-agnostic) run-tile copy much earlier.
+uint64_t element_mode_limit(uint64_t run_bytes) {
+  const uint64_t limit = static_cast<uint64_t>(tunables().gather_run_bytes);
+  return granule_of(run_bytes) == 16 ? limit : (limit + 7) / 8;
+}
+
 struct Builder {
   axr_plan* p;
   uint32_t tile_bytes;
@@ -361,7 +376,7 @@ struct Builder {
         return fail(AXR_ERR_UNSUPPORTED, "transposed tensor has too many blocks");
       ntile = batches * per_batch;
       p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, t * kTransposeLdsPitch);
-    } else if (run_bytes >= static_cast<uint64_t>(tunables().gather_run_bytes)) {
+    } else if (run_bytes >= element_mode_limit(run_bytes)) {
       dm.mode = kModeRunTiles;
       const uint64_t tpr = (run_bytes + tile_bytes - 1) / tile_bytes;
       if (tpr > 0xffffffffull || runs > 0xffffffffull)
@@ -375,10 +390,9 @@ struct Builder {
       dm.mode = kModeElements;
       // the kernel's per-granule index arithmetic is 32-bit
       if (runs > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "strided tensor has too many runs");
-      uint32_t g = 16;
-      while (g > 1 && (run_bytes % g) != 0) g >>= 1;
-      dm.granule = g;
-      ntile = (nbytes + tile_bytes - 1) / tile_bytes;
+      dm.granule = granule_of(run_bytes);
+      const uint64_t element_tile = std::max<uint32_t>(tile_bytes, kMinElementTileBytes);
+      ntile = (nbytes + element_tile - 1) / element_tile;
     }
     if (p->dims.size() + 1 >= kSegFillOnly)
       return fail(AXR_ERR_UNSUPPORTED, "too many strided tensors in one bundle");

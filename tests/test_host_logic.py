@@ -196,7 +196,7 @@ def seg_of(pkg, view, align=256, **tune):
         return plan.segments(), plan.launch_info()
     finally:
         if tune:
-            pkg.tune(tile_rows=0, gather_run_bytes=1024, transpose=1)
+            pkg.tune(tile_rows=0, gather_run_bytes=2048, transpose=1)
 
 
 def test_compact_tensor_is_one_run(pkg):
@@ -242,11 +242,21 @@ def test_short_runs_use_element_mode(pkg):
     assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 24, 8)
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 3], strides=[7, 2], dtype=(2, 96, 1)))
     assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 12, 4)
-    # the threshold is a tunable
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=200)
+    # the threshold is a tunable: runs that are multiples of 16 bytes switch at the
+    # tunable itself, others at an eighth of it
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 304], strides=[1000, 1]), gather_run_bytes=304)
     assert segs[0]["mode"] == 1
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=400)
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 304], strides=[1000, 1]), gather_run_bytes=305)
+    assert segs[0]["mode"] == 2 and segs[0]["granule"] == 16
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2400)
+    assert segs[0]["mode"] == 1
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2408)
     assert segs[0]["mode"] == 2 and segs[0]["granule"] == 4
+    # defaults: 2 KiB for 16-byte multiples, 256 B otherwise
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 2032], strides=[4000, 1]))[0][0]["mode"] == 2
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 2048], strides=[4000, 1]))[0][0]["mode"] == 1
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 252], strides=[4000, 1]))[0][0]["mode"] == 2
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 260], strides=[4000, 1]))[0][0]["mode"] == 1
 
 
 def test_transposed_views_use_square_blocks(pkg):
@@ -275,18 +285,18 @@ def test_transposed_views_use_square_blocks(pkg):
 
 
 def test_negative_and_many_strides(pkg):
-    segs, _ = seg_of(pkg, tv(pkg, 0x20000, [4, 1200], strides=[-2000, 1]))
-    assert segs[0]["stride_bytes"] == (-2000,) and segs[0]["mode"] == 1
+    segs, _ = seg_of(pkg, tv(pkg, 0x20000, [4, 2400], strides=[-4000, 1]))
+    assert segs[0]["stride_bytes"] == (-4000,) and segs[0]["mode"] == 1
     # 8 strided outer dims: the two outermost are peeled on the host
-    shape = [2, 3, 2, 2, 2, 2, 2, 2, 1200]
-    strides, acc = [], 1400
+    shape = [2, 3, 2, 2, 2, 2, 2, 2, 2400]
+    strides, acc = [], 2800
     for n in reversed(shape[:-1]):
         strides.insert(0, acc)
         acc *= n + 1                       # leave gaps so nothing merges
     strides.append(1)
     segs, _ = seg_of(pkg, tv(pkg, 0x100000, shape, strides=strides))
     assert len(segs) == 6 and all(s["ndim"] == 6 and s["mode"] == 1 for s in segs)
-    assert [s["offset"] for s in segs] == [i * 64 * 1200 for i in range(6)]
+    assert [s["offset"] for s in segs] == [i * 64 * 2400 for i in range(6)]
     assert segs[1]["address"] - segs[0]["address"] == strides[1]
     assert segs[3]["address"] - segs[0]["address"] == strides[0]
 
