@@ -136,7 +136,7 @@ class LaunchInfo(C.Structure):
         ("segments", C.c_uint32),
         ("table_bytes", C.c_uint32),
         ("host_copies", C.c_uint32),
-        ("reserved", C.c_uint32),
+        ("host_chunks", C.c_uint32),
     ]
 
 

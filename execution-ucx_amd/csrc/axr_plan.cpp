@@ -52,6 +52,19 @@ struct HostCopy {
   uint64_t bytes;
 };
 
+// Host tensors travel through pinned staging blocks: one device copy per chunk
+// of neighbouring pieces instead of one pageable copy per piece.
+constexpr size_t kStageBytes = 8u << 20;
+struct HostChunk {
+  uint32_t first, count;     // range of host_copies
+  uint64_t begin, end;       // payload byte range the chunk spans
+};
+struct HostStage {
+  TableBlock block;
+  hipEvent_t ready = nullptr;   // recorded after the device copy that uses the block
+  bool pending = false;
+};
+
 template <typename T>
 T get(const uint8_t* p) {
   T x;
@@ -107,6 +120,8 @@ struct axr_plan {
   std::vector<uint32_t> seg_tensor;  // tensor index per segment (inspection)
   std::vector<HostCopy> host_copies;
   std::vector<uint32_t> host_copy_tensor;
+  std::vector<HostChunk> host_chunks;
+  HostStage stage[2];
   bool overlapping_dst = false;      // some tensor has a zero stride over an extent > 1
   uint32_t ntiles = 0;
   LaunchConfig cfg;
@@ -186,6 +201,7 @@ void invalidate_tables(axr_plan* p) {
   p->seg_tensor.clear();
   p->host_copies.clear();
   p->host_copy_tensor.clear();
+  p->host_chunks.clear();
   p->overlapping_dst = false;
   p->ntiles = 0;
   p->cfg.lds_per_wave = 0;
@@ -404,10 +420,13 @@ struct Builder {
   int add_host(uint32_t tensor, uint64_t ptr, uint64_t off, const uint64_t* ext,
                const int64_t* str, size_t nd, uint64_t run_bytes) {
     if (nd == 0) {
-      if (p->host_copies.size() >= (1u << 20))
-        return fail(AXR_ERR_UNSUPPORTED, "host tensor needs more than 2^20 copies");
-      p->host_copies.push_back({ptr, off, run_bytes});
-      p->host_copy_tensor.push_back(tensor);
+      // pieces of at most one staging block
+      for (uint64_t done = 0; done < run_bytes; done += kStageBytes) {
+        if (p->host_copies.size() >= (1u << 20))
+          return fail(AXR_ERR_UNSUPPORTED, "host tensor needs more than 2^20 copies");
+        p->host_copies.push_back({ptr + done, off + done, std::min<uint64_t>(kStageBytes, run_bytes - done)});
+        p->host_copy_tensor.push_back(tensor);
+      }
       return AXR_OK;
     }
     uint64_t inner = run_bytes;
@@ -489,6 +508,21 @@ int build_tables(axr_plan* p) {
       return fail(AXR_ERR_UNSUPPORTED,
                   "Unsupported memory type: DLPack device " + std::to_string(t.device_type));
     }
+  }
+  // Group neighbouring host pieces (in payload order, at most an alignment gap
+  // apart) into chunks that fit one staging block.
+  for (uint32_t i = 0; i < p->host_copies.size(); ++i) {
+    const HostCopy& hc = p->host_copies[i];
+    if (!p->host_chunks.empty()) {
+      HostChunk& c = p->host_chunks.back();
+      if (hc.offset >= c.end && hc.offset - c.end < kMaxAlign &&
+          hc.offset + hc.bytes - c.begin <= kStageBytes) {
+        c.end = hc.offset + hc.bytes;
+        ++c.count;
+        continue;
+      }
+    }
+    p->host_chunks.push_back({i, 1, hc.offset, hc.offset + hc.bytes});
   }
   p->ntiles = static_cast<uint32_t>(b.tiles);
   Seg sentinel;
@@ -584,6 +618,81 @@ int ensure_uploaded(axr_plan* p, hipStream_t stream) {
   return AXR_OK;
 }
 
+int stage_ready(HostStage* st) {   // block until the staging block's last device copy is done
+  if (!st->pending) return AXR_OK;
+  st->pending = false;
+  return check_hip(hipEventSynchronize(st->ready), "hipEventSynchronize(staging)");
+}
+
+int stage_acquire(HostStage* st) {
+  if (!st->block.host) {
+    int rc = table_block_acquire(kStageBytes, &st->block);
+    if (rc) return rc;
+  }
+  if (!st->ready) {
+    int rc = check_hip(hipEventCreateWithFlags(&st->ready, hipEventDisableTiming), "hipEventCreate");
+    if (rc) return rc;
+  }
+  return stage_ready(st);
+}
+
+// kDLCPU tensors.  Pack: the pieces of a chunk are copied into a pinned block on
+// the calling thread (gaps zeroed: they are alignment padding or are rewritten by
+// the kernel that follows on the stream), then one asynchronous device copy moves
+// the chunk.  Unpack: one device copy per chunk into a pinned block; while the
+// next chunk is in flight the calling thread copies the previous one out, so the
+// call returns when the host tensors hold their data (as a copy into pageable
+// memory does).  Two blocks alternate.
+int move_host_tensors(axr_plan* p, bool pack, uint8_t* payload, hipStream_t stream) {
+  const size_t nchunks = p->host_chunks.size();
+  auto pieces_out = [p](const HostChunk& c, const uint8_t* staged) {
+    for (uint32_t i = c.first; i < c.first + c.count; ++i) {
+      const HostCopy& hc = p->host_copies[i];
+      std::memcpy(reinterpret_cast<void*>(hc.host), staged + (hc.offset - c.begin), hc.bytes);
+    }
+  };
+  for (size_t k = 0; k < nchunks; ++k) {
+    const HostChunk& c = p->host_chunks[k];
+    HostStage* st = &p->stage[k & 1];
+    if (!pack && k >= 2) {   // the block still holds chunk k - 2
+      int rc = stage_ready(st);
+      if (rc) return rc;
+      pieces_out(p->host_chunks[k - 2], static_cast<const uint8_t*>(st->block.host));
+    }
+    int rc = stage_acquire(st);
+    if (rc) return rc;
+    uint8_t* staged = static_cast<uint8_t*>(st->block.host);
+    const size_t span = static_cast<size_t>(c.end - c.begin);
+    if (pack) {
+      uint64_t at = c.begin;
+      for (uint32_t i = c.first; i < c.first + c.count; ++i) {
+        const HostCopy& hc = p->host_copies[i];
+        if (hc.offset > at) std::memset(staged + (at - c.begin), 0, hc.offset - at);
+        std::memcpy(staged + (hc.offset - c.begin), reinterpret_cast<const void*>(hc.host), hc.bytes);
+        at = hc.offset + hc.bytes;
+      }
+      rc = check_hip(hipMemcpyAsync(payload + c.begin, staged, span, hipMemcpyDefault, stream),
+                     "hipMemcpyAsync(host tensors -> payload)");
+    } else {
+      rc = check_hip(hipMemcpyAsync(staged, payload + c.begin, span, hipMemcpyDefault, stream),
+                     "hipMemcpyAsync(payload -> host tensors)");
+    }
+    if (rc) return rc;
+    rc = check_hip(hipEventRecord(st->ready, stream), "hipEventRecord(staging)");
+    if (rc) return rc;
+    st->pending = true;
+  }
+  if (!pack) {
+    for (size_t k = nchunks >= 2 ? nchunks - 2 : 0; k < nchunks; ++k) {
+      HostStage* st = &p->stage[k & 1];
+      int rc = stage_ready(st);
+      if (rc) return rc;
+      pieces_out(p->host_chunks[k], static_cast<const uint8_t*>(st->block.host));
+    }
+  }
+  return AXR_OK;
+}
+
 int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* stream_) {
   if (!p) return fail(AXR_ERR_INVALID, "null plan");
   if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
@@ -596,13 +705,10 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   if (!pack && p->overlapping_dst)
     return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  for (const HostCopy& hc : p->host_copies) {
-    void* dev = static_cast<uint8_t*>(payload) + hc.offset;
-    void* host = reinterpret_cast<void*>(hc.host);
-    rc = pack ? check_hip(hipMemcpyAsync(dev, host, hc.bytes, hipMemcpyDefault, stream),
-                          "hipMemcpyAsync(host tensor -> payload)")
-              : check_hip(hipMemcpyAsync(host, dev, hc.bytes, hipMemcpyDefault, stream),
-                          "hipMemcpyAsync(payload -> host tensor)");
+  if (!p->host_chunks.empty()) {
+    rc = move_host_tensors(p, pack, static_cast<uint8_t*>(payload), stream);
+    if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+      p->busy_streams.push_back(stream);
     if (rc) return rc;
   }
   if (p->ntiles == 0) return AXR_OK;
@@ -693,6 +799,10 @@ int axr_plan_free(axr_plan_t* plan) {
   if (plan->uploaded && plan->upload_event) (void)hipEventSynchronize(plan->upload_event);
   table_block_release(&plan->block);
   if (plan->upload_event) (void)hipEventDestroy(plan->upload_event);
+  for (HostStage& st : plan->stage) {
+    table_block_release(&st.block);
+    if (st.ready) (void)hipEventDestroy(st.ready);
+  }
   delete plan;
   return AXR_OK;
 }
@@ -892,7 +1002,7 @@ int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
   info->segments = static_cast<uint32_t>(plan->segs.size() - 1);
   info->table_bytes = static_cast<uint32_t>(plan->table_bytes);
   info->host_copies = static_cast<uint32_t>(plan->host_copies.size());
-  info->reserved = 0;
+  info->host_chunks = static_cast<uint32_t>(plan->host_chunks.size());
   return AXR_OK;
 }
 

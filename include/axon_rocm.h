@@ -220,7 +220,10 @@ typedef struct axr_plan axr_plan_t;
  * they are packed as their C-order element sequence; the reference would
  * ship the first nbytes of storage instead (dlpack_helpers.cpp:776-780).
  * Every tensor must be device-accessible (kDLROCM / kDLROCMHost) or kDLCPU;
- * kDLCPU tensors are moved with hipMemcpyAsync, one copy per contiguous run.
+ * kDLCPU tensors travel through pinned staging blocks of 8 MiB: neighbouring
+ * pieces share one device copy per block; axr_pack returns once the host
+ * tensors have been read, axr_unpack once they hold their data (the device
+ * tensors of the same bundle still complete asynchronously on the stream).
  * The plan copies shapes and strides; `tensors` may be freed on return. */
 AXR_API int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align,
                             uint32_t flags, axr_plan_t** plan);
@@ -279,8 +282,8 @@ typedef struct axr_launch_info {
   uint32_t tile_bytes;
   uint32_t segments;       /* device segment-table entries                    */
   uint32_t table_bytes;    /* device table size                               */
-  uint32_t host_copies;    /* hipMemcpyAsync calls used for kDLCPU tensors     */
-  uint32_t reserved;
+  uint32_t host_copies;    /* contiguous pieces of kDLCPU tensors              */
+  uint32_t host_chunks;    /* device copies that move them (pinned staging)    */
 } axr_launch_info_t;
 AXR_API int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info);
 

@@ -130,11 +130,61 @@ def test_c1_host_bundle(pkg, orc, gpu):
     assert np.array_equal(got, want)
     outs = [np.zeros_like(s) for s in srcs]
     rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
-    assert rplan.launch_info()["host_copies"] == 64
+    info = rplan.launch_info()
+    assert info["host_copies"] == 64 and info["host_chunks"] == 1    # one staged device copy
     rplan.unpack(buf.data_ptr(), plan.payload_bytes)
     torch.cuda.synchronize()
     for a, b in zip(srcs, outs):
         assert a.tobytes() == b.tobytes()
+
+
+def test_host_tensors_staged_with_device_tensors(pkg, orc, gpu):
+    """Host (kDLCPU) tensors interleaved with device tensors: neighbouring host
+    pieces share one staged device copy, a 20 MiB host tensor is cut over several
+    staging blocks, strided host views move piece by piece; the plan is used twice
+    so that the staging blocks are reused while their last copy may be in flight."""
+    import torch
+    rng = np.random.default_rng(11)
+    big = rng.integers(0, 256, size=20 * (1 << 20) + 12345, dtype=np.uint8)
+    mat = rng.integers(0, 2 ** 31, size=(64, 300), dtype=np.int32)
+    small = [rng.integers(0, 256, size=n, dtype=np.uint8) for n in (1, 255, 256, 70000)]
+    dev = [rand_bytes_tensor(rng, n, gpu) for n in (4096, 100, 3 << 20)]
+    tensors = [small[0], dev[0], small[1], small[2], big, dev[1], mat[::2, 10:250], small[3], dev[2]]
+
+    def chunk_of(t):
+        return tbytes(t) if isinstance(t, torch.Tensor) else np.ascontiguousarray(t).view(np.uint8).reshape(-1)
+
+    chunks = [chunk_of(t) for t in tensors]
+    for align in (256, 1):
+        plan = pkg.BundlePlan.create(tensors, align=align)
+        info = plan.launch_info()
+        assert info["host_copies"] == 4 + 3 + 32                 # 20 MiB in three pieces, 32 matrix rows
+        assert 3 <= info["host_chunks"] < info["host_copies"]
+        n = plan.payload_bytes
+        for repeat in range(2):
+            buf = device_bytes(n + 64, gpu)
+            plan.pack(buf.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            host = buf.cpu().numpy()
+            assert np.array_equal(host[:n], orc.pack(chunks, align)), (align, repeat)
+            assert (host[n:] == POISON).all()
+        outs = []
+        for t in tensors:
+            if isinstance(t, torch.Tensor):
+                outs.append(torch.zeros_like(t))
+            else:
+                outs.append(np.zeros(t.shape, dtype=t.dtype))
+        rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+        for repeat in range(2):
+            for o in outs:
+                if isinstance(o, torch.Tensor):
+                    o.zero_()
+                else:
+                    o[...] = 0
+            rplan.unpack(buf.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            for o, c in zip(outs, chunks):
+                assert np.array_equal(chunk_of(o), c), (align, repeat)
 
 
 # ------------------------------------------------------------------ config 2: mixed small tensors

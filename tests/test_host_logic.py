@@ -315,7 +315,7 @@ def test_pads_fill_segments_and_host_copies(pkg):
     assert dev[2]["offset"] == 512 + 30
     assert [(s["address"], s["offset"], s["nbytes"]) for s in host] == [
         (0x40000, 512, 10), (0x40000 + 20, 522, 10), (0x40000 + 40, 532, 10)]
-    assert plan.launch_info()["host_copies"] == 3
+    assert plan.launch_info()["host_copies"] == 3 and plan.launch_info()["host_chunks"] == 1
     assert plan.payload_bytes == 768 + 7
 
 
