@@ -379,6 +379,46 @@ def test_strided_gather_scatter_random(pkg, orc, gpu, dtype_name):
             assert len(metas) == len(views) - 1
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_strided_views_larger_extents(pkg, orc, gpu, seed):
+    """Random slices and permutations of 2- to 4-d parents with extents up to 90:
+    large enough for transposed blocks with batch dimensions, ragged edges and
+    misaligned bases, mixed in one bundle with element mode and run tiles."""
+    import torch
+    rng = np.random.default_rng(1000 + seed)
+    names = ["uint8", "int16", "float32", "float64", "complex128"]
+    for trial in range(10):
+        cases = []
+        for _ in range(int(rng.integers(1, 5))):
+            dt = getattr(torch, names[int(rng.integers(0, len(names)))])
+            item = torch.empty((), dtype=dt).element_size()
+            ndim = int(rng.integers(2, 5))
+            shape = [int(x) for x in rng.integers(1, 91 if ndim < 4 else 25, size=ndim)]
+            parent = rand_bytes_tensor(rng, int(np.prod(shape)) * item, gpu).view(dt).reshape(shape)
+            cases.append((parent, random_torch_view(rng, parent, ndim), item))
+        views = [v for _, v, _ in cases]
+        chunks = []
+        for parent, v, item in cases:
+            host_parent = parent.reshape(-1).view(torch.uint8).cpu().numpy()
+            chunks.append(orc.gather_strided(host_parent, v.data_ptr() - parent.data_ptr(),
+                                             tuple(v.shape), tuple(v.stride()), item))
+        align = int(rng.choice([1, 16, 256]))
+        got, plan, buf = run_pack(pkg, views, align, gpu)
+        assert np.array_equal(got, orc.pack(chunks, align)), (seed, trial)
+        twins, tviews = [], []
+        for parent, v, item in cases:
+            twin = device_bytes(parent.numel() * item, gpu, fill=0x77).view(parent.dtype).reshape(parent.shape)
+            twins.append(twin)
+            tviews.append(twin.as_strided(v.shape, v.stride(), v.storage_offset()))
+        pkg.BundlePlan.from_header(plan.header).bind(tviews).unpack(buf.data_ptr(), plan.payload_bytes)
+        torch.cuda.synchronize()
+        for (parent, v, item), twin, c in zip(cases, twins, chunks):
+            e = np.full(parent.numel() * item, 0x77, np.uint8)
+            orc.scatter_strided(c, e, v.data_ptr() - parent.data_ptr(), tuple(v.shape),
+                                tuple(v.stride()), item)
+            assert np.array_equal(twin.reshape(-1).view(torch.uint8).cpu().numpy(), e), (seed, trial)
+
+
 @pytest.mark.parametrize("dtype_name", ["uint8", "bfloat16", "float32", "float64", "complex128"])
 def test_transposed_views(pkg, orc, gpu, dtype_name):
     """Views whose packed-inner dimension is strided while another dimension is
