@@ -1039,12 +1039,25 @@ int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity
         o.shape[d] = dm.shape[kMaxOuterDims - dm.ndim + d];
         o.stride_bytes[d] = dm.stride[kMaxOuterDims - dm.ndim + d];
       }
-      if (dm.mode == kModeTranspose) {   // batch dims, then B (contiguous in the tensor), then A
-        o.shape[o.ndim] = dm.ext_b;
-        o.stride_bytes[o.ndim] = dm.granule;
-        o.shape[o.ndim + 1] = dm.ext_a;
-        o.stride_bytes[o.ndim + 1] = dm.stride_a;
-        o.ndim += 2;
+      if (dm.mode == kModeTranspose) {
+        // all dims in packed (C) order: the batch dims with B, the dim that is
+        // contiguous in the tensor, at its place among them, then A
+        struct Dim { uint32_t extent; int64_t stride; uint64_t packed; };
+        Dim all[kMaxOuterDims];
+        uint32_t n = 0;
+        for (uint32_t d = 0; d < dm.ndim; ++d) {
+          const uint32_t slot = kMaxBatchDims - dm.ndim + d;
+          all[n++] = {dm.shape[kMaxOuterDims - kMaxBatchDims + slot],
+                      dm.stride[kMaxOuterDims - kMaxBatchDims + slot], dm.pstride[slot]};
+        }
+        all[n++] = {dm.ext_b, static_cast<int64_t>(dm.granule), dm.pstride_b};
+        std::sort(all, all + n, [](const Dim& x, const Dim& y) { return x.packed > y.packed; });
+        all[n++] = {dm.ext_a, dm.stride_a, dm.granule};
+        for (uint32_t d = 0; d < n; ++d) {
+          o.shape[d] = all[d].extent;
+          o.stride_bytes[d] = all[d].stride;
+        }
+        o.ndim = n;
       }
     }
   }

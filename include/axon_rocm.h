@@ -292,8 +292,9 @@ typedef struct axr_segment_info {
   uint32_t tensor;        /* index of the tensor the segment belongs to       */
   uint32_t mode;          /* 0 one run, 1 strided run tiles, 2 strided
                              elements, 3 zero fill only, 4 host copy,
-                             5 transposed blocks (dims listed as batch...,
-                             the tensor-contiguous dim, the packed-inner dim) */
+                             5 transposed blocks (all dims in packed order;
+                             the one whose stride equals `granule` is
+                             contiguous in the tensor)                        */
   uint64_t address;       /* tensor-side address of the first element         */
   uint64_t offset;        /* payload offset                                   */
   uint64_t run_bytes;     /* contiguous bytes per run                         */
