@@ -6,6 +6,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <new>
 #include <string>
 #include <vector>
 
@@ -132,6 +133,20 @@ Tunables& tunables();
 
 int fail(int status, const std::string& message);   // records thread-local message
 int check_hip(int hip_error, const char* what);     // 0 or AXR_ERR_HIP
+int fail_nothrow(int status, const char* message) noexcept;
+
+// Every extern "C" entry point runs its body through this: no C++ exception
+// (std::bad_alloc from a container, in practice) crosses the C boundary.
+template <typename Body>
+int guarded(Body&& body) noexcept {
+  try {
+    return body();
+  } catch (const std::bad_alloc&) {
+    return fail_nothrow(AXR_ERR_NOMEM, "out of host memory");
+  } catch (...) {
+    return fail_nothrow(AXR_ERR_INVALID, "unexpected C++ exception");
+  }
+}
 
 // ---------------------------------------------------------------- kernels (axr_kernels.hip)
 

@@ -124,22 +124,6 @@ __device__ __forceinline__ void wave_zero(gbytes dst, uint32_t n, uint32_t lane)
   for (uint32_t i = lane; i < n; i += kWaveLanes) dst[i] = 0;
 }
 
-template <typename T>
-__device__ __forceinline__ void move_as(gcbytes src, gbytes dst) {
-  typedef T __attribute__((aligned(1))) loose;   // no alignment promise on either side
-  *reinterpret_cast<AXR_GLOBAL loose*>(dst) = *reinterpret_cast<const AXR_GLOBAL loose*>(src);
-}
-
-__device__ __forceinline__ void move_granule_dyn(uint32_t g, gcbytes src, gbytes dst) {
-  switch (g) {
-    case 16: move_as<u32x4>(src, dst); break;
-    case 8: move_as<uint64_t>(src, dst); break;
-    case 4: move_as<uint32_t>(src, dst); break;
-    case 2: move_as<uint16_t>(src, dst); break;
-    default: move_as<uint8_t>(src, dst); break;
-  }
-}
-
 typedef const AXR_CONST Seg* seg_table;
 typedef const AXR_CONST Dims* dims_table;
 
@@ -754,7 +738,7 @@ using namespace axr;
 
 extern "C" {
 
-int axr_divide_by_two(float* data, size_t count, void* stream) {
+static int divide_by_two_body(float* data, size_t count, void* stream) {
   if (count == 0) return AXR_OK;
   if (!data) return fail(AXR_ERR_INVALID, "axr_divide_by_two: null data");
   const size_t blocks = (count + 255) / 256;
@@ -763,8 +747,11 @@ int axr_divide_by_two(float* data, size_t count, void* stream) {
                      static_cast<hipStream_t>(stream), data, count);
   return check_hip(hipGetLastError(), "divide_by_two launch");
 }
+int axr_divide_by_two(float* data, size_t count, void* stream) {
+  return guarded([&] { return divide_by_two_body(data, count, stream); });
+}
 
-int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mismatches) {
+static int compare_body(const void* a, const void* b, size_t bytes, uint64_t* mismatches) {
   if (!mismatches) return fail(AXR_ERR_INVALID, "axr_compare: null result");
   *mismatches = 0;
   if (bytes == 0) return AXR_OK;
@@ -784,8 +771,11 @@ int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mismatches
   if (!rc) *mismatches = host;
   return rc;
 }
+int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mismatches) {
+  return guarded([&] { return compare_body(a, b, bytes, mismatches); });
+}
 
-int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum) {
+static int checksum_body(const void* data, size_t bytes, uint64_t start, uint64_t* sum) {
   if (!sum) return fail(AXR_ERR_INVALID, "axr_checksum: null result");
   *sum = 0;
   if (bytes == 0) return AXR_OK;
@@ -805,8 +795,11 @@ int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum) 
   if (!rc) *sum = host;
   return rc;
 }
+int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum) {
+  return guarded([&] { return checksum_body(data, bytes, start, sum); });
+}
 
-int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream) {
+static int copy_reference_body(void* dst, const void* src, size_t bytes, void* stream) {
   if (bytes == 0) return AXR_OK;
   if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_copy_reference: null range");
   if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes) & 15u) {
@@ -817,6 +810,9 @@ int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream) {
                      static_cast<hipStream_t>(stream), static_cast<u32x4*>(dst),
                      static_cast<const u32x4*>(src), nvec);
   return check_hip(hipGetLastError(), "copy_reference launch");
+}
+int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream) {
+  return guarded([&] { return copy_reference_body(dst, src, bytes, stream); });
 }
 
 }  // extern "C"

@@ -103,7 +103,7 @@ int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, u
 
 extern "C" {
 
-int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_t** ctx) {
+static int am_context_create_body(const char* name, size_t zcopy_thresh, axr_am_context_t** ctx) {
   if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_context_create: null result");
   axr_am_context* c = new (std::nothrow) axr_am_context();
   if (!c) return fail(AXR_ERR_NOMEM, "axr_am_context_create: out of host memory");
@@ -112,8 +112,11 @@ int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_
   *ctx = c;
   return AXR_OK;
 }
+int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_t** ctx) {
+  return guarded([&] { return am_context_create_body(name, zcopy_thresh, ctx); });
+}
 
-int axr_am_context_destroy(axr_am_context_t* ctx) {
+static int am_context_destroy_body(axr_am_context_t* ctx) {
   if (!ctx) return AXR_OK;
   {
     std::lock_guard<std::mutex> lock(ctx->mu);
@@ -123,8 +126,11 @@ int axr_am_context_destroy(axr_am_context_t* ctx) {
   delete ctx;
   return AXR_OK;
 }
+int axr_am_context_destroy(axr_am_context_t* ctx) {
+  return guarded([&] { return am_context_destroy_body(ctx); });
+}
 
-int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_id) {
+static int am_connect_body(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_id) {
   if (!from || !to || !conn_id) return fail(AXR_ERR_INVALID, "axr_am_connect: null argument");
   const uint64_t id = g_next_id++;
   std::lock_guard<std::mutex> lock(from->mu);
@@ -132,9 +138,11 @@ int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_
   *conn_id = id;
   return AXR_OK;
 }
+int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_id) {
+  return guarded([&] { return am_connect_body(from, to, conn_id); });
+}
 
-int axr_am_send(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* d, void* stream,
-                uint64_t* request) {
+static int am_send_body(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* d, void* stream, uint64_t* request) {
   if (!ctx || !d) return fail(AXR_ERR_INVALID, "axr_am_send: null argument");
   if (!d->header.data || d->header.size == 0)
     return fail(AXR_ERR_INVALID, "axr_am_send: the header must not be empty");
@@ -165,9 +173,15 @@ int axr_am_send(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* d,
   }
   return deliver(ctx, conn_id, std::move(m), request);
 }
+int axr_am_send(axr_am_context_t* ctx,
+                uint64_t conn_id,
+                const axr_am_data_t* d,
+                void* stream,
+                uint64_t* request) {
+  return guarded([&] { return am_send_body(ctx, conn_id, d, stream, request); });
+}
 
-int axr_am_send_iov(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* d, void* /*stream*/,
-                    uint64_t* request) {
+static int am_send_iov_body(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* d, void* stream, uint64_t* request) {
   if (!ctx || !d) return fail(AXR_ERR_INVALID, "axr_am_send_iov: null argument");
   if (!d->header.data || d->header.size == 0)
     return fail(AXR_ERR_INVALID, "axr_am_send_iov: the header must not be empty");
@@ -189,8 +203,15 @@ int axr_am_send_iov(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_
   if (!m->rndv) m->request->done.store(1);
   return deliver(ctx, conn_id, std::move(m), request);
 }
+int axr_am_send_iov(axr_am_context_t* ctx,
+                    uint64_t conn_id,
+                    const axr_am_iovec_t* d,
+                    void* stream,
+                    uint64_t* request) {
+  return guarded([&] { return am_send_iov_body(ctx, conn_id, d, stream, request); });
+}
 
-int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done) {
+static int am_request_test_body(axr_am_context_t* ctx, uint64_t request, int* done) {
   if (!ctx || !done) return fail(AXR_ERR_INVALID, "axr_am_request_test: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->requests.find(request);
@@ -209,8 +230,11 @@ int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done) {
   if (st != 0) ctx->requests.erase(it);
   return AXR_OK;
 }
+int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done) {
+  return guarded([&] { return am_request_test_body(ctx, request, done); });
+}
 
-int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* out) {
+static int am_recv_header_body(axr_am_context_t* ctx, axr_am_message_t* out) {
   if (!ctx || !out) return fail(AXR_ERR_INVALID, "axr_am_recv_header: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (ctx->arrived.empty()) return fail(AXR_ERR_NO_MESSAGE, "no message queued");
@@ -227,6 +251,9 @@ int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* out) {
   const uint64_t key = m->key;
   ctx->parked[key] = std::move(m);
   return AXR_OK;
+}
+int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* out) {
+  return guarded([&] { return am_recv_header_body(ctx, out); });
 }
 
 static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_buffer_t* vec,
@@ -280,24 +307,37 @@ static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_bu
   return rc;
 }
 
-int axr_am_recv_buffer(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst, size_t dst_bytes,
-                       void* stream) {
+static int am_recv_buffer_body(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst, size_t dst_bytes, void* stream) {
   if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null context");
   if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null buffer");
   axr_buffer_t one{dst, dst_bytes};
   return fetch(ctx, key, dst_type, &one, 1, stream);
 }
+int axr_am_recv_buffer(axr_am_context_t* ctx,
+                       uint64_t key,
+                       int dst_type,
+                       void* dst,
+                       size_t dst_bytes,
+                       void* stream) {
+  return guarded([&] { return am_recv_buffer_body(ctx, key, dst_type, dst, dst_bytes, stream); });
+}
 
-int axr_am_recv_buffer_async(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
-                             size_t dst_bytes, void* stream) {
+static int am_recv_buffer_async_body(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst, size_t dst_bytes, void* stream) {
   if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_async: null context");
   if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_async: null buffer");
   axr_buffer_t one{dst, dst_bytes};
   return fetch(ctx, key, dst_type, &one, 1, stream, /*wait=*/false);
 }
+int axr_am_recv_buffer_async(axr_am_context_t* ctx,
+                             uint64_t key,
+                             int dst_type,
+                             void* dst,
+                             size_t dst_bytes,
+                             void* stream) {
+  return guarded([&] { return am_recv_buffer_async_body(ctx, key, dst_type, dst, dst_bytes, stream); });
+}
 
-int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,
-                           const axr_buffer_t* buffer_vec, size_t buffer_count, void* stream) {
+static int am_recv_buffer_iov_body(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_buffer_t* buffer_vec, size_t buffer_count, void* stream) {
   if (!ctx || !buffer_vec || buffer_count == 0)
     return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_iov: null or empty buffer vector");
   for (size_t i = 0; i < buffer_count; ++i) {
@@ -306,8 +346,16 @@ int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,
   }
   return fetch(ctx, key, dst_type, buffer_vec, buffer_count, stream);
 }
+int axr_am_recv_buffer_iov(axr_am_context_t* ctx,
+                           uint64_t key,
+                           int dst_type,
+                           const axr_buffer_t* buffer_vec,
+                           size_t buffer_count,
+                           void* stream) {
+  return guarded([&] { return am_recv_buffer_iov_body(ctx, key, dst_type, buffer_vec, buffer_count, stream); });
+}
 
-int axr_am_message_release(axr_am_context_t* ctx, uint64_t key) {
+static int am_message_release_body(axr_am_context_t* ctx, uint64_t key) {
   if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_message_release: null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->parked.find(key);
@@ -316,12 +364,18 @@ int axr_am_message_release(axr_am_context_t* ctx, uint64_t key) {
   ctx->parked.erase(it);
   return AXR_OK;
 }
+int axr_am_message_release(axr_am_context_t* ctx, uint64_t key) {
+  return guarded([&] { return am_message_release_body(ctx, key); });
+}
 
-int axr_am_pending(axr_am_context_t* ctx, size_t* count) {
+static int am_pending_body(axr_am_context_t* ctx, size_t* count) {
   if (!ctx || !count) return fail(AXR_ERR_INVALID, "axr_am_pending: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   *count = ctx->arrived.size();
   return AXR_OK;
+}
+int axr_am_pending(axr_am_context_t* ctx, size_t* count) {
+  return guarded([&] { return am_pending_body(ctx, count); });
 }
 
 }  // extern "C"

@@ -758,13 +758,15 @@ int store_tensor(axr_plan* p, const axr_tensor_t& in, TensorRec* rec) {
 
 extern "C" {
 
-int axr_tensor_nbytes(const axr_tensor_t* t, uint64_t* nbytes) {
+static int tensor_nbytes_body(const axr_tensor_t* t, uint64_t* nbytes) {
   if (!t || !nbytes) return fail(AXR_ERR_INVALID, "axr_tensor_nbytes: null argument");
   return nbytes_rule(t->ndim, t->shape, t->dtype_bits, nbytes);
 }
+int axr_tensor_nbytes(const axr_tensor_t* t, uint64_t* nbytes) {
+  return guarded([&] { return tensor_nbytes_body(t, nbytes); });
+}
 
-int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align, uint32_t /*flags*/,
-                    axr_plan_t** plan) {
+static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t align, uint32_t flags, axr_plan_t** plan) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_create: null result");
   *plan = nullptr;
   if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_create: null tensor array");
@@ -792,8 +794,15 @@ int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align, uint3
   *plan = p;
   return AXR_OK;
 }
+int axr_plan_create(const axr_tensor_t* tensors,
+                    size_t n,
+                    uint32_t align,
+                    uint32_t flags,
+                    axr_plan_t** plan) {
+  return guarded([&] { return plan_create_body(tensors, n, align, flags, plan); });
+}
 
-int axr_plan_free(axr_plan_t* plan) {
+static int plan_free_body(axr_plan_t* plan) {
   if (!plan) return AXR_OK;
   quiesce(plan);
   if (plan->uploaded && plan->upload_event) (void)hipEventSynchronize(plan->upload_event);
@@ -806,26 +815,38 @@ int axr_plan_free(axr_plan_t* plan) {
   delete plan;
   return AXR_OK;
 }
+int axr_plan_free(axr_plan_t* plan) {
+  return guarded([&] { return plan_free_body(plan); });
+}
 
-int axr_plan_num_tensors(const axr_plan_t* plan, size_t* n) {
+static int plan_num_tensors_body(const axr_plan_t* plan, size_t* n) {
   if (!plan || !n) return fail(AXR_ERR_INVALID, "axr_plan_num_tensors: null argument");
   *n = plan->tensors.size();
   return AXR_OK;
 }
+int axr_plan_num_tensors(const axr_plan_t* plan, size_t* n) {
+  return guarded([&] { return plan_num_tensors_body(plan, n); });
+}
 
-int axr_plan_payload_bytes(const axr_plan_t* plan, uint64_t* bytes) {
+static int plan_payload_bytes_body(const axr_plan_t* plan, uint64_t* bytes) {
   if (!plan || !bytes) return fail(AXR_ERR_INVALID, "axr_plan_payload_bytes: null argument");
   *bytes = plan->payload_bytes;
   return AXR_OK;
 }
+int axr_plan_payload_bytes(const axr_plan_t* plan, uint64_t* bytes) {
+  return guarded([&] { return plan_payload_bytes_body(plan, bytes); });
+}
 
-int axr_plan_data_bytes(const axr_plan_t* plan, uint64_t* bytes) {
+static int plan_data_bytes_body(const axr_plan_t* plan, uint64_t* bytes) {
   if (!plan || !bytes) return fail(AXR_ERR_INVALID, "axr_plan_data_bytes: null argument");
   *bytes = plan->data_bytes;
   return AXR_OK;
 }
+int axr_plan_data_bytes(const axr_plan_t* plan, uint64_t* bytes) {
+  return guarded([&] { return plan_data_bytes_body(plan, bytes); });
+}
 
-int axr_plan_layout(const axr_plan_t* plan, uint64_t* offsets, uint64_t* sizes) {
+static int plan_layout_body(const axr_plan_t* plan, uint64_t* offsets, uint64_t* sizes) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_layout: null plan");
   for (size_t i = 0; i < plan->tensors.size(); ++i) {
     if (offsets) offsets[i] = plan->tensors[i].offset;
@@ -833,8 +854,11 @@ int axr_plan_layout(const axr_plan_t* plan, uint64_t* offsets, uint64_t* sizes) 
   }
   return AXR_OK;
 }
+int axr_plan_layout(const axr_plan_t* plan, uint64_t* offsets, uint64_t* sizes) {
+  return guarded([&] { return plan_layout_body(plan, offsets, sizes); });
+}
 
-int axr_plan_tensor_meta(const axr_plan_t* plan, size_t i, axr_tensor_t* meta) {
+static int plan_tensor_meta_body(const axr_plan_t* plan, size_t i, axr_tensor_t* meta) {
   if (!plan || !meta) return fail(AXR_ERR_INVALID, "axr_plan_tensor_meta: null argument");
   if (i >= plan->tensors.size()) return fail(AXR_ERR_INVALID, "axr_plan_tensor_meta: index out of range");
   const TensorRec& t = plan->tensors[i];
@@ -850,15 +874,21 @@ int axr_plan_tensor_meta(const axr_plan_t* plan, size_t i, axr_tensor_t* meta) {
   meta->byte_offset = 0;
   return AXR_OK;
 }
+int axr_plan_tensor_meta(const axr_plan_t* plan, size_t i, axr_tensor_t* meta) {
+  return guarded([&] { return plan_tensor_meta_body(plan, i, meta); });
+}
 
-int axr_plan_header(const axr_plan_t* plan, const void** header, size_t* length) {
+static int plan_header_body(const axr_plan_t* plan, const void** header, size_t* length) {
   if (!plan || !header || !length) return fail(AXR_ERR_INVALID, "axr_plan_header: null argument");
   *header = plan->header.data();
   *length = plan->header.size();
   return AXR_OK;
 }
+int axr_plan_header(const axr_plan_t* plan, const void** header, size_t* length) {
+  return guarded([&] { return plan_header_body(plan, header, length); });
+}
 
-int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan) {
+static int plan_from_header_body(const void* header, size_t length, axr_plan_t** plan) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_from_header: null result");
   *plan = nullptr;
   if (!header) return fail(AXR_ERR_INVALID, "axr_plan_from_header: null header");
@@ -928,8 +958,11 @@ int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan) {
   *plan = p;
   return AXR_OK;
 }
+int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan) {
+  return guarded([&] { return plan_from_header_body(header, length, plan); });
+}
 
-int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {
+static int plan_bind_body(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_bind: null plan");
   if (n != plan->tensors.size())
     return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor count differs from the plan");
@@ -968,9 +1001,11 @@ int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {
   plan->bound = true;
   return AXR_OK;
 }
+int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {
+  return guarded([&] { return plan_bind_body(plan, tensors, n); });
+}
 
-int axr_plan_split(const axr_plan_t* plan, void* payload, size_t payload_bytes,
-                   axr_buffer_t* views) {
+static int plan_split_body(const axr_plan_t* plan, void* payload, size_t payload_bytes, axr_buffer_t* views) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_split: null plan");
   if (plan->payload_bytes > payload_bytes)
     return fail(AXR_ERR_LENGTH, "Total size of chunks exceeds buffer size");
@@ -982,16 +1017,28 @@ int axr_plan_split(const axr_plan_t* plan, void* payload, size_t payload_bytes,
   }
   return AXR_OK;
 }
+int axr_plan_split(const axr_plan_t* plan,
+                   void* payload,
+                   size_t payload_bytes,
+                   axr_buffer_t* views) {
+  return guarded([&] { return plan_split_body(plan, payload, payload_bytes, views); });
+}
 
-int axr_pack(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream) {
+static int pack_body(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream) {
   return run(plan, true, payload, payload_bytes, stream);
 }
-
-int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes, void* stream) {
-  return run(plan, false, const_cast<void*>(payload), payload_bytes, stream);
+int axr_pack(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream) {
+  return guarded([&] { return pack_body(plan, payload, payload_bytes, stream); });
 }
 
-int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
+static int unpack_body(axr_plan_t* plan, const void* payload, size_t payload_bytes, void* stream) {
+  return run(plan, false, const_cast<void*>(payload), payload_bytes, stream);
+}
+int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes, void* stream) {
+  return guarded([&] { return unpack_body(plan, payload, payload_bytes, stream); });
+}
+
+static int plan_launch_info_body(axr_plan_t* plan, axr_launch_info_t* info) {
   if (!plan || !info) return fail(AXR_ERR_INVALID, "axr_plan_launch_info: null argument");
   int rc = build_tables(plan);
   if (rc) return rc;
@@ -1005,8 +1052,11 @@ int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
   info->host_chunks = static_cast<uint32_t>(plan->host_chunks.size());
   return AXR_OK;
 }
+int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
+  return guarded([&] { return plan_launch_info_body(plan, info); });
+}
 
-int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity, size_t* count) {
+static int plan_segments_body(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity, size_t* count) {
   if (!plan || !count) return fail(AXR_ERR_INVALID, "axr_plan_segments: null argument");
   int rc = build_tables(plan);
   if (rc) return rc;
@@ -1071,6 +1121,9 @@ int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity
     o.run_bytes = o.nbytes = plan->host_copies[i].bytes;
   }
   return AXR_OK;
+}
+int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity, size_t* count) {
+  return guarded([&] { return plan_segments_body(plan, out, capacity, count); });
 }
 
 }  // extern "C"

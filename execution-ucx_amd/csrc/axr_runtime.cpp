@@ -24,6 +24,15 @@ int fail(int status, const std::string& message) {
   return status;
 }
 
+int fail_nothrow(int status, const char* message) noexcept {
+  try {
+    g_last_error = message;
+  } catch (...) {
+    g_last_error.clear();
+  }
+  return status;
+}
+
 int check_hip(int hip_error, const char* what) {
   if (hip_error == hipSuccess) return AXR_OK;
   const hipError_t e = static_cast<hipError_t>(hip_error);
@@ -254,7 +263,7 @@ const char* axr_last_error(void) { return g_last_error.c_str(); }
 
 const char* axr_version(void) { return "0.1.0"; }
 
-int axr_dl_device_to_memory_type(int32_t t) {
+static int dl_device_to_memory_type_body(int32_t t) {
   switch (t) {
     case 2: return AXR_MEM_CUDA;
     case 13: return AXR_MEM_CUDA_MANAGED;
@@ -263,6 +272,9 @@ int axr_dl_device_to_memory_type(int32_t t) {
     case 1: return AXR_MEM_HOST;
     default: return AXR_MEM_UNKNOWN;
   }
+}
+int axr_dl_device_to_memory_type(int32_t t) {
+  return guarded([&] { return dl_device_to_memory_type_body(t); });
 }
 
 int32_t axr_memory_type_to_dl_device(int m) {
@@ -278,7 +290,7 @@ int32_t axr_memory_type_to_dl_device(int m) {
   }
 }
 
-int axr_tune_set(const char* key, int64_t value) {
+static int tune_set_body(const char* key, int64_t value) {
   if (!key) return fail(AXR_ERR_INVALID, "axr_tune_set: null key");
   Tunables& t = tunables();
   const std::string k(key);
@@ -315,8 +327,11 @@ int axr_tune_set(const char* key, int64_t value) {
   }
   return AXR_OK;
 }
+int axr_tune_set(const char* key, int64_t value) {
+  return guarded([&] { return tune_set_body(key, value); });
+}
 
-int axr_tune_get(const char* key, int64_t* value) {
+static int tune_get_body(const char* key, int64_t* value) {
   if (!key || !value) return fail(AXR_ERR_INVALID, "axr_tune_get: null argument");
   const Tunables& t = tunables();
   const std::string k(key);
@@ -332,10 +347,13 @@ int axr_tune_get(const char* key, int64_t* value) {
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }
+int axr_tune_get(const char* key, int64_t* value) {
+  return guarded([&] { return tune_get_body(key, value); });
+}
 
 // ---------------------------------------------------------------- device
 
-int axr_device_count(int* count) {
+static int device_count_body(int* count) {
   if (!count) return fail(AXR_ERR_INVALID, "axr_device_count: null result");
   *count = 0;
   const hipError_t e = hipGetDeviceCount(count);
@@ -345,15 +363,26 @@ int axr_device_count(int* count) {
   }
   return check_hip(e, "hipGetDeviceCount");
 }
+int axr_device_count(int* count) {
+  return guarded([&] { return device_count_body(count); });
+}
 
-int axr_device_get(int* device) {
+static int device_get_body(int* device) {
   if (!device) return fail(AXR_ERR_INVALID, "axr_device_get: null result");
   return check_hip(hipGetDevice(device), "hipGetDevice");
 }
+int axr_device_get(int* device) {
+  return guarded([&] { return device_get_body(device); });
+}
 
-int axr_device_set(int device) { return check_hip(hipSetDevice(device), "hipSetDevice"); }
+static int device_set_body(int device) {
+  return check_hip(hipSetDevice(device), "hipSetDevice");
+}
+int axr_device_set(int device) {
+  return guarded([&] { return device_set_body(device); });
+}
 
-int axr_device_push(int device, int* token) {
+static int device_push_body(int device, int* token) {
   if (!token) return fail(AXR_ERR_INVALID, "axr_device_push: null token");
   int prev = 0;
   int rc = check_hip(hipGetDevice(&prev), "hipGetDevice");
@@ -363,14 +392,25 @@ int axr_device_push(int device, int* token) {
   *token = prev;
   return AXR_OK;
 }
-
-int axr_device_pop(int token) { return check_hip(hipSetDevice(token), "hipSetDevice"); }
-
-int axr_device_synchronize(void) {
-  return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+int axr_device_push(int device, int* token) {
+  return guarded([&] { return device_push_body(device, token); });
 }
 
-int axr_device_info(int* compute_units, uint64_t* total_mem, uint64_t* free_mem) {
+static int device_pop_body(int token) {
+  return check_hip(hipSetDevice(token), "hipSetDevice");
+}
+int axr_device_pop(int token) {
+  return guarded([&] { return device_pop_body(token); });
+}
+
+static int device_synchronize_body() {
+  return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+}
+int axr_device_synchronize(void) {
+  return guarded([&] { return device_synchronize_body(); });
+}
+
+static int device_info_body(int* compute_units, uint64_t* total_mem, uint64_t* free_mem) {
   if (compute_units) {
     int rc = device_compute_units(compute_units);
     if (rc) return rc;
@@ -384,8 +424,11 @@ int axr_device_info(int* compute_units, uint64_t* total_mem, uint64_t* free_mem)
   }
   return AXR_OK;
 }
+int axr_device_info(int* compute_units, uint64_t* total_mem, uint64_t* free_mem) {
+  return guarded([&] { return device_info_body(compute_units, total_mem, free_mem); });
+}
 
-int axr_stream_create(void** stream) {
+static int stream_create_body(void** stream) {
   if (!stream) return fail(AXR_ERR_INVALID, "axr_stream_create: null result");
   hipStream_t s = nullptr;
   // Default priority on purpose; non-blocking so it does not serialise with the null stream.
@@ -394,25 +437,37 @@ int axr_stream_create(void** stream) {
   *stream = s;
   return AXR_OK;
 }
+int axr_stream_create(void** stream) {
+  return guarded([&] { return stream_create_body(stream); });
+}
 
-int axr_stream_destroy(void* stream) {
+static int stream_destroy_body(void* stream) {
   if (!stream) return AXR_OK;
   return check_hip(hipStreamDestroy(static_cast<hipStream_t>(stream)), "hipStreamDestroy");
 }
+int axr_stream_destroy(void* stream) {
+  return guarded([&] { return stream_destroy_body(stream); });
+}
 
-int axr_stream_synchronize(void* stream) {
+static int stream_synchronize_body(void* stream) {
   return check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)),
                    "hipStreamSynchronize");
 }
+int axr_stream_synchronize(void* stream) {
+  return guarded([&] { return stream_synchronize_body(stream); });
+}
 
-int axr_stream_wait_event(void* stream, void* event) {
+static int stream_wait_event_body(void* stream, void* event) {
   if (!event) return fail(AXR_ERR_INVALID, "axr_stream_wait_event: null event");
   return check_hip(hipStreamWaitEvent(static_cast<hipStream_t>(stream),
                                       static_cast<hipEvent_t>(event), 0),
                    "hipStreamWaitEvent");
 }
+int axr_stream_wait_event(void* stream, void* event) {
+  return guarded([&] { return stream_wait_event_body(stream, event); });
+}
 
-int axr_event_create(void** event) {
+static int event_create_body(void** event) {
   if (!event) return fail(AXR_ERR_INVALID, "axr_event_create: null result");
   hipEvent_t e = nullptr;
   int rc = check_hip(hipEventCreate(&e), "hipEventCreate");
@@ -420,25 +475,37 @@ int axr_event_create(void** event) {
   *event = e;
   return AXR_OK;
 }
+int axr_event_create(void** event) {
+  return guarded([&] { return event_create_body(event); });
+}
 
-int axr_event_destroy(void* event) {
+static int event_destroy_body(void* event) {
   if (!event) return AXR_OK;
   return check_hip(hipEventDestroy(static_cast<hipEvent_t>(event)), "hipEventDestroy");
 }
+int axr_event_destroy(void* event) {
+  return guarded([&] { return event_destroy_body(event); });
+}
 
-int axr_event_record(void* event, void* stream) {
+static int event_record_body(void* event, void* stream) {
   if (!event) return fail(AXR_ERR_INVALID, "axr_event_record: null event");
   return check_hip(hipEventRecord(static_cast<hipEvent_t>(event),
                                   static_cast<hipStream_t>(stream)),
                    "hipEventRecord");
 }
+int axr_event_record(void* event, void* stream) {
+  return guarded([&] { return event_record_body(event, stream); });
+}
 
-int axr_event_synchronize(void* event) {
+static int event_synchronize_body(void* event) {
   if (!event) return fail(AXR_ERR_INVALID, "axr_event_synchronize: null event");
   return check_hip(hipEventSynchronize(static_cast<hipEvent_t>(event)), "hipEventSynchronize");
 }
+int axr_event_synchronize(void* event) {
+  return guarded([&] { return event_synchronize_body(event); });
+}
 
-int axr_event_query(void* event, int* done) {
+static int event_query_body(void* event, int* done) {
   if (!event || !done) return fail(AXR_ERR_INVALID, "axr_event_query: null argument");
   const hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
   if (e == hipSuccess) {
@@ -451,17 +518,23 @@ int axr_event_query(void* event, int* done) {
   }
   return check_hip(e, "hipEventQuery");
 }
+int axr_event_query(void* event, int* done) {
+  return guarded([&] { return event_query_body(event, done); });
+}
 
-int axr_event_elapsed_ms(void* start, void* stop, float* ms) {
+static int event_elapsed_ms_body(void* start, void* stop, float* ms) {
   if (!start || !stop || !ms) return fail(AXR_ERR_INVALID, "axr_event_elapsed_ms: null argument");
   return check_hip(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start),
                                        static_cast<hipEvent_t>(stop)),
                    "hipEventElapsedTime");
 }
+int axr_event_elapsed_ms(void* start, void* stop, float* ms) {
+  return guarded([&] { return event_elapsed_ms_body(start, stop, ms); });
+}
 
 // ---------------------------------------------------------------- memory
 
-int axr_mem_alloc(int memory_type, size_t bytes, size_t alignment, void** ptr) {
+static int mem_alloc_body(int memory_type, size_t bytes, size_t alignment, void** ptr) {
   if (!ptr) return fail(AXR_ERR_INVALID, "axr_mem_alloc: null result");
   *ptr = nullptr;
   switch (memory_type) {
@@ -497,8 +570,11 @@ int axr_mem_alloc(int memory_type, size_t bytes, size_t alignment, void** ptr) {
       return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
   }
 }
+int axr_mem_alloc(int memory_type, size_t bytes, size_t alignment, void** ptr) {
+  return guarded([&] { return mem_alloc_body(memory_type, bytes, alignment, ptr); });
+}
 
-int axr_mem_free(int memory_type, void* ptr, size_t /*bytes*/) {
+static int mem_free_body(int memory_type, void* ptr, size_t bytes) {
   if (!ptr) return AXR_OK;
   switch (memory_type) {
     case AXR_MEM_HOST:
@@ -518,6 +594,9 @@ int axr_mem_free(int memory_type, void* ptr, size_t /*bytes*/) {
       return fail(AXR_ERR_UNSUPPORTED, "Unsupported memory type");
   }
 }
+int axr_mem_free(int memory_type, void* ptr, size_t bytes) {
+  return guarded([&] { return mem_free_body(memory_type, ptr, bytes); });
+}
 
 static int copy_kind(int dst_type, int src_type, hipMemcpyKind* kind) {
   auto is_host = [](int t) { return t == AXR_MEM_HOST || t == AXR_MEM_ROCM_MANAGED; };
@@ -530,7 +609,7 @@ static int copy_kind(int dst_type, int src_type, hipMemcpyKind* kind) {
   return AXR_OK;
 }
 
-int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t bytes) {
+static int memcpy_body(int dst_type, void* dst, int src_type, const void* src, size_t bytes) {
   if (bytes == 0) return AXR_OK;
   if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_memcpy: null pointer");
   hipMemcpyKind kind;
@@ -542,9 +621,11 @@ int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t by
   }
   return check_hip(hipMemcpy(dst, src, bytes, kind), "hipMemcpy");
 }
+int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t bytes) {
+  return guarded([&] { return memcpy_body(dst_type, dst, src_type, src, bytes); });
+}
 
-int axr_memcpy_async(int dst_type, void* dst, int src_type, const void* src, size_t bytes,
-                     void* stream) {
+static int memcpy_async_body(int dst_type, void* dst, int src_type, const void* src, size_t bytes, void* stream) {
   if (bytes == 0) return AXR_OK;
   if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_memcpy_async: null pointer");
   hipMemcpyKind kind;
@@ -553,16 +634,27 @@ int axr_memcpy_async(int dst_type, void* dst, int src_type, const void* src, siz
   return check_hip(hipMemcpyAsync(dst, src, bytes, kind, static_cast<hipStream_t>(stream)),
                    "hipMemcpyAsync");
 }
+int axr_memcpy_async(int dst_type,
+                     void* dst,
+                     int src_type,
+                     const void* src,
+                     size_t bytes,
+                     void* stream) {
+  return guarded([&] { return memcpy_async_body(dst_type, dst, src_type, src, bytes, stream); });
+}
 
-int axr_memset_async(void* dst, int value, size_t bytes, void* stream) {
+static int memset_async_body(void* dst, int value, size_t bytes, void* stream) {
   if (bytes == 0) return AXR_OK;
   if (!dst) return fail(AXR_ERR_INVALID, "axr_memset_async: null pointer");
   return launch_fill(dst, value, bytes, stream);
 }
+int axr_memset_async(void* dst, int value, size_t bytes, void* stream) {
+  return guarded([&] { return memset_async_body(dst, value, bytes, stream); });
+}
 
 // ---------------------------------------------------------------- pool
 
-int axr_pool_create(int device, size_t slab_bytes, axr_pool_t** pool) {
+static int pool_create_body(int device, size_t slab_bytes, axr_pool_t** pool) {
   if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_create: null result");
   int count = 0;
   int rc = axr_device_count(&count);
@@ -576,8 +668,11 @@ int axr_pool_create(int device, size_t slab_bytes, axr_pool_t** pool) {
   *pool = p;
   return AXR_OK;
 }
+int axr_pool_create(int device, size_t slab_bytes, axr_pool_t** pool) {
+  return guarded([&] { return pool_create_body(device, slab_bytes, pool); });
+}
 
-int axr_pool_destroy(axr_pool_t* pool) {
+static int pool_destroy_body(axr_pool_t* pool) {
   if (!pool) return AXR_OK;
   {
     std::lock_guard<std::mutex> lock(pool->mu);
@@ -590,8 +685,11 @@ int axr_pool_destroy(axr_pool_t* pool) {
   delete pool;
   return AXR_OK;
 }
+int axr_pool_destroy(axr_pool_t* pool) {
+  return guarded([&] { return pool_destroy_body(pool); });
+}
 
-int axr_pool_default(axr_pool_t** pool) {
+static int pool_default_body(axr_pool_t** pool) {
   if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_default: null result");
   int dev = 0;
   int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
@@ -607,9 +705,11 @@ int axr_pool_default(axr_pool_t** pool) {
   *pool = it->second;
   return AXR_OK;
 }
+int axr_pool_default(axr_pool_t** pool) {
+  return guarded([&] { return pool_default_body(pool); });
+}
 
-int axr_pool_set_registrar(axr_pool_t* pool, axr_register_fn reg, axr_unregister_fn unreg,
-                           void* user) {
+static int pool_set_registrar_body(axr_pool_t* pool, axr_register_fn reg, axr_unregister_fn unreg, void* user) {
   if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_set_registrar: null pool");
   std::lock_guard<std::mutex> lock(pool->mu);
   if (!pool->slabs.empty())
@@ -619,8 +719,14 @@ int axr_pool_set_registrar(axr_pool_t* pool, axr_register_fn reg, axr_unregister
   pool->user = user;
   return AXR_OK;
 }
+int axr_pool_set_registrar(axr_pool_t* pool,
+                           axr_register_fn reg,
+                           axr_unregister_fn unreg,
+                           void* user) {
+  return guarded([&] { return pool_set_registrar_body(pool, reg, unreg, user); });
+}
 
-int axr_pool_alloc(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr, void** mem_h) {
+static int pool_alloc_body(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr, void** mem_h) {
   if (!pool || !ptr) return fail(AXR_ERR_INVALID, "axr_pool_alloc: null argument");
   *ptr = nullptr;
   if (mem_h) *mem_h = nullptr;
@@ -659,8 +765,11 @@ int axr_pool_alloc(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr,
   }
   return fail(AXR_ERR_NOMEM, "axr_pool_alloc: no block after growing the pool");
 }
+int axr_pool_alloc(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr, void** mem_h) {
+  return guarded([&] { return pool_alloc_body(pool, bytes, alignment, ptr, mem_h); });
+}
 
-int axr_pool_free(axr_pool_t* pool, void* ptr) {
+static int pool_free_body(axr_pool_t* pool, void* ptr) {
   if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_free: null pool");
   if (!ptr) return AXR_OK;
   std::lock_guard<std::mutex> lock(pool->mu);
@@ -674,8 +783,11 @@ int axr_pool_free(axr_pool_t* pool, void* ptr) {
   pool->add_free(block, used);
   return AXR_OK;
 }
+int axr_pool_free(axr_pool_t* pool, void* ptr) {
+  return guarded([&] { return pool_free_body(pool, ptr); });
+}
 
-int axr_pool_trim(axr_pool_t* pool) {
+static int pool_trim_body(axr_pool_t* pool) {
   if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_trim: null pool");
   std::lock_guard<std::mutex> lock(pool->mu);
   DeviceGuard guard;
@@ -698,8 +810,11 @@ int axr_pool_trim(axr_pool_t* pool) {
   }
   return AXR_OK;
 }
+int axr_pool_trim(axr_pool_t* pool) {
+  return guarded([&] { return pool_trim_body(pool); });
+}
 
-int axr_pool_get_stats(axr_pool_t* pool, axr_pool_stats_t* stats) {
+static int pool_get_stats_body(axr_pool_t* pool, axr_pool_stats_t* stats) {
   if (!pool || !stats) return fail(AXR_ERR_INVALID, "axr_pool_get_stats: null argument");
   std::lock_guard<std::mutex> lock(pool->mu);
   stats->slabs = pool->slabs.size();
@@ -709,6 +824,9 @@ int axr_pool_get_stats(axr_pool_t* pool, axr_pool_stats_t* stats) {
   stats->live_blocks = pool->live.size();
   stats->peak_bytes = pool->peak;
   return AXR_OK;
+}
+int axr_pool_get_stats(axr_pool_t* pool, axr_pool_stats_t* stats) {
+  return guarded([&] { return pool_get_stats_body(pool, stats); });
 }
 
 }  // extern "C"
