@@ -48,6 +48,51 @@ inline ucxx::UcxBuffer ReceiveBufferFor(const void* header, size_t header_length
                          [pmr, bytes](void* p) { pmr->deallocate(ucx_memory_type::ROCM, p, bytes); });
 }
 
+// Bytes of the packed payload for a list of tensor metas: the layout rule of the
+// bundle (offset[i+1] = align_up(offset[i] + nbytes[i])) with the reference's size
+// rule (rpc_core/utils/tensor_meta.hpp:91-104).  `Metas` is any range of records
+// with the fields of rpc::utils::TensorMeta (`ndim`, `dtype.bits`, `shape[i]`),
+// e.g. rpc::utils::TensorMetaSpan.
+template <typename Metas>
+inline size_t BundleBytesFor(const Metas& metas, uint32_t align) {
+  uint64_t end = 0;
+  for (const auto& m : metas) {
+    uint64_t nbytes = 0;
+    if (m.ndim != 0) {
+      nbytes = (static_cast<uint64_t>(m.dtype.bits) + 7) / 8;
+      for (int32_t d = 0; d < m.ndim; ++d) nbytes *= static_cast<uint64_t>(m.shape[d]);
+    }
+    end = (end + align - 1) / align * align + nbytes;
+  }
+  return static_cast<size_t>(end);
+}
+
+// A receive-side memory policy: callable with the tensor metas of an incoming
+// rendezvous message, returns ONE ROCm pool block (with the slab's ucp_mem_h) that
+// the whole bundle lands in.  Usable as eux::axon::CustomMemoryPolicy<ucxx::UcxBuffer>
+// (axon/include/axon/memory_policy.hpp:28-36,72-73); the worker calls it from
+// ProcessRndvBufferImpl_ (axon/src/axon_worker.cpp:1150-1172).  Copyable, as the
+// facade requires; the manager must outlive it.
+class RocmBundleReceivePolicy {
+ public:
+  RocmBundleReceivePolicy(ucxx::UcxRocmMemoryResourceManager& mr, uint32_t align)
+      : mr_(&mr), align_(align) {}
+
+  template <typename Metas>
+  ucxx::UcxBuffer operator()(Metas metas) const {
+    const size_t bytes = BundleBytesFor(metas, align_);
+    void* mem_h = nullptr;
+    void* data = mr_->allocate_registered(bytes ? bytes : 1, 256, &mem_h);
+    ucxx::UcxRocmMemoryResourceManager* mr = mr_;
+    return ucxx::UcxBuffer(*mr, ucx_memory_type::ROCM, data, bytes, mem_h, /*own_buffer=*/true,
+                           [mr, bytes](void* p) { mr->deallocate(ucx_memory_type::ROCM, p, bytes); });
+  }
+
+ private:
+  ucxx::UcxRocmMemoryResourceManager* mr_;
+  uint32_t align_;
+};
+
 // Zero-copy split of a received payload: UcxBuffer::to_buffer_vec with the sizes
 // the bundle header carries, valid for the tight layout (align == 1) the
 // reference understands; aligned layouts use SplitPayload instead.

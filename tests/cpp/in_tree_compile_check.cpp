@@ -31,3 +31,22 @@ eux::ucxx::UcxBufferVec Exercise(eux::ucxx::UcxRocmMemoryResourceManager& mr, co
             sent.second.size());
   return eux::axon::rocm::ToUcxBufferVec(std::move(recv), sent.first.data(), sent.first.size());
 }
+
+// The receive policy is generic over the meta record; rpc::utils::TensorMeta itself
+// needs cista, which is not installed here, so a record with the same fields stands in.
+namespace {
+struct MetaLike {
+  struct { int32_t device_type, device_id; } device;
+  int32_t ndim;
+  struct { uint8_t code, bits; uint16_t lanes; } dtype;
+  uint64_t byte_offset;
+  std::vector<int64_t> shape, strides;
+};
+}  // namespace
+
+eux::ucxx::UcxBuffer ExercisePolicy(eux::ucxx::UcxRocmMemoryResourceManager& mr,
+                                    const std::vector<MetaLike>& metas) {
+  eux::axon::rocm::RocmBundleReceivePolicy policy(mr, 256);
+  eux::axon::rocm::RocmBundleReceivePolicy copy = policy;   // the facade copies providers
+  return copy(metas);
+}
