@@ -320,6 +320,39 @@ def host_bundle_c1(h, reps=30):
             "GBps_pcie_inclusive_4P": round(4.0 * nbytes / t / 1e9, 2)}
 
 
+def checkpoint_staging(h, tensors=4096, each=64 * 1024, reps=5):
+    """A packed device bundle to host byte arrays, one per tensor: the staged
+    path (8 MiB pinned blocks, one device copy each) against one pageable copy
+    per tensor, which is how the reference's checkpoint writer fetches a payload
+    (axon/src/storage/avro_serialization.cpp:478-523)."""
+    import numpy as np
+    torch = h.torch
+    src = torch.randint(0, 256, (tensors, each), dtype=torch.uint8, device="cuda")
+    bundle = h.pkg.pack_bundle([src[i] for i in range(tensors)], align=256)
+    torch.cuda.synchronize()
+    nbytes = tensors * each
+    staged, naive = [], []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        arrays = h.pkg.bundle_to_host(bundle.header, bundle.payload, bundle.payload_bytes)
+        staged.append(time.perf_counter() - t0)
+        outs = [np.empty(each, dtype=np.uint8) for _ in range(tensors)]
+        t0 = time.perf_counter()
+        for i, o in enumerate(outs):
+            h.capi.check(h.lib.axr_memcpy(h.capi.MEM_HOST, o.ctypes.data, h.capi.MEM_ROCM,
+                                          bundle.payload.data + i * each, each))
+        naive.append(time.perf_counter() - t0)
+    host = src.cpu().numpy()
+    if any(not np.array_equal(a, host[i]) for i, a in enumerate(arrays)) or \
+            any(not np.array_equal(o, host[i]) for i, o in enumerate(outs)):
+        raise SystemExit("bench.py: staged host copy differs")
+    bundle.plan.close()
+    bundle.payload.release()
+    return {"tensors": tensors, "payload_bytes_P": nbytes,
+            "staged_GBps": round(nbytes / sorted(staged)[reps // 2] / 1e9, 2),
+            "copy_per_tensor_GBps": round(nbytes / sorted(naive)[reps // 2] / 1e9, 2)}
+
+
 def cpu_baseline(spec, seed=0):
     """Reference host path on this box's cores: memcpy concat + split of the same bundle."""
     import numpy as np
@@ -466,6 +499,7 @@ def main():
         del tr
         torch.cuda.empty_cache()
         extras["c1_host_bundle"] = host_bundle_c1(h)
+        extras["checkpoint_to_host"] = checkpoint_staging(h)
         extras["c5_streamed_8GiB"] = stream_c5(h)
         torch.cuda.empty_cache()
         c4 = make_c4_set(h)

@@ -244,3 +244,30 @@ def unpack_bundle(header: bytes, payload: Any, payload_bytes: Optional[int] = No
         results.append(from_dlpack_fn(exp) if from_dlpack_fn else exp)
     plan.close()
     return results
+
+
+def bundle_to_host(header: bytes, payload: Any, payload_bytes: Optional[int] = None,
+                   stream=None) -> List[Any]:
+    """The tensors of a device payload as host ``numpy`` byte arrays, one per
+    tensor: the staging a checkpoint writer needs (the reference copies buffer by
+    buffer with ``mr.memcpy(HOST, ...)``, axon/src/storage/avro_serialization.cpp:478-523).
+    The payload crosses the bus in 8 MiB pinned blocks, one device copy per block
+    whatever the tensor count.  Returns when the arrays are filled."""
+    import numpy as np
+
+    from .dlpack import TensorView
+    if isinstance(payload, PoolBuffer):
+        ptr, size = payload.data, payload.size
+    else:
+        ptr, size = int(payload), payload_bytes
+    if payload_bytes is not None:
+        size = payload_bytes
+    with BundlePlan.from_header(header) as plan:
+        metas = plan.metas()
+        arrays = [np.empty(m.nbytes, dtype=np.uint8) for m in metas]
+        views = [TensorView(data=a.ctypes.data if a.size else 0, device_type=_capi.kDLCPU, device_id=0,
+                            dtype=m.dtype, shape=tuple(m.shape), strides=None)
+                 for a, m in zip(arrays, metas)]
+        plan.bind(views)
+        plan.unpack(ptr, size, stream)
+    return arrays

@@ -189,6 +189,33 @@ inline BundlePlan UnpackTensors(const void* header, size_t header_length, const 
   return plan;
 }
 
+// A device payload as one host byte vector per tensor: what the reference's
+// checkpoint writer builds buffer by buffer with mr.memcpy(HOST, ...) per tensor
+// (axon/src/storage/avro_serialization.cpp:478-523).  Here the payload crosses the
+// bus in 8 MiB pinned blocks, one device copy per block whatever the tensor count,
+// and the pieces are cut out on the host.  Blocks until the vectors are filled.
+inline std::vector<std::vector<uint8_t>> PayloadToHost(const void* header, size_t header_length,
+                                                       const void* payload, size_t payload_bytes,
+                                                       void* stream) {
+  BundlePlan plan = BundlePlan::FromHeader(header, header_length);
+  const size_t n = plan.size();
+  std::vector<uint64_t> sizes(n);
+  Check(axr_plan_layout(plan.get(), nullptr, sizes.data()), "axr_plan_layout");
+  std::vector<std::vector<uint8_t>> out(n);
+  std::vector<axr_tensor_t> dst(n);
+  for (size_t i = 0; i < n; ++i) {
+    out[i].resize(sizes[i]);
+    Check(axr_plan_tensor_meta(plan.get(), i, &dst[i]), "axr_plan_tensor_meta");
+    dst[i].data = out[i].empty() ? nullptr : out[i].data();
+    dst[i].device_type = 1;   // kDLCPU
+    dst[i].device_id = 0;
+    dst[i].strides = nullptr;
+  }
+  plan.bind(dst.data(), n);
+  plan.unpack(payload, payload_bytes, stream);
+  return out;
+}
+
 // Zero-copy receive: views into the payload at the header's offsets.
 inline std::vector<ucx_buffer_t> SplitPayload(const void* header, size_t header_length, void* payload,
                                               size_t payload_bytes) {

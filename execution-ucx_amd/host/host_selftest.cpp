@@ -152,6 +152,17 @@ int main(int argc, char** argv) {
       mr.deallocate(ucx_memory_type::ROCM, outs[s], lens[s]);
       mr.deallocate(ucx_memory_type::ROCM, segs[s], lens[s]);
     }
+    // checkpoint path: the payload as one host vector per tensor
+    {
+      auto vecs = bundle::PayloadToHost(am.header.data, am.header.size, am.buffer.data, am.buffer.size,
+                                        nullptr);
+      EXPECT(vecs.size() == 3);
+      size_t k = 0;
+      for (int s = 0; s < 3; ++s) {
+        EXPECT(vecs[s].size() == lens[s]);
+        for (size_t i = 0; i < lens[s]; ++i, ++k) EXPECT(vecs[s][i] == static_cast<uint8_t>(k % 256));
+      }
+    }
     packed.release();
     EXPECT(mr.stats().live_blocks == 0);
 

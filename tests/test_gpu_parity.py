@@ -696,6 +696,30 @@ def test_dlpack_rocm_capsules_and_zero_copy_receive(pkg, gpu):
     assert [o.data_ptr() - base for o in outs] == packed.plan.layout()[0]   # views, not copies
 
 
+def test_bundle_to_host_for_checkpointing(pkg, orc, gpu):
+    """A packed device bundle staged to host byte arrays, one per tensor (what the
+    reference's checkpoint writer builds with one memcpy per buffer,
+    avro_serialization.cpp:478-523): 300 tensors and 40 MiB cross in 8 MiB blocks."""
+    import torch
+    rng = np.random.default_rng(21)
+    sizes = [int(x) for x in rng.integers(0, 280000, size=300)]
+    tensors = [rand_bytes_tensor(rng, n, gpu)[:n] for n in sizes]
+    tensors[7] = rand_bytes_tensor(rng, 6000, gpu).view(torch.float32).reshape(30, 50).t()   # strided source
+    bundle = pkg.pack_bundle(tensors, align=256)
+    torch.cuda.synchronize()
+    info = pkg.BundlePlan.from_header(bundle.header)
+    arrays = pkg.bundle_to_host(bundle.header, bundle.payload, bundle.payload_bytes)
+    assert len(arrays) == len(tensors)
+    for a, t in zip(arrays, tensors):
+        assert np.array_equal(a, tbytes(t))
+    # few device copies for many tensors
+    metas = info.metas()
+    assert metas[7].shape == (50, 30)
+    info.close()
+    bundle.plan.close()
+    bundle.payload.release()
+
+
 def test_pinned_host_destination(pkg, orc, gpu):
     """Scatter a device payload straight into pinned host tensors (the staging a
     checkpoint writer needs) and gather from them: the kernel addresses pinned
