@@ -152,6 +152,12 @@ class BundlePlan:
         return out
 
     # ---- data movement
+    def prepare(self, stream=None) -> "BundlePlan":
+        """Upload the device tables now; pack/unpack are then single kernel launches
+        that a HIP graph can capture."""
+        _capi.check(self._lib.axr_plan_prepare(self._h, _stream_handle(stream)))
+        return self
+
     def pack(self, payload: int, payload_bytes: int, stream=None) -> None:
         _capi.check(self._lib.axr_pack(self._h, payload, payload_bytes, _stream_handle(stream)))
 

@@ -129,6 +129,7 @@ struct axr_plan {
   size_t table_bytes = 0;
   size_t dims_at = 0, wave_at = 0;
   bool uploaded = false;
+  bool resident = false;             // upload known to be complete (axr_plan_prepare)
   hipEvent_t upload_event = nullptr;
   hipStream_t upload_stream = nullptr;
   std::vector<hipStream_t> busy_streams;   // streams with launches since the last quiesce
@@ -195,6 +196,7 @@ int check_align(uint32_t align) {
 void invalidate_tables(axr_plan* p) {
   p->tables_built = false;
   p->uploaded = false;
+  p->resident = false;
   p->segs.clear();
   p->dims.clear();
   p->wave_seg.clear();
@@ -705,6 +707,21 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   if (!pack && p->overlapping_dst)
     return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  // Under stream capture only the kernel launch may be recorded: the tables must be
+  // resident already (axr_plan_prepare) and nothing may wait on the host.
+  bool capturing = false;
+  if (stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    rc = check_hip(hipStreamIsCapturing(stream, &status), "hipStreamIsCapturing");
+    if (rc) return rc;
+    capturing = status == hipStreamCaptureStatusActive;
+  }
+  if (capturing) {
+    if (!p->host_chunks.empty())
+      return fail(AXR_ERR_UNSUPPORTED, "a bundle with host (kDLCPU) tensors cannot be captured in a graph");
+    if (p->ntiles && !p->resident)
+      return fail(AXR_ERR_INVALID, "call axr_plan_prepare before capturing this plan in a graph");
+  }
   if (!p->host_chunks.empty()) {
     rc = move_host_tensors(p, pack, static_cast<uint8_t*>(payload), stream);
     if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
@@ -712,8 +729,10 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
     if (rc) return rc;
   }
   if (p->ntiles == 0) return AXR_OK;
-  rc = ensure_uploaded(p, stream);
-  if (rc) return rc;
+  if (!p->resident) {
+    rc = ensure_uploaded(p, stream);
+    if (rc) return rc;
+  }
   KernelArgs a;
   uint8_t* d = static_cast<uint8_t*>(p->block.device);
   a.segs = reinterpret_cast<const Seg*>(d);
@@ -727,7 +746,10 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   a.seg_shift = p->cfg.seg_shift;
   rc = launch_bundle_kernel(pack, a, p->cfg, stream);
   if (rc) return rc;
-  if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+  // a capturing stream cannot be drained later; the caller keeps the plan alive
+  // for as long as the graph can run
+  if (!capturing &&
+      std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
     p->busy_streams.push_back(stream);
   return AXR_OK;
 }
@@ -1052,6 +1074,24 @@ static int plan_launch_info_body(axr_plan_t* plan, axr_launch_info_t* info) {
   info->host_chunks = static_cast<uint32_t>(plan->host_chunks.size());
   return AXR_OK;
 }
+static int plan_prepare_body(axr_plan_t* plan, void* stream_) {
+  if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_prepare: null plan");
+  if (!plan->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
+  int rc = build_tables(plan);
+  if (rc) return rc;
+  if (plan->ntiles == 0 || plan->resident) return AXR_OK;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  rc = ensure_uploaded(plan, stream);
+  if (rc) return rc;
+  rc = check_hip(hipEventSynchronize(plan->upload_event), "hipEventSynchronize(plan tables)");
+  if (rc) return rc;
+  plan->resident = true;
+  return AXR_OK;
+}
+int axr_plan_prepare(axr_plan_t* plan, void* stream) {
+  return guarded([&] { return plan_prepare_body(plan, stream); });
+}
+
 int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
   return guarded([&] { return plan_launch_info_body(plan, info); });
 }

@@ -84,6 +84,9 @@ class BundlePlan {
     return std::vector<uint8_t>(b, b + n);
   }
   void bind(const axr_tensor_t* tensors, size_t n) { Check(axr_plan_bind(plan_, tensors, n), "axr_plan_bind"); }
+  // Upload the device tables now: pack/unpack are then single kernel launches
+  // that stream capture can record into a HIP graph.
+  void prepare(void* stream) { Check(axr_plan_prepare(plan_, stream), "axr_plan_prepare"); }
   void pack(void* payload, size_t bytes, void* stream) { Check(axr_pack(plan_, payload, bytes, stream), "axr_pack"); }
   void unpack(const void* payload, size_t bytes, void* stream) {
     Check(axr_unpack(plan_, payload, bytes, stream), "axr_unpack");

@@ -274,6 +274,17 @@ AXR_API int axr_pack(axr_plan_t* plan, void* payload, size_t payload_bytes, void
 AXR_API int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes,
                        void* stream);
 
+/* Builds the plan's device tables, uploads them on `stream` and waits until they
+ * are resident.  Afterwards axr_pack / axr_unpack of this plan only launch one
+ * kernel (no allocation, no copy, no host wait), so they may be recorded into a
+ * HIP graph by stream capture; without it a capturing call fails with
+ * AXR_ERR_INVALID.  While a graph that holds such a launch can still run, the
+ * plan must stay alive and must not be rebound, and the tensors and the payload
+ * must stay where they are.  Bundles with kDLCPU tensors cannot be captured
+ * (AXR_ERR_UNSUPPORTED).  No counterpart in the reference, whose payload never
+ * passes through a kernel. */
+AXR_API int axr_plan_prepare(axr_plan_t* plan, void* stream);
+
 /* Launch geometry of a plan's kernel, for profiling reports. */
 typedef struct axr_launch_info {
   uint32_t workgroups;

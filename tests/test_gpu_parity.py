@@ -784,6 +784,63 @@ def test_plan_reuse_rebind_and_streams(pkg, orc, gpu):
         pkg._capi.check(lib.axr_stream_destroy(s))
 
 
+def test_pack_and_unpack_in_a_hip_graph(pkg, orc, gpu):
+    """A prepared plan's pack and unpack are single kernel launches that stream
+    capture can record.  The graph is replayed several times with eager work and
+    synchronisations in between, and every replay is checked against the oracle
+    for the tensors' contents at that moment."""
+    import torch
+    rng = np.random.default_rng(77)
+    sizes = [int(x) for x in rng.integers(1, 50000, size=120)]
+    tensors = [rand_bytes_tensor(rng, n, gpu) for n in sizes]
+    mat = rand_bytes_tensor(rng, 2 * 200 * 136, gpu).view(torch.int16).reshape(200, 136)
+    tensors += [mat.t(), mat[:, 8:72]]                       # transposed blocks (LDS) and short runs
+    outs = [torch.zeros_like(t, memory_format=torch.contiguous_format) for t in tensors]
+    plan = pkg.BundlePlan.create(tensors, align=256)
+    n = plan.payload_bytes
+    buf = device_bytes(n, gpu)
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+    side = torch.cuda.Stream()
+
+    # an unprepared plan refuses to be captured and records nothing
+    g0 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g0, stream=side):
+        with pytest.raises(pkg.AxonRocmError):
+            plan.pack(buf.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+    del g0
+
+    plan.prepare()
+    rplan.prepare()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        handle = torch.cuda.current_stream().cuda_stream
+        plan.pack(buf.data_ptr(), n, handle)
+        rplan.unpack(buf.data_ptr(), n, handle)
+    for replay in range(4):
+        # eager work between replays: new contents, poisoned payload and outputs
+        for t in tensors[:120]:
+            t.add_(replay + 1)
+        mat.add_(replay + 3)
+        buf.fill_(POISON)
+        for o in outs:
+            o.zero_()
+        torch.cuda.synchronize()
+        chunks = [tbytes(t) for t in tensors]
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(buf.cpu().numpy()[:n], orc.pack(chunks, 256)), replay
+        for o, c in zip(outs, chunks):
+            assert np.array_equal(tbytes(o), c), replay
+    # the same plans still work eagerly afterwards
+    buf.fill_(POISON)
+    plan.pack(buf.data_ptr(), n)
+    torch.cuda.synchronize()
+    assert np.array_equal(buf.cpu().numpy()[:n], orc.pack([tbytes(t) for t in tensors], 256))
+    del graph
+    plan.close()
+    rplan.close()
+
+
 def test_error_paths(pkg, gpu):
     import torch
     a = [torch.zeros(100, device=gpu), torch.zeros(7, device=gpu)]
