@@ -320,6 +320,20 @@ def host_bundle_c1(h, reps=30):
             "GBps_pcie_inclusive_4P": round(4.0 * nbytes / t / 1e9, 2)}
 
 
+def python_boundary(h, spec, reps=5):
+    """Planning a 4096-tensor bundle from torch tensors through the Python layer
+    (one __dlpack__() call per tensor, descriptors read in C): us per 1k tensors."""
+    from execution_ucx_amd import workloads
+    arena, tensors = workloads.materialize_mixed(spec, "cuda", seed=5)
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        plan = h.pkg.BundlePlan.create(tensors, align=256)
+        times.append(time.perf_counter() - t0)
+        plan.close()
+    return round(sorted(times)[reps // 2] * 1e6 / (len(tensors) / 1000.0), 1)
+
+
 def checkpoint_staging(h, tensors=4096, each=64 * 1024, reps=5):
     """A packed device bundle to per-tensor host buffers (pageable, already
     touched): the staged path (8 MiB pinned blocks, one device copy each, pieces
@@ -512,6 +526,7 @@ def main():
         del tr
         torch.cuda.empty_cache()
         extras["c1_host_bundle"] = host_bundle_c1(h)
+        extras["python_plan_us_per_1k_tensors"] = python_boundary(h, spec)
         extras["checkpoint_to_host"] = checkpoint_staging(h)
         extras["c5_streamed_8GiB"] = stream_c5(h)
         torch.cuda.empty_cache()

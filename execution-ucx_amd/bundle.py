@@ -60,14 +60,11 @@ class BundlePlan:
         """Sender side: ``tensors`` are DLPack producers (or TensorViews), laid
         out in argument order.  ``align=1`` is the reference's tight layout."""
         lib = _capi.load()
-        if isinstance(tensors, TensorArray):      # descriptors prepared once, reused per call
-            arr, views = tensors, tensors.views
-        else:
-            views = extract_many(tensors)
-            arr = TensorArray(views)
+        # descriptors may be prepared once and reused per call
+        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
         h = C.c_void_p()
         _capi.check(lib.axr_plan_create(arr.pointer(), arr.count, align, 0, C.byref(h)))
-        return cls(h.value, keepalive=views)
+        return cls(h.value, keepalive=arr)     # the array holds the producers' capsules
 
     @classmethod
     def from_header(cls, header: bytes) -> "BundlePlan":
@@ -78,13 +75,9 @@ class BundlePlan:
         return cls(h.value)
 
     def bind(self, tensors: Sequence[Any]) -> "BundlePlan":
-        if isinstance(tensors, TensorArray):
-            arr, views = tensors, tensors.views
-        else:
-            views = extract_many(tensors)
-            arr = TensorArray(views)
+        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
         _capi.check(self._lib.axr_plan_bind(self._h, arr.pointer(), arr.count))
-        self._keep = views
+        self._keep = arr
         return self
 
     # ---- queries

@@ -1,4 +1,4 @@
-"""DLPack in and out, without a compiled Python extension.
+"""DLPack in and out.
 
 Mirrors the reference's ``axon/python/src/dlpack_helpers.cpp``:
 
@@ -8,6 +8,12 @@ Mirrors the reference's ``axon/python/src/dlpack_helpers.cpp``:
 * ``DLPackExport`` <- DLPackCapsuleWrapper (dlpack_helpers.hpp:63-170): an
   object with ``__dlpack__`` and ``__dlpack_device__`` over memory the bundle
   path owns, consumable once by ``torch.from_dlpack`` / ``numpy.from_dlpack``.
+
+``TensorArray.from_objects`` does the extraction of a whole tensor list in C
+(``csrc/py_dlpack.c``, built as ``lib/_axr_dlpack*.so``) when that helper is
+present: one ``__dlpack__()`` call per tensor and no other per-tensor Python
+work; the pure-Python ``extract`` gives the same descriptors and serves single
+tensors, ``TensorView`` inputs and installations without the helper.
 
 kDLROCM (10), kDLROCMHost (11) and kDLCPU (1) tensors are accepted; the
 reference maps kDLROCM to ucx_memory_type::ROCM (:92-97, :123-126) but its
@@ -146,8 +152,9 @@ class TensorArray:
     """A C array of ``axr_tensor_t`` plus the shape/stride storage it points to."""
 
     def __init__(self, views: Sequence[TensorView]):
-        self.views = list(views)
-        n = len(self.views)
+        self._views = list(views)
+        self._owners = None
+        n = len(self._views)
         self.array = (_capi.Tensor * max(n, 1))()
         total = sum(v.ndim * (2 if v.strides is not None else 1) for v in self.views)
         self._dims = (C.c_int64 * max(total, 1))()
@@ -174,6 +181,57 @@ class TensorArray:
 
     def pointer(self):
         return C.cast(self.array, C.POINTER(_capi.Tensor))
+
+    @classmethod
+    def from_objects(cls, objs: Sequence[Any]) -> "TensorArray":
+        """Descriptors of DLPack producers (or ``TensorView``s)."""
+        native = _native()
+        if native is None or any(isinstance(o, TensorView) or not (
+                hasattr(o, "__dlpack__") or type(o).__name__ == "PyCapsule") for o in objs):
+            return cls(extract_many(objs))
+        descs, dims, owners = native.describe(objs)
+        self = cls.__new__(cls)
+        n = len(owners)
+        self.count = n
+        self._descs, self._dims, self._owners = descs, dims, (owners, list(objs))
+        self.array = (_capi.Tensor * max(n, 1)).from_buffer(descs) if n else (_capi.Tensor * 1)()
+        self._views = None
+        return self
+
+    @property
+    def views(self) -> List[TensorView]:
+        if self._views is None:   # native path: materialised only when somebody asks
+            owners = self._owners[0]
+            self._views = [_read(self.array[i], owners[i]) for i in range(self.count)]
+        return self._views
+
+    @views.setter
+    def views(self, value):
+        self._views = value
+
+
+_NATIVE: Any = False
+
+
+def _native():
+    """The C helper module, or None when it has not been built."""
+    global _NATIVE
+    if _NATIVE is False:
+        import glob
+        import importlib.machinery
+        import importlib.util
+        import os
+        _NATIVE = None
+        here = os.path.dirname(os.path.abspath(__file__))
+        for path in glob.glob(os.path.join(here, "lib", "_axr_dlpack*.so")):
+            loader = importlib.machinery.ExtensionFileLoader("_axr_dlpack", path)
+            spec = importlib.util.spec_from_loader("_axr_dlpack", loader)
+            mod = importlib.util.module_from_spec(spec)
+            loader.exec_module(mod)
+            if mod.TENSOR_BYTES == C.sizeof(_capi.Tensor):
+                _NATIVE = mod
+            break
+    return _NATIVE
 
 
 # ---------------------------------------------------------------- export

@@ -413,3 +413,38 @@ def test_missing_library_is_an_import_error(pkg, monkeypatch):
     monkeypatch.setattr(pkg._capi, "LIBRARY_PATH", "/nonexistent/libaxon_rocm.so")
     with pytest.raises(ImportError):
         pkg._capi.load()
+
+
+# ------------------------------------------------------------------ native DLPack extraction
+
+def test_native_extraction_matches_the_python_path(pkg):
+    """csrc/py_dlpack.c builds the same axr_tensor_t array as the ctypes reader,
+    for contiguous, strided, 0-d and empty producers (numpy and torch, CPU)."""
+    import torch
+    from execution_ucx_amd import dlpack
+    assert dlpack._native() is not None, "build lib/_axr_dlpack*.so with `make -C execution-ucx_amd`"
+    base = np.arange(5 * 7 * 3, dtype=np.float32).reshape(5, 7, 3)
+    objs = [base, base[1:4, ::2], np.zeros((0, 4), np.int16), np.array(3.0),
+            torch.arange(24, dtype=torch.int64).reshape(2, 3, 4).permute(2, 0, 1),
+            torch.zeros(17, dtype=torch.bfloat16)]
+    native = dlpack.TensorArray.from_objects(objs)
+    python = dlpack.TensorArray(dlpack.extract_many(objs))
+    assert native.count == python.count == len(objs)
+    fields = ("data", "device_type", "device_id", "ndim", "dtype_code", "dtype_bits", "dtype_lanes",
+              "byte_offset")
+    for i in range(native.count):
+        a, b = native.array[i], python.array[i]
+        assert [getattr(a, f) for f in fields] == [getattr(b, f) for f in fields], i
+        assert [a.shape[d] for d in range(a.ndim)] == [b.shape[d] for d in range(b.ndim)]
+        assert bool(a.strides) == bool(b.strides)
+        if a.strides:
+            assert [a.strides[d] for d in range(a.ndim)] == [b.strides[d] for d in range(b.ndim)]
+    assert [v.shape for v in native.views] == [v.shape for v in python.views]
+    # both give the same plan
+    assert pkg.BundlePlan.create(objs, align=64).header == \
+        pkg.BundlePlan.create(dlpack.extract_many(objs), align=64).header
+    # TensorViews and foreign objects take the Python path / fail as before
+    mixed = dlpack.TensorArray.from_objects([objs[0], dlpack.extract(objs[1])])
+    assert mixed.count == 2
+    with pytest.raises(TypeError):
+        dlpack.TensorArray.from_objects([object()])
