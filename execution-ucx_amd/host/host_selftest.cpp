@@ -164,7 +164,36 @@ int main(int argc, char** argv) {
       }
     }
     packed.release();
+    packed.release();   // idempotent, like a moved-from UcxBuffer
     EXPECT(mr.stats().live_blocks == 0);
+
+    // ownership (the release-function rules of ucx_context_data_test.cpp:85-128):
+    // a detached block is no longer released by the bundle, an owned one exactly once
+    {
+      std::vector<uint8_t> fill(4096, 7);
+      void* seg = mr.allocate(ucx_memory_type::ROCM, fill.size());
+      mr.memcpy(ucx_memory_type::ROCM, seg, ucx_memory_type::HOST, fill.data(), fill.size());
+      int64_t shape = static_cast<int64_t>(fill.size());
+      axr_tensor_t one = Tensor1D(seg, &shape, 10, 1, 8);
+      void* kept = nullptr;
+      size_t kept_bytes = 0;
+      {
+        bundle::TensorBundle b = bundle::PackTensors(mr, &one, 1, 256, nullptr);
+        EXPECT(axr_device_synchronize() == AXR_OK);
+        kept_bytes = b.payload_bytes();
+        kept = b.detach();
+      }   // destructor runs: nothing to release
+      EXPECT(mr.stats().live_blocks == 2);
+      {
+        bundle::TensorBundle b = bundle::PackTensors(mr, &one, 1, 256, nullptr);
+        bundle::TensorBundle moved = std::move(b);
+        EXPECT(b.payload() == nullptr && moved.payload() != nullptr);
+      }   // released once, by the moved-to object
+      EXPECT(mr.stats().live_blocks == 2);
+      mr.deallocate(ucx_memory_type::ROCM, kept, kept_bytes);
+      mr.deallocate(ucx_memory_type::ROCM, seg, fill.size());
+      EXPECT(mr.stats().live_blocks == 0);
+    }
 
     // unsupported types throw std::runtime_error like the reference's manager
     bool threw = false;

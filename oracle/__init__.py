@@ -90,6 +90,9 @@ def ref_lib() -> Optional[C.CDLL]:
         L.ref_time_pack_unpack.argtypes = [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                            C.POINTER(C.c_uint64), C.c_size_t, C.c_void_p,
                                            C.c_int, C.c_int]
+        if hasattr(L, "ref_release_count"):
+            L.ref_release_count.restype = C.c_int
+            L.ref_release_count.argtypes = [C.c_int]
         _ref = L
     return _ref
 

@@ -72,6 +72,29 @@ __attribute__((visibility("default"))) int ref_split(void* base, uint64_t size,
   }
 }
 
+// Release-function ownership of the live UcxBuffer, the scenario of
+// ucx_context_data_test.cpp:85-128: an external 16-byte block with a release
+// callback is moved into a second buffer with own_buffer = `own`.  Returns how
+// often the callback ran once both buffers are gone, or a negative number when
+// an intermediate state differs from what that test expects.
+__attribute__((visibility("default"))) int ref_release_count(int own) {
+  int release_count = 0;
+  auto* external = new uint8_t[16];
+  int state = 0;
+  {
+    UcxBuffer buffer(mr(), ucx_memory_type::HOST, external, 16, nullptr, true,
+                     [&release_count](void* ptr) {
+                       ++release_count;
+                       delete[] static_cast<uint8_t*>(ptr);
+                     });
+    auto moved = UcxBuffer(std::move(buffer), own != 0);
+    if (buffer.data() != nullptr || buffer.own_buffer()) state = -1;
+    if (moved.data() != external || moved.own_buffer() != (own != 0)) state = -2;
+  }
+  if (!own) delete[] external;
+  return state ? state : release_count;
+}
+
 // Median seconds of one pack + unpack through the reference memcpy dispatch.
 __attribute__((visibility("default"))) double ref_time_pack_unpack(
     const void* const* srcs, void* const* dsts, const uint64_t* sizes, size_t n, void* packed,

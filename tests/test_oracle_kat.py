@@ -73,6 +73,16 @@ def test_split_matches_compiled_reference(orc):
             assert list(vs[:n]) == sizes
 
 
+def test_release_function_ownership_kat(orc):
+    """ucx_context_data_test.cpp:85-128 on the compiled UcxBuffer: a release callback
+    moved with own_buffer=true runs exactly once, moved with own_buffer=false never."""
+    ref = orc.ref_lib()
+    if ref is None:
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    assert ref.ref_release_count(1) == 1
+    assert ref.ref_release_count(0) == 0
+
+
 # ---- pack = ordered tight concat --------------------------------------------
 
 @pytest.mark.parametrize("lens", [(256, 512, 300),                       # ucx_am_connection_test.cpp:933-994
