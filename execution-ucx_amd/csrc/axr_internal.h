@@ -49,10 +49,15 @@ constexpr uint32_t kModeRunTiles = 0;   // every tile is a piece of one contiguo
 constexpr uint32_t kModeElements = 1;   // tile covers packed bytes; lanes decode granules
 constexpr uint32_t kModeTranspose = 2;  // tile is a square block transposed through LDS
 
-// Transposed tiles are T x T elements with T = kTransposeRowBytes / element size,
-// so that a tile row is 128 bytes (eight 16-byte vectors) on both sides.
-constexpr uint32_t kTransposeRowBytes = 128;
-constexpr uint32_t kTransposeLdsPitch = kTransposeRowBytes + 4;   // one dword of padding per row
+// Transposed blocks are T x T elements; a block row is 128 bytes (eight 16-byte
+// vectors) for elements up to 4 bytes and 256 bytes for wider ones, so that a
+// block is 4 to 16 KiB.  In LDS every row carries one dword of padding.
+constexpr uint32_t transpose_edge(uint32_t element_bytes) {
+  return (element_bytes <= 4 ? 128u : 256u) / element_bytes;   // 128, 64, 32, 32, 16
+}
+constexpr uint32_t transpose_lds_pitch(uint32_t element_bytes) {
+  return transpose_edge(element_bytes) * element_bytes + 4u;
+}
 constexpr uint32_t kMaxBatchDims = 4;
 constexpr uint32_t kMinElementTileBytes = 8192;   // element-mode work unit (measured: 8 KiB beats 2, 4 and 16)
 

@@ -289,12 +289,15 @@ template <uint32_t E>
 __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gbytes wr,
                                                int64_t wr_pitch, lbytes lds, uint32_t lane,
                                                bool nt_rd, bool nt_wr) {
-  constexpr uint32_t T = kTransposeRowBytes / E, NK = T / 8, EV = kVecBytes / E;
+  constexpr uint32_t T = transpose_edge(E), PITCH = transpose_lds_pitch(E), EV = kVecBytes / E;
+  constexpr uint32_t NC = T * E / kVecBytes;   // vectors per block row: 8 or 16
+  constexpr uint32_t RPI = kWaveLanes / NC;    // block rows one wave-wide access covers
+  constexpr uint32_t NK = T / RPI;
   typedef typename unit_of<E>::type U;
   typedef U __attribute__((aligned(E < 4 ? E : 4))) lds_unit;
   // at most eight vectors per lane in flight: a block of bytes (128 rows) moves in two halves
   constexpr uint32_t B = NK < 8 ? NK : 8;
-  const uint32_t r8 = lane >> 3, v = lane & 7;
+  const uint32_t r8 = lane / NC, v = lane % NC;
   // The cache hints are wave-uniform: one branch around each batch, not per access.
   // The empty asm statements keep the two arms distinct: without them the optimizer
   // merges the arms' identical accesses and the hint is lost.
@@ -305,17 +308,17 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
       asm volatile("");
 #pragma unroll
       for (uint32_t k = 0; k < B; ++k)
-        x[k] = load16<true>(rd + static_cast<int64_t>((kb + k) * 8 + r8) * rd_pitch + v * kVecBytes);
+        x[k] = load16<true>(rd + static_cast<int64_t>((kb + k) * RPI + r8) * rd_pitch + v * kVecBytes);
       asm volatile("");
     } else {
 #pragma unroll
       for (uint32_t k = 0; k < B; ++k)
-        x[k] = load16<false>(rd + static_cast<int64_t>((kb + k) * 8 + r8) * rd_pitch + v * kVecBytes);
+        x[k] = load16<false>(rd + static_cast<int64_t>((kb + k) * RPI + r8) * rd_pitch + v * kVecBytes);
     }
 #pragma unroll
     for (uint32_t k = 0; k < B; ++k) {
       AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(
-          lds + ((kb + k) * 8 + r8) * kTransposeLdsPitch + v * kVecBytes);
+          lds + ((kb + k) * RPI + r8) * PITCH + v * kVecBytes);
       w[0] = x[k].x;
       w[1] = x[k].y;
       w[2] = x[k].z;
@@ -328,23 +331,23 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
     u32x4 out[B];
 #pragma unroll
     for (uint32_t k = 0; k < B; ++k) {
-      const uint32_t c = (kb + k) * 8 + r8;
+      const uint32_t c = (kb + k) * RPI + r8;
       U e[EV];
 #pragma unroll
       for (uint32_t i = 0; i < EV; ++i)
-        e[i] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + (v * EV + i) * kTransposeLdsPitch + c * E);
+        e[i] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + (v * EV + i) * PITCH + c * E);
       __builtin_memcpy(&out[k], e, kVecBytes);
     }
     if (nt_wr) {
       asm volatile("");
 #pragma unroll
       for (uint32_t k = 0; k < B; ++k)
-        store16<true>(wr + static_cast<int64_t>((kb + k) * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
+        store16<true>(wr + static_cast<int64_t>((kb + k) * RPI + r8) * wr_pitch + v * kVecBytes, out[k]);
       asm volatile("");
     } else {
 #pragma unroll
       for (uint32_t k = 0; k < B; ++k)
-        store16<false>(wr + static_cast<int64_t>((kb + k) * 8 + r8) * wr_pitch + v * kVecBytes, out[k]);
+        store16<false>(wr + static_cast<int64_t>((kb + k) * RPI + r8) * wr_pitch + v * kVecBytes, out[k]);
     }
   }
   __builtin_amdgcn_wave_barrier();
@@ -415,9 +418,10 @@ __device__ __forceinline__ uint32_t small_div(uint32_t idx, uint32_t d, uint32_t
 
 // Partial or misaligned block: the same two phases one element per lane.  Both
 // global sides still see consecutive lanes on consecutive elements.
-__device__ __forceinline__ void transpose_edge(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
+__device__ __forceinline__ void transpose_partial(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
                                                int64_t wr_pitch, uint32_t nr, uint32_t nc,
                                                lbytes lds, uint32_t lane) {
+  const uint32_t lds_pitch = transpose_lds_pitch(E);
   const uint32_t total = nr * nc;
   const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
   const uint32_t mc = 0xffffffffu / nc + 1u, mr = 0xffffffffu / nr + 1u;
@@ -425,13 +429,13 @@ __device__ __forceinline__ void transpose_edge(uint32_t E, gcbytes rd, int64_t r
     const uint32_t r = small_div(i, nc, mc);
     const uint32_t c = i - r * nc;
     lds_put(E, rd + static_cast<int64_t>(r) * rd_pitch + (c << es),
-            lds + r * kTransposeLdsPitch + (c << es));
+            lds + r * lds_pitch + (c << es));
   }
   __builtin_amdgcn_wave_barrier();
   for (uint32_t i = lane; i < total; i += kWaveLanes) {
     const uint32_t c = small_div(i, nr, mr);
     const uint32_t r = i - c * nr;
-    lds_get(E, lds + r * kTransposeLdsPitch + (c << es),
+    lds_get(E, lds + r * lds_pitch + (c << es),
             wr + static_cast<int64_t>(c) * wr_pitch + (r << es));
   }
   __builtin_amdgcn_wave_barrier();
@@ -442,10 +446,9 @@ __device__ __forceinline__ void transpose_edge(uint32_t E, gcbytes rd, int64_t r
 __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
                                                 int64_t wr_pitch, uint32_t nr, uint32_t nc,
                                                 lbytes lds, uint32_t lane, bool nt_rd, bool nt_wr) {
-  const uint32_t T = kTransposeRowBytes >> __builtin_ctz(E);
-  const uint64_t bits = reinterpret_cast<uintptr_t>(rd) | static_cast<uint64_t>(rd_pitch) |
-                        reinterpret_cast<uintptr_t>(wr) | static_cast<uint64_t>(wr_pitch);
-  if (nr == T && nc == T && (bits & 15u) == 0) {
+  // Whole blocks take the vector path whatever the alignment of the two sides
+  // (global 16-byte accesses need none; the LDS side is always aligned).
+  if (nr == transpose_edge(E) && nc == transpose_edge(E)) {
     switch (E) {
       case 1: transpose_full<1>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
       case 2: transpose_full<2>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
@@ -454,7 +457,7 @@ __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t 
       default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
     }
   } else {
-    transpose_edge(E, rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane);
+    transpose_partial(E, rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane);
   }
 }
 
@@ -465,7 +468,7 @@ __device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, 
                                                uint32_t nt_bits) {
   const uint32_t E = dm->granule;
   const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
-  const uint32_t T = kTransposeRowBytes >> es;
+  const uint32_t T = transpose_edge(E);
   const uint32_t ta = dm->tiles_a, tb = dm->tiles_b;
   const uint32_t per_batch = ta * tb;
   uint32_t o = q / per_batch;

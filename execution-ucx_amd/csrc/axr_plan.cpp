@@ -357,7 +357,7 @@ struct Builder {
     }
     if (dim_b < nd) {
       const uint32_t e = static_cast<uint32_t>(run_bytes);
-      const uint32_t t = kTransposeRowBytes / e;
+      const uint32_t t = transpose_edge(e);
       const size_t dim_a = nd - 1;
       dm.mode = kModeTranspose;
       dm.granule = e;
@@ -393,7 +393,7 @@ struct Builder {
       if (per_batch > 0xffffffffull || batches > 0xffffffffull / per_batch)
         return fail(AXR_ERR_UNSUPPORTED, "transposed tensor has too many blocks");
       ntile = batches * per_batch;
-      p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, t * kTransposeLdsPitch);
+      p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, t * transpose_lds_pitch(e));
     } else if (run_bytes >= element_mode_limit(run_bytes)) {
       dm.mode = kModeRunTiles;
       const uint64_t tpr = (run_bytes + tile_bytes - 1) / tile_bytes;

@@ -213,7 +213,8 @@ def views_of_torch(tensors: Sequence) -> List[TensorView]:
     code = {torch.float16: (kDLFloat, 16, 1), torch.bfloat16: (kDLBfloat, 16, 1),
             torch.float32: (kDLFloat, 32, 1), torch.float64: (kDLFloat, 64, 1),
             torch.int32: (kDLInt, 32, 1), torch.int8: (kDLInt, 8, 1), torch.int16: (kDLInt, 16, 1),
-            torch.int64: (kDLInt, 64, 1), torch.uint8: (1, 8, 1), torch.bool: (6, 8, 1)}
+            torch.int64: (kDLInt, 64, 1), torch.uint8: (1, 8, 1), torch.bool: (6, 8, 1),
+            torch.complex64: (5, 64, 1), torch.complex128: (5, 128, 1)}
     out = []
     for t in tensors:
         dev = _capi.kDLROCM if t.is_cuda else _capi.kDLCPU

@@ -428,7 +428,7 @@ def test_transposed_views(pkg, orc, gpu, dtype_name):
     import torch
     dt = getattr(torch, dtype_name)
     item = torch.empty((), dtype=dt).element_size()
-    t = 128 // item                                            # block edge in elements
+    t = (128 if item <= 4 else 256) // item                    # block edge in elements
     rng = np.random.default_rng(100 + item)
 
     def parent_of(shape):

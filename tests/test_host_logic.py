@@ -279,9 +279,11 @@ def test_transposed_views_use_square_blocks(pkg):
     # tiny extents and odd element sizes stay in element mode
     assert seg_of(pkg, tv(pkg, 0x10000, [30, 4], strides=[1, 30]))[0][0]["mode"] == 2
     assert seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(2, 96, 1)))[0][0]["mode"] == 2
-    # 16-byte elements transpose as 8 x 8 blocks
+    # 16-byte elements transpose as 16 x 16 blocks, 8-byte ones as 32 x 32
     s = seg_of(pkg, tv(pkg, 0x10000, [30, 20], strides=[1, 30], dtype=(2, 128, 1)))[0][0]
-    assert (s["mode"], s["granule"], s["tiles"]) == (5, 16, 4 * 3)
+    assert (s["mode"], s["granule"], s["tiles"]) == (5, 16, 2 * 2)
+    s = seg_of(pkg, tv(pkg, 0x10000, [70, 40], strides=[1, 70], dtype=(2, 64, 1)))[0][0]
+    assert (s["mode"], s["granule"], s["tiles"]) == (5, 8, 3 * 2)
 
 
 def test_negative_and_many_strides(pkg):
