@@ -243,7 +243,10 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
         uint32_t v = idx0[d] + carry;
         uint32_t c = 0;
         if (__builtin_amdgcn_ballot_w64(v >= extent) != 0) {
-          c = v / extent;
+          // v < extent + 2^14: for extents below 2^15 the multiply-high quotient is
+          // exact (v * extent < 2^32)
+          c = extent < 32768u ? __umulhi(v, 0xffffffffu / extent + 1u) : v / extent;
+          c = extent == 1 ? v : c;
           v -= c * extent;
         }
         toff += static_cast<int64_t>(static_cast<int32_t>(v - idx0[d])) * dm->stride[d];
@@ -506,8 +509,11 @@ __device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, 
   }
 }
 
+// At least four waves per SIMD (at most 128 VGPRs): the streaming instantiations
+// use far fewer, and the general ones sit just around that limit, where one
+// register too many would cost a quarter of the occupancy.
 template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
-__global__ __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
+__global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
     const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
     uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
     uint32_t lds_per_wave, uint32_t nt_bits) {
