@@ -58,10 +58,14 @@ constexpr uint32_t transpose_edge(uint32_t element_bytes) {
 constexpr uint32_t transpose_lds_pitch(uint32_t element_bytes) {
   return transpose_edge(element_bytes) * element_bytes + 4u;
 }
+// When one of the two block dimensions is shorter than a square block's edge the
+// block becomes a rectangle of about this many bytes, its long edge capped.
+constexpr uint32_t kRectBlockBytes = 8192;
+constexpr uint32_t kRectMaxEdge = 1024;
 constexpr uint32_t kMaxBatchDims = 4;
 constexpr uint32_t kMinElementTileBytes = 8192;   // element-mode work unit (measured: 8 KiB beats 2, 4 and 16)
 
-struct Dims {             // 160 bytes, one per strided segment
+struct Dims {             // 176 bytes, one per strided segment
   uint32_t mode;
   uint32_t ndim;          // outer (non-run) dimensions after collapsing, <= kMaxOuterDims;
                           // kModeTranspose: batch dimensions (<= kMaxBatchDims)
@@ -79,8 +83,10 @@ struct Dims {             // 160 bytes, one per strided segment
   uint64_t pstride_b;              // packed byte stride of B
   uint32_t ext_a, ext_b;
   uint32_t tiles_a, tiles_b;
+  uint32_t edge_a, edge_b;         // block extent along A and B (elements)
+  uint32_t reserved[2];
 };
-static_assert(sizeof(Dims) == 160, "Dims layout");
+static_assert(sizeof(Dims) == 176, "Dims layout");
 
 struct KernelArgs {
   const Seg* segs;            // nseg + 1 entries, last is a sentinel with tile_begin == ntiles

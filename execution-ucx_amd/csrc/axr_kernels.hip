@@ -356,90 +356,61 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
   __builtin_amdgcn_wave_barrier();
 }
 
-__device__ __forceinline__ void lds_put(uint32_t E, gcbytes src, lbytes dst) {
-  switch (E) {
-    case 16: {
-      typedef u32x4 __attribute__((aligned(1))) gl;
-      const u32x4 x = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
-      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(dst);
-      w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
-      break;
-    }
-    case 8: {
-      typedef uint64_t __attribute__((aligned(1))) gl;
-      typedef uint64_t __attribute__((aligned(4))) ll;
-      *reinterpret_cast<AXR_LDS ll*>(dst) = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
-      break;
-    }
-    case 4: {
-      typedef uint32_t __attribute__((aligned(1))) gl;
-      *reinterpret_cast<AXR_LDS uint32_t*>(dst) = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
-      break;
-    }
-    case 2: {
-      typedef uint16_t __attribute__((aligned(1))) gl;
-      *reinterpret_cast<AXR_LDS uint16_t*>(dst) = *reinterpret_cast<const AXR_GLOBAL gl*>(src);
-      break;
-    }
-    default: *dst = *src; break;
-  }
-}
-
-__device__ __forceinline__ void lds_get(uint32_t E, const AXR_LDS uint8_t* src, gbytes dst) {
-  switch (E) {
-    case 16: {
-      typedef u32x4 __attribute__((aligned(1))) gl;
-      const AXR_LDS uint32_t* r = reinterpret_cast<const AXR_LDS uint32_t*>(src);
-      const u32x4 x = {r[0], r[1], r[2], r[3]};
-      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = x;
-      break;
-    }
-    case 8: {
-      typedef uint64_t __attribute__((aligned(1))) gl;
-      typedef uint64_t __attribute__((aligned(4))) ll;
-      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = *reinterpret_cast<const AXR_LDS ll*>(src);
-      break;
-    }
-    case 4: {
-      typedef uint32_t __attribute__((aligned(1))) gl;
-      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = *reinterpret_cast<const AXR_LDS uint32_t*>(src);
-      break;
-    }
-    case 2: {
-      typedef uint16_t __attribute__((aligned(1))) gl;
-      *reinterpret_cast<AXR_GLOBAL gl*>(dst) = *reinterpret_cast<const AXR_LDS uint16_t*>(src);
-      break;
-    }
-    default: *dst = *src; break;
-  }
-}
-
-// Quotient idx / d for idx < 2^14, d <= 128, by multiplication (exact in that range).
+// Quotient idx / d by multiplication, exact while idx * d < 2^32 (blocks hold at
+// most 2^14 elements with edges up to 2^10).
 __device__ __forceinline__ uint32_t small_div(uint32_t idx, uint32_t d, uint32_t magic) {
   return d == 1 ? idx : __umulhi(idx, magic);
 }
 
-// Partial or misaligned block: the same two phases one element per lane.  Both
-// global sides still see consecutive lanes on consecutive elements.
-__device__ __forceinline__ void transpose_partial(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
-                                               int64_t wr_pitch, uint32_t nr, uint32_t nc,
-                                               lbytes lds, uint32_t lane) {
-  const uint32_t lds_pitch = transpose_lds_pitch(E);
+// Partial or rectangular block: the same two phases one element per lane, eight
+// elements per lane in flight.  Both global sides still see consecutive lanes on
+// consecutive elements.  Rows in LDS are nc elements plus one dword apart.
+template <uint32_t E>
+__device__ __forceinline__ void transpose_partial(gcbytes rd, int64_t rd_pitch, gbytes wr,
+                                                  int64_t wr_pitch, uint32_t nr, uint32_t nc,
+                                                  lbytes lds, uint32_t lane) {
+  typedef typename unit_of<E>::type U;
+  typedef U __attribute__((aligned(1))) global_unit;
+  typedef U __attribute__((aligned(E < 4 ? E : 4))) lds_unit;
+  constexpr uint32_t B = E == 16 ? 4 : 8;   // elements per lane and round
+  const uint32_t lds_pitch = nc * E + 4u;
   const uint32_t total = nr * nc;
-  const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
   const uint32_t mc = 0xffffffffu / nc + 1u, mr = 0xffffffffu / nr + 1u;
-  for (uint32_t i = lane; i < total; i += kWaveLanes) {
-    const uint32_t r = small_div(i, nc, mc);
-    const uint32_t c = i - r * nc;
-    lds_put(E, rd + static_cast<int64_t>(r) * rd_pitch + (c << es),
-            lds + r * lds_pitch + (c << es));
+  for (uint32_t i0 = lane; i0 < total; i0 += B * kWaveLanes) {
+    U x[B];
+    uint32_t at[B];
+#pragma unroll
+    for (uint32_t k = 0; k < B; ++k) {
+      const uint32_t i = i0 + k * kWaveLanes;
+      const uint32_t ic = i < total ? i : total - 1u;   // slots past the end repeat the last element
+      const uint32_t r = small_div(ic, nc, mc);
+      const uint32_t c = ic - r * nc;
+      at[k] = r * lds_pitch + c * E;
+      x[k] = *reinterpret_cast<const AXR_GLOBAL global_unit*>(rd + static_cast<int64_t>(r) * rd_pitch + c * E);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < B; ++k) *reinterpret_cast<AXR_LDS lds_unit*>(lds + at[k]) = x[k];
   }
   __builtin_amdgcn_wave_barrier();
-  for (uint32_t i = lane; i < total; i += kWaveLanes) {
-    const uint32_t c = small_div(i, nr, mr);
-    const uint32_t r = i - c * nr;
-    lds_get(E, lds + r * lds_pitch + (c << es),
-            wr + static_cast<int64_t>(c) * wr_pitch + (r << es));
+  for (uint32_t i0 = lane; i0 < total; i0 += B * kWaveLanes) {
+    U x[B];
+#pragma unroll
+    for (uint32_t k = 0; k < B; ++k) {
+      const uint32_t i = i0 + k * kWaveLanes;
+      const uint32_t ic = i < total ? i : total - 1u;
+      const uint32_t c = small_div(ic, nr, mr);
+      const uint32_t r = ic - c * nr;
+      x[k] = *reinterpret_cast<const AXR_LDS lds_unit*>(lds + r * lds_pitch + c * E);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < B; ++k) {
+      const uint32_t i = i0 + k * kWaveLanes;
+      if (i < total) {
+        const uint32_t c = small_div(i, nr, mr);
+        const uint32_t r = i - c * nr;
+        *reinterpret_cast<AXR_GLOBAL global_unit*>(wr + static_cast<int64_t>(c) * wr_pitch + r * E) = x[k];
+      }
+    }
   }
   __builtin_amdgcn_wave_barrier();
 }
@@ -448,10 +419,11 @@ __device__ __forceinline__ void transpose_partial(uint32_t E, gcbytes rd, int64_
 // nr elements (rows wr_pitch bytes apart).
 __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
                                                 int64_t wr_pitch, uint32_t nr, uint32_t nc,
-                                                lbytes lds, uint32_t lane, bool nt_rd, bool nt_wr) {
+                                                bool square, lbytes lds, uint32_t lane, bool nt_rd,
+                                                bool nt_wr) {
   // Whole blocks take the vector path whatever the alignment of the two sides
   // (global 16-byte accesses need none; the LDS side is always aligned).
-  if (nr == transpose_edge(E) && nc == transpose_edge(E)) {
+  if (square) {
     switch (E) {
       case 1: transpose_full<1>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
       case 2: transpose_full<2>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
@@ -460,7 +432,13 @@ __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t 
       default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
     }
   } else {
-    transpose_partial(E, rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane);
+    switch (E) {
+      case 1: transpose_partial<1>(rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane); break;
+      case 2: transpose_partial<2>(rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane); break;
+      case 4: transpose_partial<4>(rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane); break;
+      case 8: transpose_partial<8>(rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane); break;
+      default: transpose_partial<16>(rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane); break;
+    }
   }
 }
 
@@ -472,6 +450,7 @@ __device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, 
   const uint32_t E = dm->granule;
   const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
   const uint32_t T = transpose_edge(E);
+  const uint32_t edge_a = dm->edge_a, edge_b = dm->edge_b;
   const uint32_t ta = dm->tiles_a, tb = dm->tiles_b;
   const uint32_t per_batch = ta * tb;
   uint32_t o = q / per_batch;
@@ -492,19 +471,20 @@ __device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, 
       o = next;
     }
   }
-  const uint32_t a0 = ia * T, b0 = ib * T;
+  const uint32_t a0 = ia * edge_a, b0 = ib * edge_b;
   const uint32_t ra = dm->ext_a - a0, rb = dm->ext_b - b0;
-  const uint32_t na = ra < T ? ra : T, nb = rb < T ? rb : T;
+  const uint32_t na = ra < edge_a ? ra : edge_a, nb = rb < edge_b ? rb : edge_b;
+  const bool square = na == T && nb == T;   // a whole square block: the vector path
   const int64_t stride_a = dm->stride_a;
   const uint64_t pstride_b = dm->pstride_b;
   gbytes ten = as_global(seg_ptr) + toff + static_cast<int64_t>(a0) * stride_a +
                (static_cast<uint64_t>(b0) << es);
   gbytes pp = pay + poff + static_cast<uint64_t>(b0) * pstride_b + (static_cast<uint64_t>(a0) << es);
   if constexpr (PACK) {
-    transpose_block(E, ten, stride_a, pp, static_cast<int64_t>(pstride_b), na, nb, lds, lane,
+    transpose_block(E, ten, stride_a, pp, static_cast<int64_t>(pstride_b), na, nb, square, lds, lane,
                     (nt_bits & 1u) != 0, (nt_bits & 2u) != 0);
   } else {
-    transpose_block(E, pp, static_cast<int64_t>(pstride_b), ten, stride_a, nb, na, lds, lane,
+    transpose_block(E, pp, static_cast<int64_t>(pstride_b), ten, stride_a, nb, na, square, lds, lane,
                     (nt_bits & 2u) != 0, (nt_bits & 1u) != 0);
   }
 }

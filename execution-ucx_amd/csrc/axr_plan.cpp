@@ -346,18 +346,37 @@ struct Builder {
     // A transposition: no contiguous inner run beyond one element, but some outer
     // dimension (B) is contiguous in the tensor.  Blocks of A x B go through LDS.
     size_t dim_b = nd;
+    uint32_t edge_a = 0, edge_b = 0;
     if (nd >= 2 && run_bytes <= kVecBytes && (run_bytes & (run_bytes - 1)) == 0 &&
-        tunables().transpose != 0 && ext[nd - 1] >= 8) {
+        tunables().transpose != 0) {
       for (size_t d = 0; d + 1 < nd; ++d) {
-        if (str[d] == static_cast<int64_t>(run_bytes) && ext[d] >= 8) {
+        if (str[d] == static_cast<int64_t>(run_bytes)) {
           dim_b = d;
           break;
         }
       }
     }
     if (dim_b < nd) {
+      // Square blocks when both dimensions reach a block edge; otherwise the short
+      // dimension is taken whole (up to an edge) and the other one stretches until
+      // the block holds about 8 KiB.  Blocks under 1 KiB are not worth a wave:
+      // such views stay in element mode.
       const uint32_t e = static_cast<uint32_t>(run_bytes);
-      const uint32_t t = transpose_edge(e);
+      const uint64_t t = transpose_edge(e), ea = ext[nd - 1], eb = ext[dim_b];
+      const uint64_t elems = kRectBlockBytes / e;
+      if (ea >= t && eb >= t) {
+        edge_a = edge_b = static_cast<uint32_t>(t);
+      } else if (ea <= eb) {
+        edge_a = static_cast<uint32_t>(std::min(ea, t));
+        edge_b = static_cast<uint32_t>(std::min<uint64_t>({eb, kRectMaxEdge, elems / edge_a}));
+      } else {
+        edge_b = static_cast<uint32_t>(std::min(eb, t));
+        edge_a = static_cast<uint32_t>(std::min<uint64_t>({ea, kRectMaxEdge, elems / edge_b}));
+      }
+      if (static_cast<uint64_t>(edge_a) * edge_b * e < 1024) dim_b = nd;
+    }
+    if (dim_b < nd) {
+      const uint32_t e = static_cast<uint32_t>(run_bytes);
       const size_t dim_a = nd - 1;
       dm.mode = kModeTranspose;
       dm.granule = e;
@@ -387,13 +406,17 @@ struct Builder {
       dm.pstride_b = packed[dim_b];
       dm.ext_a = static_cast<uint32_t>(ext[dim_a]);
       dm.ext_b = static_cast<uint32_t>(ext[dim_b]);
-      dm.tiles_a = (dm.ext_a + t - 1) / t;
-      dm.tiles_b = (dm.ext_b + t - 1) / t;
+      dm.edge_a = edge_a;
+      dm.edge_b = edge_b;
+      dm.tiles_a = (dm.ext_a + edge_a - 1) / edge_a;
+      dm.tiles_b = (dm.ext_b + edge_b - 1) / edge_b;
       const uint64_t per_batch = static_cast<uint64_t>(dm.tiles_a) * dm.tiles_b;
       if (per_batch > 0xffffffffull || batches > 0xffffffffull / per_batch)
         return fail(AXR_ERR_UNSUPPORTED, "transposed tensor has too many blocks");
       ntile = batches * per_batch;
-      p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, t * transpose_lds_pitch(e));
+      // rows of one side plus a dword each, whichever direction needs more
+      const uint32_t lds = edge_a * edge_b * e + 4u * std::max(edge_a, edge_b);
+      p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, (lds + 15u) & ~15u);
     } else if (run_bytes >= element_mode_limit(run_bytes)) {
       dm.mode = kModeRunTiles;
       const uint64_t tpr = (run_bytes + tile_bytes - 1) / tile_bytes;

@@ -439,7 +439,14 @@ def test_transposed_views(pkg, orc, gpu, dtype_name):
     m3 = parent_of([t + 5, 2 * t + 3])
     m4 = parent_of([3, 20, 2, 24])
     m5 = parent_of([2, 9, 70])
+    m6 = parent_of([4, 3, 20, 30])                              # NCHW
+    m7 = parent_of([4, 20, 30, 3])                              # NHWC
+    m8 = parent_of([3000, 2])
     cases = [
+        (m6, m6.permute(0, 2, 3, 1)),                          # channels last: 3 x 600 rectangles
+        (m7, m7.permute(0, 3, 1, 2)),                          # and back
+        (m8, m8.t()),                                          # interleaved pairs to two planes
+        (m8, m8[5:2900:1].t()),
         (m2, m2.t()),                                          # whole aligned blocks only
         (m3, m3.t()),                                          # ragged in both directions
         (m3, m3[1:, 3:].t()),                                  # base off the 16-byte grid
@@ -452,7 +459,7 @@ def test_transposed_views(pkg, orc, gpu, dtype_name):
     views = [v for _, v in cases]
     plan = pkg.BundlePlan.create(views, align=256)
     modes = [s["mode"] for s in plan.segments()]
-    assert modes.count(5) >= 5, modes
+    assert modes.count(5) >= 9, modes
     chunks = []
     for parent, v in cases:
         host_parent = parent.reshape(-1).view(torch.uint8).cpu().numpy()
