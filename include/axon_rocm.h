@@ -156,7 +156,9 @@ AXR_API int axr_event_elapsed_ms(void* start, void* stop, float* ms);
 AXR_API int axr_mem_alloc(int memory_type, size_t bytes, size_t alignment, void** ptr);
 AXR_API int axr_mem_free(int memory_type, void* ptr, size_t bytes);
 /* Blocking copy between any two of HOST / ROCM / ROCM_MANAGED; the table
- * of ucx_cuda_memory_manager.hpp:62-78 extended with the pinned type. */
+ * of ucx_cuda_memory_manager.hpp:62-78 extended with the pinned type.  ROCM to
+ * HOST copies of 16 MiB and more go through two pinned staging blocks (the
+ * checkpoint writer's mr.memcpy(HOST, ...), avro_serialization.cpp:478-523). */
 AXR_API int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t bytes);
 /* Same, enqueued on `stream`; pageable host memory makes it synchronous. */
 AXR_API int axr_memcpy_async(int dst_type, void* dst, int src_type, const void* src,
