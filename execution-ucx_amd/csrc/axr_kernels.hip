@@ -415,6 +415,120 @@ __device__ __forceinline__ void transpose_partial(gcbytes rd, int64_t rd_pitch, 
   __builtin_amdgcn_wave_barrier();
 }
 
+// Rectangular blocks with 16-byte accesses on both global sides.  One side of
+// such a block is a few long rows ("planes"), the other one is contiguous and
+// holds the same elements interleaved (nr planes of nc elements <-> nc groups of
+// nr elements).  Only the LDS side works element by element.
+
+// nr rows of nc elements (row bytes a multiple of 16) -> one contiguous range.
+template <uint32_t E>
+__device__ __forceinline__ void rows_to_interleaved(gcbytes rd, int64_t rd_pitch, gbytes wr,
+                                                    uint32_t nr, uint32_t nc, lbytes lds,
+                                                    uint32_t lane) {
+  typedef typename unit_of<E>::type U;
+  constexpr uint32_t EV = kVecBytes / E;
+  const uint32_t pitch = nc * E + 4u, vpr = nc * E / kVecBytes, nvec = nr * vpr;
+  const uint32_t mv = 0xffffffffu / vpr + 1u, mr = 0xffffffffu / nr + 1u;
+  for (uint32_t v0 = lane; v0 < nvec; v0 += 4 * kWaveLanes) {
+    u32x4 x[4];
+    uint32_t at[4];
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+      const uint32_t v = v0 + k * kWaveLanes < nvec ? v0 + k * kWaveLanes : nvec - 1u;
+      const uint32_t r = small_div(v, vpr, mv);
+      const uint32_t cv = v - r * vpr;
+      at[k] = r * pitch + cv * kVecBytes;
+      x[k] = load16<false>(rd + static_cast<int64_t>(r) * rd_pitch + cv * kVecBytes);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {   // slots past the end repeat the last vector: same bytes
+      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(lds + at[k]);
+      w[0] = x[k].x;
+      w[1] = x[k].y;
+      w[2] = x[k].z;
+      w[3] = x[k].w;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  for (uint32_t j0 = lane; j0 < nvec; j0 += 2 * kWaveLanes) {
+    u32x4 out[2];
+#pragma unroll
+    for (uint32_t k = 0; k < 2; ++k) {
+      const uint32_t j = j0 + k * kWaveLanes < nvec ? j0 + k * kWaveLanes : nvec - 1u;
+      U e[EV];
+#pragma unroll
+      for (uint32_t i = 0; i < EV; ++i) {
+        const uint32_t p = j * EV + i;           // packed element: group b, member a
+        const uint32_t b = small_div(p, nr, mr);
+        const uint32_t a = p - b * nr;
+        e[i] = *reinterpret_cast<const AXR_LDS U*>(lds + a * pitch + b * E);
+      }
+      __builtin_memcpy(&out[k], e, kVecBytes);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < 2; ++k) {
+      const uint32_t j = j0 + k * kWaveLanes;
+      if (j < nvec) store16<false>(wr + static_cast<uint64_t>(j) * kVecBytes, out[k]);
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+// One contiguous range of nr groups of nc elements -> nc rows of nr elements
+// (row bytes a multiple of 16).  In LDS every 128 bytes are followed by a pad
+// dword, which spreads the strided element reads over the banks.
+template <uint32_t E>
+__device__ __forceinline__ void interleaved_to_rows(gcbytes rd, gbytes wr, int64_t wr_pitch,
+                                                    uint32_t nr, uint32_t nc, lbytes lds,
+                                                    uint32_t lane) {
+  typedef typename unit_of<E>::type U;
+  constexpr uint32_t EV = kVecBytes / E;
+  const uint32_t vpr = nr * E / kVecBytes, nvec = nc * vpr;
+  const uint32_t mv = 0xffffffffu / vpr + 1u;
+  for (uint32_t j0 = lane; j0 < nvec; j0 += 4 * kWaveLanes) {
+    u32x4 x[4];
+    uint32_t at[4];
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+      const uint32_t j = j0 + k * kWaveLanes < nvec ? j0 + k * kWaveLanes : nvec - 1u;
+      at[k] = j * kVecBytes + (j >> 3) * 4u;
+      x[k] = load16<false>(rd + static_cast<uint64_t>(j) * kVecBytes);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(lds + at[k]);
+      w[0] = x[k].x;
+      w[1] = x[k].y;
+      w[2] = x[k].z;
+      w[3] = x[k].w;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  for (uint32_t v0 = lane; v0 < nvec; v0 += 2 * kWaveLanes) {
+    u32x4 out[2];
+    uint32_t c[2], cv[2];
+#pragma unroll
+    for (uint32_t k = 0; k < 2; ++k) {
+      const uint32_t v = v0 + k * kWaveLanes < nvec ? v0 + k * kWaveLanes : nvec - 1u;
+      c[k] = small_div(v, vpr, mv);
+      cv[k] = v - c[k] * vpr;
+      U e[EV];
+#pragma unroll
+      for (uint32_t i = 0; i < EV; ++i) {
+        const uint32_t q = ((cv[k] * EV + i) * nc + c[k]) * E;   // byte of element (group r, member c)
+        e[i] = *reinterpret_cast<const AXR_LDS U*>(lds + q + (q >> 7) * 4u);
+      }
+      __builtin_memcpy(&out[k], e, kVecBytes);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < 2; ++k) {
+      if (v0 + k * kWaveLanes < nvec)
+        store16<false>(wr + static_cast<int64_t>(c[k]) * wr_pitch + cv[k] * kVecBytes, out[k]);
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
 // Reads nr rows of nc elements (rows rd_pitch bytes apart) and writes nc rows of
 // nr elements (rows wr_pitch bytes apart).
 __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t rd_pitch, gbytes wr,
@@ -431,6 +545,16 @@ __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t 
       case 8: transpose_full<8>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
       default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
     }
+  } else if ((E == 2 || E == 4) && wr_pitch == static_cast<int64_t>(nr * E) &&
+             ((nc * E) & 15u) == 0) {
+    // the written side is contiguous: a few long rows become interleaved groups
+    if (E == 2) rows_to_interleaved<2>(rd, rd_pitch, wr, nr, nc, lds, lane);
+    else rows_to_interleaved<4>(rd, rd_pitch, wr, nr, nc, lds, lane);
+  } else if ((E == 2 || E == 4) && rd_pitch == static_cast<int64_t>(nc * E) &&
+             ((nr * E) & 15u) == 0) {
+    // the read side is contiguous: interleaved groups become a few long rows
+    if (E == 2) interleaved_to_rows<2>(rd, wr, wr_pitch, nr, nc, lds, lane);
+    else interleaved_to_rows<4>(rd, wr, wr_pitch, nr, nc, lds, lane);
   } else {
     switch (E) {
       case 1: transpose_partial<1>(rd, rd_pitch, wr, wr_pitch, nr, nc, lds, lane); break;

@@ -366,12 +366,21 @@ struct Builder {
       const uint64_t elems = kRectBlockBytes / e;
       if (ea >= t && eb >= t) {
         edge_a = edge_b = static_cast<uint32_t>(t);
-      } else if (ea <= eb) {
-        edge_a = static_cast<uint32_t>(std::min(ea, t));
-        edge_b = static_cast<uint32_t>(std::min<uint64_t>({eb, kRectMaxEdge, elems / edge_a}));
       } else {
-        edge_b = static_cast<uint32_t>(std::min(eb, t));
-        edge_a = static_cast<uint32_t>(std::min<uint64_t>({ea, kRectMaxEdge, elems / edge_b}));
+        // the long edge is a whole number of 16-byte vectors where it can be
+        const uint64_t ev = kVecBytes / e;
+        auto long_edge = [&](uint64_t extent, uint32_t short_edge) {
+          uint64_t edge = std::min<uint64_t>({extent, kRectMaxEdge, elems / short_edge});
+          if (edge >= ev) edge -= edge % ev;
+          return static_cast<uint32_t>(edge);
+        };
+        if (ea <= eb) {
+          edge_a = static_cast<uint32_t>(std::min(ea, t));
+          edge_b = long_edge(eb, edge_a);
+        } else {
+          edge_b = static_cast<uint32_t>(std::min(eb, t));
+          edge_a = long_edge(ea, edge_b);
+        }
       }
       if (static_cast<uint64_t>(edge_a) * edge_b * e < 1024) dim_b = nd;
     }
@@ -415,7 +424,9 @@ struct Builder {
         return fail(AXR_ERR_UNSUPPORTED, "transposed tensor has too many blocks");
       ntile = batches * per_batch;
       // rows of one side plus a dword each, whichever direction needs more
-      const uint32_t lds = edge_a * edge_b * e + 4u * std::max(edge_a, edge_b);
+      // (or one pad dword per 128 bytes, for blocks staged as one contiguous range)
+      const uint32_t block_bytes = edge_a * edge_b * e;
+      const uint32_t lds = block_bytes + std::max(4u * std::max(edge_a, edge_b), block_bytes / 32u + 16u);
       p->cfg.lds_per_wave = std::max<uint32_t>(p->cfg.lds_per_wave, (lds + 15u) & ~15u);
     } else if (run_bytes >= element_mode_limit(run_bytes)) {
       dm.mode = kModeRunTiles;
