@@ -8,6 +8,11 @@
 // tile is at most ROWS x 1 KiB; a wave moves it with ROWS independent 16-byte
 // loads per lane issued back to back, then ROWS 16-byte stores, so each wave
 // keeps ROWS KiB in flight and every access is a fully coalesced 1 KiB row.
+//
+// Strided views with long runs use the same tile copy per run.  Views with
+// short runs (element mode) and transpositions (square or rectangular blocks
+// staged through LDS) live in separate instantiations of the kernel, so that
+// bundles without them run the small streaming kernels.
 #include <hip/hip_runtime.h>
 
 #include "axr_internal.h"
