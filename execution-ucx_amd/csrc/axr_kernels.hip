@@ -420,7 +420,8 @@ __device__ __forceinline__ void transpose_partial(gcbytes rd, int64_t rd_pitch, 
   __builtin_amdgcn_wave_barrier();
 }
 
-// Rectangular blocks with 16-byte accesses on both global sides.  One side of
+// Rectangular blocks of 1-, 2- and 4-byte elements with 16-byte accesses on both
+// global sides.  One side of
 // such a block is a few long rows ("planes"), the other one is contiguous and
 // holds the same elements interleaved (nr planes of nc elements <-> nc groups of
 // nr elements).  Only the LDS side works element by element.
@@ -432,13 +433,14 @@ __device__ __forceinline__ void rows_to_interleaved(gcbytes rd, int64_t rd_pitch
                                                     uint32_t lane) {
   typedef typename unit_of<E>::type U;
   constexpr uint32_t EV = kVecBytes / E;
+  constexpr uint32_t IN = E == 1 ? 2 : 4, OUT = E == 1 ? 1 : 2;   // vectors per lane and round
   const uint32_t pitch = nc * E + 4u, vpr = nc * E / kVecBytes, nvec = nr * vpr;
   const uint32_t mv = 0xffffffffu / vpr + 1u, mr = 0xffffffffu / nr + 1u;
-  for (uint32_t v0 = lane; v0 < nvec; v0 += 4 * kWaveLanes) {
-    u32x4 x[4];
-    uint32_t at[4];
+  for (uint32_t v0 = lane; v0 < nvec; v0 += IN * kWaveLanes) {
+    u32x4 x[IN];
+    uint32_t at[IN];
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {
+    for (uint32_t k = 0; k < IN; ++k) {
       const uint32_t v = v0 + k * kWaveLanes < nvec ? v0 + k * kWaveLanes : nvec - 1u;
       const uint32_t r = small_div(v, vpr, mv);
       const uint32_t cv = v - r * vpr;
@@ -446,7 +448,7 @@ __device__ __forceinline__ void rows_to_interleaved(gcbytes rd, int64_t rd_pitch
       x[k] = load16<false>(rd + static_cast<int64_t>(r) * rd_pitch + cv * kVecBytes);
     }
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {   // slots past the end repeat the last vector: same bytes
+    for (uint32_t k = 0; k < IN; ++k) {   // slots past the end repeat the last vector: same bytes
       AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(lds + at[k]);
       w[0] = x[k].x;
       w[1] = x[k].y;
@@ -455,10 +457,10 @@ __device__ __forceinline__ void rows_to_interleaved(gcbytes rd, int64_t rd_pitch
     }
   }
   __builtin_amdgcn_wave_barrier();
-  for (uint32_t j0 = lane; j0 < nvec; j0 += 2 * kWaveLanes) {
-    u32x4 out[2];
+  for (uint32_t j0 = lane; j0 < nvec; j0 += OUT * kWaveLanes) {
+    u32x4 out[OUT];
 #pragma unroll
-    for (uint32_t k = 0; k < 2; ++k) {
+    for (uint32_t k = 0; k < OUT; ++k) {
       const uint32_t j = j0 + k * kWaveLanes < nvec ? j0 + k * kWaveLanes : nvec - 1u;
       U e[EV];
 #pragma unroll
@@ -471,7 +473,7 @@ __device__ __forceinline__ void rows_to_interleaved(gcbytes rd, int64_t rd_pitch
       __builtin_memcpy(&out[k], e, kVecBytes);
     }
 #pragma unroll
-    for (uint32_t k = 0; k < 2; ++k) {
+    for (uint32_t k = 0; k < OUT; ++k) {
       const uint32_t j = j0 + k * kWaveLanes;
       if (j < nvec) store16<false>(wr + static_cast<uint64_t>(j) * kVecBytes, out[k]);
     }
@@ -488,19 +490,20 @@ __device__ __forceinline__ void interleaved_to_rows(gcbytes rd, gbytes wr, int64
                                                     uint32_t lane) {
   typedef typename unit_of<E>::type U;
   constexpr uint32_t EV = kVecBytes / E;
+  constexpr uint32_t IN = E == 1 ? 2 : 4, OUT = E == 1 ? 1 : 2;   // vectors per lane and round
   const uint32_t vpr = nr * E / kVecBytes, nvec = nc * vpr;
   const uint32_t mv = 0xffffffffu / vpr + 1u;
-  for (uint32_t j0 = lane; j0 < nvec; j0 += 4 * kWaveLanes) {
-    u32x4 x[4];
-    uint32_t at[4];
+  for (uint32_t j0 = lane; j0 < nvec; j0 += IN * kWaveLanes) {
+    u32x4 x[IN];
+    uint32_t at[IN];
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {
+    for (uint32_t k = 0; k < IN; ++k) {
       const uint32_t j = j0 + k * kWaveLanes < nvec ? j0 + k * kWaveLanes : nvec - 1u;
       at[k] = j * kVecBytes + (j >> 3) * 4u;
       x[k] = load16<false>(rd + static_cast<uint64_t>(j) * kVecBytes);
     }
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {
+    for (uint32_t k = 0; k < IN; ++k) {
       AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(lds + at[k]);
       w[0] = x[k].x;
       w[1] = x[k].y;
@@ -509,11 +512,11 @@ __device__ __forceinline__ void interleaved_to_rows(gcbytes rd, gbytes wr, int64
     }
   }
   __builtin_amdgcn_wave_barrier();
-  for (uint32_t v0 = lane; v0 < nvec; v0 += 2 * kWaveLanes) {
-    u32x4 out[2];
-    uint32_t c[2], cv[2];
+  for (uint32_t v0 = lane; v0 < nvec; v0 += OUT * kWaveLanes) {
+    u32x4 out[OUT];
+    uint32_t c[OUT], cv[OUT];
 #pragma unroll
-    for (uint32_t k = 0; k < 2; ++k) {
+    for (uint32_t k = 0; k < OUT; ++k) {
       const uint32_t v = v0 + k * kWaveLanes < nvec ? v0 + k * kWaveLanes : nvec - 1u;
       c[k] = small_div(v, vpr, mv);
       cv[k] = v - c[k] * vpr;
@@ -526,7 +529,7 @@ __device__ __forceinline__ void interleaved_to_rows(gcbytes rd, gbytes wr, int64
       __builtin_memcpy(&out[k], e, kVecBytes);
     }
 #pragma unroll
-    for (uint32_t k = 0; k < 2; ++k) {
+    for (uint32_t k = 0; k < OUT; ++k) {
       if (v0 + k * kWaveLanes < nvec)
         store16<false>(wr + static_cast<int64_t>(c[k]) * wr_pitch + cv[k] * kVecBytes, out[k]);
     }
@@ -550,15 +553,15 @@ __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t 
       case 8: transpose_full<8>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
       default: transpose_full<16>(rd, rd_pitch, wr, wr_pitch, lds, lane, nt_rd, nt_wr); break;
     }
-  } else if ((E == 2 || E == 4) && wr_pitch == static_cast<int64_t>(nr * E) &&
-             ((nc * E) & 15u) == 0) {
+  } else if (E <= 4 && wr_pitch == static_cast<int64_t>(nr * E) && ((nc * E) & 15u) == 0) {
     // the written side is contiguous: a few long rows become interleaved groups
-    if (E == 2) rows_to_interleaved<2>(rd, rd_pitch, wr, nr, nc, lds, lane);
+    if (E == 1) rows_to_interleaved<1>(rd, rd_pitch, wr, nr, nc, lds, lane);
+    else if (E == 2) rows_to_interleaved<2>(rd, rd_pitch, wr, nr, nc, lds, lane);
     else rows_to_interleaved<4>(rd, rd_pitch, wr, nr, nc, lds, lane);
-  } else if ((E == 2 || E == 4) && rd_pitch == static_cast<int64_t>(nc * E) &&
-             ((nr * E) & 15u) == 0) {
+  } else if (E <= 4 && rd_pitch == static_cast<int64_t>(nc * E) && ((nr * E) & 15u) == 0) {
     // the read side is contiguous: interleaved groups become a few long rows
-    if (E == 2) interleaved_to_rows<2>(rd, wr, wr_pitch, nr, nc, lds, lane);
+    if (E == 1) interleaved_to_rows<1>(rd, wr, wr_pitch, nr, nc, lds, lane);
+    else if (E == 2) interleaved_to_rows<2>(rd, wr, wr_pitch, nr, nc, lds, lane);
     else interleaved_to_rows<4>(rd, wr, wr_pitch, nr, nc, lds, lane);
   } else {
     switch (E) {
@@ -572,8 +575,11 @@ __device__ __forceinline__ void transpose_block(uint32_t E, gcbytes rd, int64_t 
 }
 
 // Tile q of a transposed segment: batch index (outer dims), then block (ia, ib).
+// Deliberately not inlined: the block routines get a register allocation of
+// their own (inlined into the kernel's segment walk they spilled and cost the
+// other modes registers too), and forty kernel instantiations share two copies.
 template <bool PACK>
-__device__ __forceinline__ void transpose_tile(uint64_t seg_ptr, dims_table dm, gbytes pay,
+__device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_table dm, gbytes pay,
                                                uint32_t q, lbytes lds, uint32_t lane,
                                                uint32_t nt_bits) {
   const uint32_t E = dm->granule;
