@@ -320,6 +320,79 @@ def host_bundle_c1(h, reps=30):
             "GBps_pcie_inclusive_4P": round(4.0 * nbytes / t / 1e9, 2)}
 
 
+def iov_against_bundle(h, spec, reps=7):
+    """The C2 tensors from sender memory to receiver memory on one device, two ways
+    through the loopback context: the reference's way (one iov entry per tensor on
+    both sides, ucx_connection.cpp:401-426: the transport copies entry by entry)
+    and as a packed bundle (pack, ONE contiguous payload, unpack).  Microseconds
+    per transfer, descriptors prepared beforehand."""
+    from execution_ucx_amd import workloads
+    from execution_ucx_amd.loopback import LoopbackAmContext
+    torch = h.torch
+    arena, _ = workloads.materialize_mixed(spec, "cuda", seed=17)
+    dst = torch.zeros_like(arena)
+    src_iov = [(arena.data_ptr() + s.arena_offset, s.nbytes) for s in spec.segments]
+    dst_iov = [(dst.data_ptr() + s.arena_offset, s.nbytes) for s in spec.segments]
+    client, server = LoopbackAmContext("client"), LoopbackAmContext("server")
+    conn = client.connect(server)
+    t_iov, t_bundle = [], []
+    capi, lib = h.capi, h.lib
+    nseg = len(src_iov)
+    svec, dvec = (capi.Buffer * nseg)(), (capi.Buffer * nseg)()
+    for i in range(nseg):
+        svec[i] = capi.Buffer(src_iov[i][0], src_iov[i][1])
+        dvec[i] = capi.Buffer(dst_iov[i][0], dst_iov[i][1])
+    hdr = C.create_string_buffer(b"iov", 3)
+    d = capi.AmIovec()
+    d.header = capi.Buffer(C.addressof(hdr), 3)
+    d.buffer_vec = C.cast(svec, C.POINTER(capi.Buffer))
+    d.buffer_count = nseg
+    d.buffer_type = capi.MEM_ROCM
+    for _ in range(reps):
+        h.sync()
+        t0 = time.perf_counter()
+        req, m = C.c_uint64(), capi.AmMessage()
+        capi.check(lib.axr_am_send_iov(client._h, conn, C.byref(d), h.stream, C.byref(req)))
+        capi.check(lib.axr_am_recv_header(server._h, C.byref(m)))
+        capi.check(lib.axr_am_recv_buffer_iov(server._h, m.key, capi.MEM_ROCM, dvec, nseg, h.stream))
+        h.sync()
+        t_iov.append(time.perf_counter() - t0)
+        done = C.c_int()
+        capi.check(lib.axr_am_request_test(client._h, req.value, C.byref(done)))
+    ok_iov = all(bool(torch.equal(arena[s.arena_offset:s.arena_offset + s.nbytes],
+                                  dst[s.arena_offset:s.arena_offset + s.nbytes])) for s in spec.segments[::97])
+    dst.zero_()
+    from execution_ucx_amd.dlpack import TensorArray
+    plan = h.pkg.BundlePlan.create(TensorArray(workloads.mixed_views(spec, arena.data_ptr())), align=256)
+    rplan = h.pkg.BundlePlan.from_header(plan.header).bind(
+        TensorArray(workloads.mixed_views(spec, dst.data_ptr())))
+    n = plan.payload_bytes
+    sendbuf = torch.empty(n, dtype=torch.uint8, device="cuda")
+    recvbuf = torch.empty(n, dtype=torch.uint8, device="cuda")
+    for _ in range(reps):
+        h.sync()
+        t0 = time.perf_counter()
+        plan.pack(sendbuf.data_ptr(), n, h.stream)
+        h.sync()                                  # the transport reads a finished buffer
+        req = client.send(conn, plan.header, sendbuf.data_ptr(), n, stream=h.stream)
+        msg = server.recv_header()
+        server.recv_into(msg, recvbuf.data_ptr(), n, stream=h.stream, wait=False)
+        rplan.unpack(recvbuf.data_ptr(), n, h.stream)
+        h.sync()
+        t_bundle.append(time.perf_counter() - t0)
+        client.test(req)
+    ok_bundle = all(bool(torch.equal(arena[s.arena_offset:s.arena_offset + s.nbytes],
+                                     dst[s.arena_offset:s.arena_offset + s.nbytes])) for s in spec.segments[::97])
+    if not (ok_iov and ok_bundle):
+        raise SystemExit("bench.py: loopback transfer differs")
+    client.close()
+    server.close()
+    a, b = sorted(t_iov)[reps // 2] * 1e6, sorted(t_bundle)[reps // 2] * 1e6
+    return {"tensors": len(spec.segments), "payload_bytes_P": plan.data_bytes,
+            "iov_per_tensor_copies_us": round(a, 1), "packed_bundle_us": round(b, 1),
+            "speedup": round(a / b, 1)}
+
+
 def python_boundary(h, spec, reps=5):
     """Planning a 4096-tensor bundle from torch tensors through the Python layer
     (one __dlpack__() call per tensor, descriptors read in C): us per 1k tensors."""
@@ -526,6 +599,7 @@ def main():
         del tr
         torch.cuda.empty_cache()
         extras["c1_host_bundle"] = host_bundle_c1(h)
+        extras["loopback_iov_vs_bundle"] = iov_against_bundle(h, spec)
         extras["python_plan_us_per_1k_tensors"] = python_boundary(h, spec)
         extras["checkpoint_to_host"] = checkpoint_staging(h)
         extras["c5_streamed_8GiB"] = stream_c5(h)
