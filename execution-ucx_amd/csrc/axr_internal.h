@@ -133,10 +133,13 @@ struct Tunables {
   int64_t nontemporal = -1;
   int64_t payload_cache_bytes = 256ll << 20;
   // Strided runs shorter than this use element mode when they are multiples of
-  // 16 bytes, shorter than an eighth of it otherwise (measured crossovers).
+  // 16 bytes; other runs of 16 bytes or more up to five eighths of it (ragged
+  // granules), anything else up to an eighth (measured crossovers).
   int64_t gather_run_bytes = 2048;
   int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
   int64_t transpose = 1;          // move transposed views as square blocks through LDS
+  int64_t ragged_runs = 1;        // short runs of 16+ bytes that are no multiple of 16 move in
+                                  // 16-byte granules (the last one overlapping) instead of narrower ones
 };
 Tunables& tunables();
 

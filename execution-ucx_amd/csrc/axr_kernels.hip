@@ -155,6 +155,8 @@ __device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
 // Moves the ng granules (type T) of one element-mode tile, U per lane at a
 // time: addresses first, then all loads, then all stores, so a lane keeps U
 // accesses in flight instead of a load-wait-store chain per granule.
+// decode(e, &packed) gives granule e's tensor-side offset from tbase and its
+// payload offset from pbase.
 template <bool PACK, typename T, uint32_t U, typename DECODE>
 __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32_t ng,
                                               uint32_t lane, DECODE decode) {
@@ -166,8 +168,9 @@ __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32
     for (uint32_t u = 0; u < U; ++u) {
       const uint32_t e = e0 + u * kWaveLanes;
       const uint32_t ec = e < ng ? e : ng - 1u;   // slots past the end repeat the last granule's load
-      tp[u] = tbase + decode(ec);
-      pp[u] = pbase + static_cast<uint64_t>(ec) * sizeof(T);
+      uint64_t packed;
+      tp[u] = tbase + decode(ec, &packed);
+      pp[u] = pbase + packed;
     }
 #pragma unroll
     for (uint32_t u = 0; u < U; ++u)
@@ -198,12 +201,27 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   constexpr uint32_t kTile = ROWS * kRowBytes < kMinElementTileBytes ? kMinElementTileBytes : ROWS * kRowBytes;
   const uint32_t g = dm->granule;
   const uint32_t gs = static_cast<uint32_t>(__builtin_ctz(g));
-  const uint32_t gpr = static_cast<uint32_t>(run_bytes >> gs);
+  // Ragged runs (16 bytes or longer, not a multiple of 16): a run is ceil(run / 16)
+  // granules of 16 bytes and its last granule covers the run's final 16 bytes,
+  // overlapping the one before it with identical data.  Tiles then count
+  // granules, not packed bytes.
+  const bool ragged = dm->tiles_per_run != 0;
+  const uint32_t run32 = static_cast<uint32_t>(run_bytes);
+  const uint32_t gpr = ragged ? (run32 + 15u) >> 4 : static_cast<uint32_t>(run_bytes >> gs);
   const uint32_t nd = dm->ndim;
-  const uint64_t b0 = static_cast<uint64_t>(q) * kTile;
-  const uint64_t left = dm->nbytes - b0;
-  const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
-  const uint64_t e0 = b0 >> gs;
+  const uint64_t b0 = static_cast<uint64_t>(q) * kTile;   // exact runs: packed byte of the tile
+  uint64_t e0;
+  uint32_t ng;
+  if (ragged) {
+    e0 = static_cast<uint64_t>(q) * (kTile / kVecBytes);
+    const uint64_t left = dm->pstride[0] - e0;            // granules of the whole segment
+    ng = left < kTile / kVecBytes ? static_cast<uint32_t>(left) : kTile / kVecBytes;
+  } else {
+    const uint64_t left = dm->nbytes - b0;
+    const uint32_t n = left < kTile ? static_cast<uint32_t>(left) : kTile;
+    e0 = b0 >> gs;
+    ng = n >> gs;
+  }
   uint32_t run0, w0;
   if ((e0 >> 32) == 0) {
     const uint32_t e32 = static_cast<uint32_t>(e0);
@@ -229,17 +247,24 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
       }
     }
   }
-  const uint32_t ng = n >> gs;
   const uint32_t gpr_magic = 0xffffffffu / gpr + 1u;
   gbytes tbase = as_global(seg_ptr) + base;
-  gbytes pbase = pay + b0;
-  // tensor-side byte offset (relative to the tile's first run) of granule e of the tile
-  auto decode = [&](uint32_t e) -> int64_t {
+  gbytes pbase = ragged ? pay + static_cast<uint64_t>(run0) * run32 : pay + b0;
+  // tensor-side byte offset (relative to the tile's first run) of granule e of the
+  // tile, and its payload offset (relative to pbase)
+  auto decode = [&](uint32_t e, uint64_t* packed) -> int64_t {
     uint32_t w = w0 + e;
     // w < gpr + tile / g: for gpr <= 2^15, w * gpr < 2^32 and the multiply-high quotient is exact
     uint32_t carry = gpr == 1 ? w : (gpr <= 32768u ? __umulhi(w, gpr_magic) : w / gpr);
     w -= carry * gpr;
-    int64_t toff = static_cast<int64_t>(w << gs);
+    uint32_t in_run = w << gs;
+    if (ragged) {
+      in_run = w + 1u == gpr ? run32 - kVecBytes : in_run;
+      *packed = static_cast<uint64_t>(carry) * run32 + in_run;
+    } else {
+      *packed = static_cast<uint64_t>(e) << gs;
+    }
+    int64_t toff = static_cast<int64_t>(in_run);
 #pragma unroll
     for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
       if (static_cast<uint32_t>(d) + nd >= kMaxOuterDims) {

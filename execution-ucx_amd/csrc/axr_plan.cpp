@@ -286,7 +286,10 @@ uint32_t granule_of(uint64_t run_bytes) {
 // bytes per access and lose to the (length-agnostic) run-tile copy much earlier.
 uint64_t element_mode_limit(uint64_t run_bytes) {
   const uint64_t limit = static_cast<uint64_t>(tunables().gather_run_bytes);
-  return granule_of(run_bytes) == 16 ? limit : (limit + 7) / 8;
+  if (granule_of(run_bytes) == 16) return limit;
+  // ragged 16-byte granules: measured ahead of run tiles at 1001-byte runs, behind at 1500
+  if (run_bytes >= kVecBytes && tunables().ragged_runs != 0) return limit * 5 / 8;
+  return (limit + 7) / 8;
 }
 
 struct Builder {
@@ -444,7 +447,18 @@ struct Builder {
       if (runs > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "strided tensor has too many runs");
       dm.granule = granule_of(run_bytes);
       const uint64_t element_tile = std::max<uint32_t>(tile_bytes, kMinElementTileBytes);
-      ntile = (nbytes + element_tile - 1) / element_tile;
+      if (dm.granule != kVecBytes && run_bytes >= kVecBytes && tunables().ragged_runs != 0) {
+        // ragged runs: ceil(run / 16) granules of 16 bytes per run, the last one
+        // covering the run's final 16 bytes; tiles count granules
+        dm.granule = kVecBytes;
+        dm.tiles_per_run = 1;
+        const uint64_t granules = runs * ((run_bytes + kVecBytes - 1) / kVecBytes);
+        dm.pstride[0] = granules;
+        const uint64_t per_tile = element_tile / kVecBytes;
+        ntile = (granules + per_tile - 1) / per_tile;
+      } else {
+        ntile = (nbytes + element_tile - 1) / element_tile;
+      }
     }
     if (p->dims.size() + 1 >= kSegFillOnly)
       return fail(AXR_ERR_UNSUPPORTED, "too many strided tensors in one bundle");

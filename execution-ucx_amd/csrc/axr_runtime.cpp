@@ -320,6 +320,8 @@ static int tune_set_body(const char* key, int64_t value) {
     t.threads = value;
   } else if (k == "xcd_remap") {
     t.xcd_remap = value ? 1 : 0;
+  } else if (k == "ragged_runs") {
+    t.ragged_runs = value ? 1 : 0;
   } else if (k == "transpose") {
     t.transpose = value ? 1 : 0;
   } else {
@@ -344,6 +346,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "threads") *value = t.threads;
   else if (k == "xcd_remap") *value = t.xcd_remap;
   else if (k == "transpose") *value = t.transpose;
+  else if (k == "ragged_runs") *value = t.ragged_runs;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

@@ -330,7 +330,9 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "max_waves", "threads" (workgroup size), "nontemporal" (-1 auto, or bit 0
  * tensor side / bit 1 payload side), "payload_cache_bytes", "gather_run_bytes",
  * "xcd_remap", "transpose" (1: transposed views move as square blocks through
- * LDS; 0: element by element).  Unknown key -> AXR_ERR_INVALID. */
+ * LDS; 0: element by element), "ragged_runs" (1: short strided runs whose
+ * length is no multiple of 16 bytes still move in 16-byte granules).  Unknown
+ * key -> AXR_ERR_INVALID. */
 AXR_API int axr_tune_set(const char* key, int64_t value);
 AXR_API int axr_tune_get(const char* key, int64_t* value);
 

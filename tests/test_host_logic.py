@@ -196,7 +196,7 @@ def seg_of(pkg, view, align=256, **tune):
         return plan.segments(), plan.launch_info()
     finally:
         if tune:
-            pkg.tune(tile_rows=0, gather_run_bytes=2048, transpose=1)
+            pkg.tune(tile_rows=0, gather_run_bytes=2048, transpose=1, ragged_runs=1)
 
 
 def test_compact_tensor_is_one_run(pkg):
@@ -237,26 +237,36 @@ def test_short_runs_use_element_mode(pkg):
     s = segs[0]
     assert (s["mode"], s["run_bytes"], s["granule"]) == (2, 2, 2)
     assert s["shape"] == (30, 20) and s["stride_bytes"] == (2, 60)
-    # 24-byte runs of fp64 -> 8-byte granules; 12-byte elements -> 4-byte granules
+    # 24-byte runs of fp64 -> ragged 16-byte granules (two per run, the second one
+    # overlapping); 12-byte elements are shorter than a vector -> 4-byte granules
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 3], strides=[10, 1], dtype=(2, 64, 1)))
+    assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 24, 16)
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 3], strides=[10, 1], dtype=(2, 64, 1)), ragged_runs=0)
     assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 24, 8)
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 3], strides=[7, 2], dtype=(2, 96, 1)))
     assert (segs[0]["mode"], segs[0]["run_bytes"], segs[0]["granule"]) == (2, 12, 4)
-    # the threshold is a tunable: runs that are multiples of 16 bytes switch at the
-    # tunable itself, others at an eighth of it
+    # the threshold is a tunable
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 304], strides=[1000, 1]), gather_run_bytes=304)
     assert segs[0]["mode"] == 1
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 304], strides=[1000, 1]), gather_run_bytes=305)
     assert segs[0]["mode"] == 2 and segs[0]["granule"] == 16
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2400)
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=480)
     assert segs[0]["mode"] == 1
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2408)
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=488)
+    assert segs[0]["mode"] == 2 and segs[0]["granule"] == 16          # ragged: below 5/8 of it
+    # without ragged granules, runs that are no multiple of 16 switch at an eighth of it
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2400,
+                     ragged_runs=0)
+    assert segs[0]["mode"] == 1
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2408,
+                     ragged_runs=0)
     assert segs[0]["mode"] == 2 and segs[0]["granule"] == 4
-    # defaults: 2 KiB for 16-byte multiples, 256 B otherwise
+    # defaults: 2 KiB
     assert seg_of(pkg, tv(pkg, 0x10000, [5, 2032], strides=[4000, 1]))[0][0]["mode"] == 2
     assert seg_of(pkg, tv(pkg, 0x10000, [5, 2048], strides=[4000, 1]))[0][0]["mode"] == 1
-    assert seg_of(pkg, tv(pkg, 0x10000, [5, 252], strides=[4000, 1]))[0][0]["mode"] == 2
-    assert seg_of(pkg, tv(pkg, 0x10000, [5, 260], strides=[4000, 1]))[0][0]["mode"] == 1
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 1279], strides=[4000, 1]))[0][0]["mode"] == 2
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 1281], strides=[4000, 1]))[0][0]["mode"] == 1
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 260], strides=[4000, 1]), ragged_runs=0)[0][0]["mode"] == 1
 
 
 def test_transposed_views_use_square_blocks(pkg):
