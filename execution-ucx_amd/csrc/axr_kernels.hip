@@ -350,8 +350,11 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
     }
 #pragma unroll
     for (uint32_t k = 0; k < B; ++k) {
-      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(
-          lds + ((kb + k) * RPI + r8) * PITCH + v * kVecBytes);
+      const uint32_t row = (kb + k) * RPI + r8;
+      // byte blocks: the 16-byte chunks of a row are permuted by the row's group of
+      // 16, which spreads the dword column reads below over the banks
+      const uint32_t chunk = E == 1 ? v ^ ((row >> 4) & 7u) : v;
+      AXR_LDS uint32_t* w = reinterpret_cast<AXR_LDS uint32_t*>(lds + row * PITCH + chunk * kVecBytes);
       w[0] = x[k].x;
       w[1] = x[k].y;
       w[2] = x[k].z;
@@ -359,6 +362,47 @@ __device__ __forceinline__ void transpose_full(gcbytes rd, int64_t rd_pitch, gby
     }
   }
   __builtin_amdgcn_wave_barrier();
+  if constexpr (E == 1) {
+    // Bytes: a lane produces four output rows at once.  It reads the dword
+    // (4 columns) of 16 consecutive block rows and transposes each 4 x 4 byte
+    // square in registers (v_perm_b32), a quarter of the LDS reads of a
+    // byte-by-byte gather.  256 units of (4 output rows) x (one 16-byte vector).
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+      const uint32_t cg = (lane >> 3) + 8u * k;   // output rows 4 cg .. 4 cg + 3
+      const AXR_LDS uint8_t* col = lds + (((cg >> 2) ^ v) * kVecBytes) + (cg & 3u) * 4u;
+      u32x4 out[4];
+#pragma unroll
+      for (uint32_t m = 0; m < 4; ++m) {
+        uint32_t d[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+          d[j] = *reinterpret_cast<const AXR_LDS uint32_t*>(col + (v * 16u + m * 4u + j) * PITCH);
+        // perm(hi, lo, sel): selector values 0-3 take bytes of lo, 4-7 bytes of hi
+        const uint32_t ab_lo = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u);
+        const uint32_t ab_hi = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+        const uint32_t cd_lo = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+        const uint32_t cd_hi = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+        out[0][m] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);
+        out[1][m] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);
+        out[2][m] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);
+        out[3][m] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
+      }
+      if (nt_wr) {
+        asm volatile("");
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i)
+          store16<true>(wr + static_cast<int64_t>(4u * cg + i) * wr_pitch + v * kVecBytes, out[i]);
+        asm volatile("");
+      } else {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i)
+          store16<false>(wr + static_cast<int64_t>(4u * cg + i) * wr_pitch + v * kVecBytes, out[i]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    return;
+  }
 #pragma unroll
   for (uint32_t kb = 0; kb < NK; kb += B) {
     u32x4 out[B];
