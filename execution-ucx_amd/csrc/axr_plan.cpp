@@ -977,6 +977,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_from_header: out of host memory");
   p->align = align;
   p->tensors.resize(n);
+  p->dims64.reserve((length - kFixedHeader - static_cast<size_t>(n) * kTensorHeader) / 8);   // all shapes
   size_t at = kFixedHeader;
   for (uint32_t i = 0; i < n; ++i) {
     if (length - at < kTensorHeader) {
@@ -1037,34 +1038,27 @@ static int plan_bind_body(axr_plan_t* plan, const axr_tensor_t* tensors, size_t 
   if (n != plan->tensors.size())
     return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor count differs from the plan");
   if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_bind: null tensor array");
-  // validate everything before touching the plan
-  for (size_t i = 0; i < n; ++i) {
-    const TensorRec& t = plan->tensors[i];
-    const axr_tensor_t& in = tensors[i];
-    uint64_t nb = 0;
-    int rc = nbytes_rule(in.ndim, in.shape, in.dtype_bits, &nb);
-    if (rc) return rc;
-    if (nb != t.nbytes || (nb != 0 && (in.dtype_bits + 7) / 8 != (t.bits + 7) / 8))
-      return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor " + std::to_string(i) +
-                                        " does not match the plan's size or element width");
-    if (nb != 0 && !in.data) return fail(AXR_ERR_INVALID, "axr_plan_bind: null tensor data");
-  }
-  quiesce(plan);
-  invalidate_tables(plan);
+  // Everything is validated and staged in temporaries first: a failure leaves the
+  // plan as it was.
   std::vector<int64_t> dims64;
   std::vector<TensorRec> recs(n);
   {
     axr_plan tmp;   // reuse store_tensor's bookkeeping
+    tmp.dims64.reserve(plan->dims64.size() * 2);
     for (size_t i = 0; i < n; ++i) {
-      int rc = store_tensor(&tmp, tensors[i], &recs[i]);
+      const TensorRec& t = plan->tensors[i];
+      int rc = store_tensor(&tmp, tensors[i], &recs[i]);   // size rule, null checks
       if (rc) return rc;
+      if (recs[i].nbytes != t.nbytes ||
+          (t.nbytes != 0 && (recs[i].bits + 7) / 8 != (t.bits + 7) / 8))
+        return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor " + std::to_string(i) +
+                                          " does not match the plan's size or element width");
+      recs[i].offset = t.offset;
     }
     dims64.swap(tmp.dims64);
   }
-  for (size_t i = 0; i < n; ++i) {
-    recs[i].offset = plan->tensors[i].offset;
-    recs[i].nbytes = plan->tensors[i].nbytes;
-  }
+  quiesce(plan);
+  invalidate_tables(plan);
   // The header keeps describing what was sent; the bound records describe memory.
   plan->tensors.swap(recs);
   plan->dims64.swap(dims64);
