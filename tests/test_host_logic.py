@@ -468,3 +468,23 @@ def test_native_extraction_matches_the_python_path(pkg):
     assert mixed.count == 2
     with pytest.raises(TypeError):
         dlpack.TensorArray.from_objects([object()])
+
+
+# ------------------------------------------------------------------ bench.py contract (no GPU needed)
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=120)
+    assert out.returncode != 0
+    assert "one GPU" in (out.stderr + out.stdout)
+
+
+def test_product_never_imports_the_oracle():
+    """The oracle is test infrastructure: nothing under the package may import it."""
+    pkg_dir = os.path.join(ROOT, "execution-ucx_amd")
+    for name in os.listdir(pkg_dir):
+        if name.endswith(".py"):
+            text = open(os.path.join(pkg_dir, name)).read()
+            assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), name
