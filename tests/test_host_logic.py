@@ -488,3 +488,32 @@ def test_product_never_imports_the_oracle():
         if name.endswith(".py"):
             text = open(os.path.join(pkg_dir, name)).read()
             assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), name
+
+
+# ------------------------------------------------------------------ edge cases of the planner
+
+def test_empty_and_extreme_bundles(pkg, orc):
+    # no tensors at all: an empty payload and a header that round-trips
+    plan = pkg.BundlePlan.create([], align=256)
+    assert plan.payload_bytes == 0 and plan.num_tensors == 0
+    back = pkg.BundlePlan.from_header(plan.header)
+    assert back.num_tensors == 0 and back.payload_bytes == 0
+    assert orc.decode_header(plan.header) == (256, 0, [])
+    # only empty and 0-d tensors: offsets exist, no bytes, no segments
+    views = [tv(pkg, 0, [0]), tv(pkg, 0, []), tv(pkg, 0, [4, 0, 3])]
+    plan = pkg.BundlePlan.create(views, align=64)
+    assert plan.payload_bytes == 0 and plan.segments() == []
+    assert plan.launch_info()["tiles"] == 0
+    # 64 dimensions (the most a tensor may have); 65 are refused
+    shape = [1] * 62 + [3, 5]
+    plan = pkg.BundlePlan.create([tv(pkg, 0x1000, shape)], align=1)
+    assert plan.payload_bytes == 15 and plan.segments()[0]["mode"] == 0
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.create([tv(pkg, 0x1000, [1] * 65)], align=1)
+    # element counts that overflow 64 bits are refused, unless an extent is zero
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.create([tv(pkg, 0x1000, [2 ** 40, 2 ** 40])], align=1)
+    assert pkg.BundlePlan.create([tv(pkg, 0, [2 ** 40, 2 ** 40, 0])], align=1).payload_bytes == 0
+    # a null data pointer is only acceptable for an empty tensor
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.create([tv(pkg, 0, [8])], align=1)
