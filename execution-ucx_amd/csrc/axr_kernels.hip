@@ -802,7 +802,7 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
 }
 
 __global__ __launch_bounds__(256) void fill_kernel(uint8_t* dst, uint8_t value, size_t bytes) {
-  // 16-byte stores on the aligned body, bytes at both ends.
+  // 16-byte streaming stores on the aligned body, bytes at both ends.
   const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
   const size_t head = (16u - (reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
@@ -812,37 +812,101 @@ __global__ __launch_bounds__(256) void fill_kernel(uint8_t* dst, uint8_t value, 
   const uint32_t w = value * 0x01010101u;
   const u32x4 v = {w, w, w, w};
   u32x4* d = reinterpret_cast<u32x4*>(dst + h);
-  for (size_t i = tid; i < body; i += nthreads) d[i] = v;
+  for (size_t i = tid; i < body; i += nthreads) __builtin_nontemporal_store(v, d + i);
   const size_t done = h + (body << 4);
   for (size_t i = done + tid; i < bytes; i += nthreads) dst[i] = value;
 }
 
+// The reference's device-side test step (x /= 2 per element), four floats per
+// access where the array allows it.
 __global__ __launch_bounds__(256) void divide_by_two_kernel(float* data, size_t count) {
-  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < count) data[i] /= 2.0f;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const size_t head_all = ((16u - (reinterpret_cast<uintptr_t>(data) & 15u)) & 15u) / sizeof(float);
+  const size_t head = head_all < count ? head_all : count;
+  for (size_t i = tid; i < head; i += nthreads) data[i] /= 2.0f;
+  const size_t body = (count - head) / 4;
+  f32x4* d = reinterpret_cast<f32x4*>(data + head);
+  for (size_t i = tid; i < body; i += nthreads) {
+    f32x4 x = d[i];
+    x.x /= 2.0f;
+    x.y /= 2.0f;
+    x.z /= 2.0f;
+    x.w /= 2.0f;
+    d[i] = x;
+  }
+  for (size_t i = head + body * 4 + tid; i < count; i += nthreads) data[i] /= 2.0f;
 }
 
+// One atomic per workgroup instead of one per thread, spread over kSumSlots
+// counters that the host adds up: atomics on one address are served one after
+// the other (about 12 ns each on MI355X), which dominated these kernels whenever
+// every thread had something to add.
+constexpr uint32_t kSumSlots = 64;
+__device__ __forceinline__ void block_atomic_add(unsigned long long* slots, unsigned long long local) {
+  __shared__ unsigned long long partial[4];   // launched with 256 threads
+#pragma unroll
+  for (int step = 32; step >= 1; step >>= 1) local += __shfl_xor(local, step, 64);
+  if ((threadIdx.x & (kWaveLanes - 1)) == 0) partial[threadIdx.x >> 6] = local;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned long long total = partial[0] + partial[1] + partial[2] + partial[3];
+    if (total) atomicAdd(slots + blockIdx.x % kSumSlots, total);
+  }
+}
+
+// Number of bytes that differ, 16 bytes per access (no alignment needed).
 __global__ __launch_bounds__(256) void compare_kernel(const uint8_t* a, const uint8_t* b,
                                                       size_t bytes,
                                                       unsigned long long* mismatches) {
   const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const size_t nvec = bytes >> 4;
   unsigned long long local = 0;
-  for (size_t i = tid; i < bytes; i += nthreads) local += (a[i] != b[i]) ? 1u : 0u;
-  if (local) atomicAdd(mismatches, local);
+  for (size_t i = tid; i < nvec; i += nthreads) {
+    const u32x4 x = *reinterpret_cast<const u32x4_loose*>(a + (i << 4));
+    const u32x4 y = *reinterpret_cast<const u32x4_loose*>(b + (i << 4));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t d = x[k] ^ y[k];
+      // bit 7 of every byte that is not zero
+      const uint32_t nz = (((d & 0x7f7f7f7fu) + 0x7f7f7f7fu) | d) & 0x80808080u;
+      local += __builtin_popcount(nz);
+    }
+  }
+  for (size_t i = (nvec << 4) + tid; i < bytes; i += nthreads) local += (a[i] != b[i]) ? 1u : 0u;
+  block_atomic_add(mismatches, local);
 }
 
+// sum of byte[i] * (1 + (start + i) mod 65521): the modulus is taken once per
+// 16 bytes and stepped from there.
 __global__ __launch_bounds__(256) void checksum_kernel(const uint8_t* data, size_t bytes,
                                                        uint64_t start,
                                                        unsigned long long* sum) {
   const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const size_t nvec = bytes >> 4;
   unsigned long long local = 0;
-  for (size_t i = tid; i < bytes; i += nthreads) {
+  for (size_t i = tid; i < nvec; i += nthreads) {
+    const u32x4 x = *reinterpret_cast<const u32x4_loose*>(data + (i << 4));
+    uint32_t m = static_cast<uint32_t>((start + (i << 4)) % 65521u);
+    uint32_t part = 0;   // 16 * 255 * 65521 fits 32 bits
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        part += ((x[k] >> (8 * j)) & 0xffu) * (m + 1u);
+        m = m + 1u == 65521u ? 0u : m + 1u;
+      }
+    }
+    local += part;
+  }
+  for (size_t i = (nvec << 4) + tid; i < bytes; i += nthreads) {
     const uint64_t wgt = 1u + ((start + i) % 65521u);
     local += static_cast<unsigned long long>(data[i]) * wgt;
   }
-  atomicAdd(sum, local);
+  block_atomic_add(sum, local);
 }
 
 __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__ dst,
@@ -919,7 +983,7 @@ int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& 
 
 int launch_fill(void* dst, int value, size_t bytes, void* stream) {
   if (bytes == 0) return AXR_OK;
-  hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(bytes / 16 + 1, 4096)), dim3(256), 0,
+  hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(bytes / 16 + 1, 1u << 16)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<uint8_t*>(dst),
                      static_cast<uint8_t>(value), bytes);
   return check_hip(hipGetLastError(), "fill kernel launch");
@@ -929,14 +993,38 @@ int launch_fill(void* dst, int value, size_t bytes, void* stream) {
 
 using namespace axr;
 
+namespace {
+// Runs `launch(slots)` with kSumSlots zeroed device counters and returns their sum.
+template <typename Launch>
+int sum_over_slots(Launch&& launch, const char* what, uint64_t* total) {
+  unsigned long long* dev = nullptr;
+  const size_t bytes = kSumSlots * sizeof(*dev);
+  int rc = check_hip(hipMalloc(reinterpret_cast<void**>(&dev), bytes), "hipMalloc");
+  if (rc) return rc;
+  rc = check_hip(hipMemset(dev, 0, bytes), "hipMemset");
+  if (!rc) {
+    launch(dev);
+    rc = check_hip(hipGetLastError(), what);
+  }
+  unsigned long long host[kSumSlots] = {};
+  if (!rc) rc = check_hip(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost), "hipMemcpy");
+  (void)hipFree(dev);
+  if (!rc) {
+    uint64_t sum = 0;
+    for (unsigned long long v : host) sum += v;
+    *total = sum;
+  }
+  return rc;
+}
+
+}  // namespace
+
 extern "C" {
 
 static int divide_by_two_body(float* data, size_t count, void* stream) {
   if (count == 0) return AXR_OK;
   if (!data) return fail(AXR_ERR_INVALID, "axr_divide_by_two: null data");
-  const size_t blocks = (count + 255) / 256;
-  if (blocks > 0x7fffffffu) return fail(AXR_ERR_INVALID, "axr_divide_by_two: count too large");
-  hipLaunchKernelGGL(divide_by_two_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+  hipLaunchKernelGGL(divide_by_two_kernel, dim3(blocks_for(count / 4 + 1, 1u << 18)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), data, count);
   return check_hip(hipGetLastError(), "divide_by_two launch");
 }
@@ -949,20 +1037,13 @@ static int compare_body(const void* a, const void* b, size_t bytes, uint64_t* mi
   *mismatches = 0;
   if (bytes == 0) return AXR_OK;
   if (!a || !b) return fail(AXR_ERR_INVALID, "axr_compare: null range");
-  unsigned long long* dev = nullptr;
-  int rc = check_hip(hipMalloc(reinterpret_cast<void**>(&dev), sizeof(*dev)), "hipMalloc");
-  if (rc) return rc;
-  rc = check_hip(hipMemset(dev, 0, sizeof(*dev)), "hipMemset");
-  if (!rc) {
-    hipLaunchKernelGGL(compare_kernel, dim3(blocks_for(bytes, 8192)), dim3(256), 0, nullptr,
-                       static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), bytes, dev);
-    rc = check_hip(hipGetLastError(), "compare launch");
-  }
-  unsigned long long host = 0;
-  if (!rc) rc = check_hip(hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost), "hipMemcpy");
-  (void)hipFree(dev);
-  if (!rc) *mismatches = host;
-  return rc;
+  return sum_over_slots(
+      [&](unsigned long long* slots) {
+        hipLaunchKernelGGL(compare_kernel, dim3(blocks_for(bytes / 16 + 1, 1u << 16)), dim3(256), 0,
+                           nullptr, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
+                           bytes, slots);
+      },
+      "compare launch", mismatches);
 }
 int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mismatches) {
   return guarded([&] { return compare_body(a, b, bytes, mismatches); });
@@ -973,20 +1054,12 @@ static int checksum_body(const void* data, size_t bytes, uint64_t start, uint64_
   *sum = 0;
   if (bytes == 0) return AXR_OK;
   if (!data) return fail(AXR_ERR_INVALID, "axr_checksum: null range");
-  unsigned long long* dev = nullptr;
-  int rc = check_hip(hipMalloc(reinterpret_cast<void**>(&dev), sizeof(*dev)), "hipMalloc");
-  if (rc) return rc;
-  rc = check_hip(hipMemset(dev, 0, sizeof(*dev)), "hipMemset");
-  if (!rc) {
-    hipLaunchKernelGGL(checksum_kernel, dim3(blocks_for(bytes, 8192)), dim3(256), 0, nullptr,
-                       static_cast<const uint8_t*>(data), bytes, start, dev);
-    rc = check_hip(hipGetLastError(), "checksum launch");
-  }
-  unsigned long long host = 0;
-  if (!rc) rc = check_hip(hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost), "hipMemcpy");
-  (void)hipFree(dev);
-  if (!rc) *sum = host;
-  return rc;
+  return sum_over_slots(
+      [&](unsigned long long* slots) {
+        hipLaunchKernelGGL(checksum_kernel, dim3(blocks_for(bytes / 16 + 1, 1u << 16)), dim3(256), 0,
+                           nullptr, static_cast<const uint8_t*>(data), bytes, start, slots);
+      },
+      "checksum launch", sum);
 }
 int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum) {
   return guarded([&] { return checksum_body(data, bytes, start, sum); });
@@ -999,7 +1072,7 @@ static int copy_reference_body(void* dst, const void* src, size_t bytes, void* s
     return fail(AXR_ERR_INVALID, "axr_copy_reference: pointers and size must be multiples of 16");
   }
   const size_t nvec = bytes / 16;
-  hipLaunchKernelGGL(copy_reference_kernel, dim3(blocks_for(nvec, 256 * 32)), dim3(256), 0,
+  hipLaunchKernelGGL(copy_reference_kernel, dim3(blocks_for(nvec, 1u << 20)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<u32x4*>(dst),
                      static_cast<const u32x4*>(src), nvec);
   return check_hip(hipGetLastError(), "copy_reference launch");
