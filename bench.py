@@ -395,7 +395,7 @@ def iov_against_bundle(h, spec, reps=7):
 
 def python_boundary(h, spec, reps=5):
     """Planning a 4096-tensor bundle from torch tensors through the Python layer
-    (one __dlpack__() call per tensor, descriptors read in C): us per 1k tensors."""
+    (one DLPack export per tensor from C, descriptors read in C): us per 1k tensors."""
     from execution_ucx_amd import workloads
     arena, tensors = workloads.materialize_mixed(spec, "cuda", seed=5)
     times = []

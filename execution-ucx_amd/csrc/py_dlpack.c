@@ -5,13 +5,23 @@
  * else.  The result is a ready array of axr_tensor_t (layout-identical to
  * DLTensor) for axr_plan_create / axr_plan_bind.
  *
- * describe(sequence) -> (descs: bytearray, dims: bytearray, owners: list)
+ * describe(sequence[, fast_type, fast_export, device_id])
+ *     -> (descs: bytearray, dims: bytearray, owners: list)
  *   descs   n * sizeof(axr_tensor_t); shape/strides point into `dims`
  *   dims    the copied shapes and strides (int64)
  *   owners  the capsules; they stay unconsumed, so dropping them runs the
  *           producers' deleters
  * Every element must provide `__dlpack__()` or be a capsule named "dltensor"
- * or "dltensor_versioned".
+ * or "dltensor_versioned"; describe() returns None when it meets anything else.
+ *
+ * Objects whose type is exactly `fast_type` are exported with
+ * `fast_export(obj)` instead, when `obj.requires_grad` and `obj.is_conj()` are
+ * both False and the exported tensor is in host memory or on GPU `device_id`.
+ * The caller passes torch.Tensor and torch.utils.dlpack.to_dlpack here: the
+ * C exporter that Tensor.__dlpack__ ends in, minus a dozen Python-level checks
+ * per tensor (about 0.15 us instead of 1.7 us).  Whatever fails one of the
+ * conditions, or makes `fast_export` raise, goes through `__dlpack__()` and
+ * gets that method's verdict.
  */
 #define PY_SSIZE_T_CLEAN
 #include <Python.h>
@@ -37,8 +47,59 @@ static const axr_tensor_t* tensor_of_capsule(PyObject* capsule) {
   return NULL;
 }
 
-static PyObject* describe(PyObject* self, PyObject* arg) {
+static PyObject* str_requires_grad;
+static PyObject* str_is_conj;
+static PyObject* str_dlpack;
+
+/* 1 when `obj` carries nothing that Tensor.__dlpack__ refuses to export. */
+static int plain_tensor(PyObject* obj) {
+  PyObject* grad = PyObject_GetAttr(obj, str_requires_grad);
+  if (!grad) {
+    PyErr_Clear();
+    return 0;
+  }
+  const int no_grad = grad == Py_False;
+  Py_DECREF(grad);
+  if (!no_grad) return 0;
+  PyObject* conj = PyObject_CallMethodNoArgs(obj, str_is_conj);
+  if (!conj) {
+    PyErr_Clear();
+    return 0;
+  }
+  const int no_conj = conj == Py_False;
+  Py_DECREF(conj);
+  return no_conj;
+}
+
+/* The capsule of `obj` through the fast exporter, or NULL (no error set) when
+ * the object has to take the `__dlpack__()` route. */
+static PyObject* export_fast(PyObject* obj, PyObject* fast_export, long device_id) {
+  if (!plain_tensor(obj)) return NULL;
+  PyObject* capsule = PyObject_CallOneArg(fast_export, obj);
+  if (!capsule) {
+    PyErr_Clear();
+    return NULL;
+  }
+  const axr_tensor_t* t = PyCapsule_IsValid(capsule, "dltensor")
+                              ? (const axr_tensor_t*)PyCapsule_GetPointer(capsule, "dltensor")
+                              : NULL;
+  /* DLDeviceType: 2 kDLCUDA, 10 kDLROCM -- memory of one particular GPU */
+  const int on_gpu = t && (t->device_type == 10 || t->device_type == 2);
+  if (!t || (on_gpu && t->device_id != device_id)) {
+    Py_DECREF(capsule);   /* unconsumed: its destructor runs the producer's deleter */
+    return NULL;
+  }
+  return capsule;
+}
+
+static PyObject* describe(PyObject* self, PyObject* args) {
   (void)self;
+  PyObject* arg = NULL;
+  PyObject* fast_type = Py_None;
+  PyObject* fast_export = Py_None;
+  long device_id = -1;
+  if (!PyArg_ParseTuple(args, "O|OOl", &arg, &fast_type, &fast_export, &device_id)) return NULL;
+  if (fast_type == Py_None || fast_export == Py_None) fast_type = NULL;
   PyObject* seq = PySequence_Fast(arg, "describe() needs a sequence of DLPack producers");
   if (!seq) return NULL;
   const Py_ssize_t n = PySequence_Fast_GET_SIZE(seq);
@@ -56,7 +117,21 @@ static PyObject* describe(PyObject* self, PyObject* arg) {
       capsule = obj;
       Py_INCREF(capsule);
     } else {
-      capsule = PyObject_CallMethod(obj, "__dlpack__", NULL);
+      capsule = fast_type && (PyObject*)Py_TYPE(obj) == fast_type
+                    ? export_fast(obj, fast_export, device_id)
+                    : NULL;
+      if (!capsule) {
+        PyObject* method = PyObject_GetAttr(obj, str_dlpack);
+        if (!method) {   /* not a DLPack producer: the caller's business */
+          if (!PyErr_ExceptionMatches(PyExc_AttributeError)) goto done;
+          PyErr_Clear();
+          result = Py_None;
+          Py_INCREF(result);
+          goto done;
+        }
+        capsule = PyObject_CallNoArgs(method);
+        Py_DECREF(method);
+      }
       if (!capsule) goto done;
     }
     PyList_SET_ITEM(owners, i, capsule);   /* steals */
@@ -108,8 +183,9 @@ done:
 }
 
 static PyMethodDef methods[] = {
-    {"describe", describe, METH_O,
-     "describe(sequence) -> (descs bytearray, dims bytearray, owners list)"},
+    {"describe", describe, METH_VARARGS,
+     "describe(sequence[, fast_type, fast_export, device_id]) -> "
+     "(descs bytearray, dims bytearray, owners list)"},
     {NULL, NULL, 0, NULL}};
 
 static struct PyModuleDef module = {PyModuleDef_HEAD_INIT, "_axr_dlpack",
@@ -117,6 +193,10 @@ static struct PyModuleDef module = {PyModuleDef_HEAD_INIT, "_axr_dlpack",
                                     NULL, NULL, NULL, NULL};
 
 PyMODINIT_FUNC PyInit__axr_dlpack(void) {
+  str_requires_grad = PyUnicode_InternFromString("requires_grad");
+  str_is_conj = PyUnicode_InternFromString("is_conj");
+  str_dlpack = PyUnicode_InternFromString("__dlpack__");
+  if (!str_requires_grad || !str_is_conj || !str_dlpack) return NULL;
   PyObject* m = PyModule_Create(&module);
   if (m) PyModule_AddIntConstant(m, "TENSOR_BYTES", (long)sizeof(axr_tensor_t));
   return m;

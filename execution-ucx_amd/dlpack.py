@@ -186,10 +186,10 @@ class TensorArray:
     def from_objects(cls, objs: Sequence[Any]) -> "TensorArray":
         """Descriptors of DLPack producers (or ``TensorView``s)."""
         native = _native()
-        if native is None or any(isinstance(o, TensorView) or not (
-                hasattr(o, "__dlpack__") or type(o).__name__ == "PyCapsule") for o in objs):
+        described = native.describe(objs, *_torch_exporter()) if native is not None else None
+        if described is None:   # no helper, or something that is not a DLPack producer
             return cls(extract_many(objs))
-        descs, dims, owners = native.describe(objs)
+        descs, dims, owners = described
         self = cls.__new__(cls)
         n = len(owners)
         self.count = n
@@ -208,6 +208,29 @@ class TensorArray:
     @views.setter
     def views(self, value):
         self._views = value
+
+
+def _torch_exporter() -> tuple:
+    """``(torch.Tensor, to_dlpack, device)`` for the C helper, or ``()``.
+
+    ``Tensor.__dlpack__()`` is a page of Python around ``to_dlpack``: it refuses
+    tensors that require gradients or carry the conjugate bit, refuses GPU
+    tensors of another device than the current one, and makes the default stream
+    wait for torch's current stream when the two differ.  The helper repeats the
+    first three checks in C; the fourth does nothing while torch runs on its
+    default stream, which is checked here once per bundle.  Anywhere else every
+    tensor goes through ``__dlpack__()``.
+    """
+    import sys
+    torch = sys.modules.get("torch")
+    if torch is None:
+        return ()
+    device = -1   # no GPU context: only host tensors can exist
+    if torch.cuda.is_initialized():
+        if torch.cuda.current_stream() != torch.cuda.default_stream():
+            return ()
+        device = torch.cuda.current_device()
+    return (torch.Tensor, torch.utils.dlpack.to_dlpack, device)
 
 
 _NATIVE: Any = False

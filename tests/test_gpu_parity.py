@@ -703,6 +703,33 @@ def test_dlpack_rocm_capsules_and_zero_copy_receive(pkg, gpu):
     assert [o.data_ptr() - base for o in outs] == packed.plan.layout()[0]   # views, not copies
 
 
+def test_torch_device_tensors_through_the_short_export_route(pkg, orc, gpu):
+    """GPU tensors are exported from C with to_dlpack while torch runs on its default
+    stream, and through Tensor.__dlpack__ (which orders the streams) on any other;
+    both routes describe the same memory and pack the oracle's bytes."""
+    import torch
+    from execution_ucx_amd import dlpack
+    rng = np.random.default_rng(33)
+    tensors = [rand_bytes_tensor(rng, n, gpu) for n in (4096, 10, 70002, 0, 512)]
+    tensors[2] = tensors[2][2:70002].view(torch.int16).reshape(100, 350)[:, 3:77]
+    fast = dlpack._torch_exporter()
+    assert fast and fast[2] == torch.cuda.current_device()
+    short = dlpack.TensorArray.from_objects(tensors).views
+    plain = dlpack.extract_many(tensors)
+    assert [(x.data, x.device_type, x.shape, x.strides, x.dtype) for x in short] == \
+        [(x.data, x.device_type, x.shape, x.strides, x.dtype) for x in plain]
+    want = orc.pack([tbytes(t) for t in tensors], 64)
+    got, plan, _ = run_pack(pkg, tensors, 64, gpu)
+    assert np.array_equal(got, want)
+    plan.close()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        assert dlpack._torch_exporter() == ()
+        got, plan, _ = run_pack(pkg, tensors, 64, gpu)       # packs on `side`
+    assert np.array_equal(got, want)
+    plan.close()
+
+
 def test_bundle_to_host_for_checkpointing(pkg, orc, gpu):
     """A packed device bundle staged to host byte arrays, one per tensor (what the
     reference's checkpoint writer builds with one memcpy per buffer,

@@ -470,6 +470,47 @@ def test_native_extraction_matches_the_python_path(pkg):
         dlpack.TensorArray.from_objects([object()])
 
 
+def test_torch_tensors_skip_the_python_wrapper_but_keep_its_refusals(pkg):
+    """Plain torch.Tensor objects are exported with torch.utils.dlpack.to_dlpack from
+    C; what Tensor.__dlpack__ refuses is still refused with its own error, subclasses
+    keep going through __dlpack__, and both routes describe the same memory."""
+    import torch
+    from execution_ucx_amd import dlpack
+    native = dlpack._native()
+    assert native is not None
+    fast = dlpack._torch_exporter()
+    assert fast[0] is torch.Tensor and fast[2] == -1      # no GPU context in this process
+
+    tensors = [torch.arange(60, dtype=torch.float32).reshape(3, 4, 5)[:, 1:3],
+               torch.zeros(0, 7, dtype=torch.int8), torch.tensor(2.5, dtype=torch.float64),
+               torch.arange(8, dtype=torch.int16).view(torch.bfloat16)]
+    calls = []
+    counting = (fast[0], lambda t: (calls.append(1), fast[1](t))[1], fast[2])
+    a = native.describe(tensors, *counting)
+    b = native.describe(tensors)
+    assert len(calls) == len(tensors)
+    assert bytes(a[0])[:8] == bytes(b[0])[:8] and bytes(a[1]) == bytes(b[1])
+    va = dlpack.TensorArray.from_objects(tensors).views
+    vb = dlpack.extract_many(tensors)
+    assert [(x.data, x.shape, x.strides or None, x.dtype) for x in va] == \
+        [(x.data, x.shape, x.strides or None, x.dtype) for x in vb]   # 0-d: () or None
+
+    class Wrapped(torch.Tensor):
+        pass
+    calls.clear()
+    native.describe([tensors[0].as_subclass(Wrapped)], *counting)
+    assert calls == []                                    # a subclass may override __dlpack__
+
+    for bad, text in ((torch.zeros(3, requires_grad=True), "gradient"),
+                      (torch.zeros(3, dtype=torch.complex64).conj(), "conjugate"),
+                      (torch.zeros(3, 3).to_sparse(), "layout")):
+        with pytest.raises(BufferError, match=text):
+            dlpack.TensorArray.from_objects([tensors[0], bad])
+    # a GPU tensor of another device than the one passed goes to __dlpack__ as well:
+    # with device -1 every GPU tensor does, so a process without a context never
+    # hands out GPU memory through the short route (checked on the capsule in C)
+
+
 # ------------------------------------------------------------------ bench.py contract (no GPU needed)
 
 def test_bench_refuses_more_than_one_gpu():
