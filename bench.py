@@ -112,6 +112,41 @@ def run_sets(h: Harness, sets, steps, warmup):
     return ms
 
 
+def run_sets_two_streams(h: Harness, sets, steps, warmup):
+    """The same steps with the bundles alternating between two streams, so that one
+    bundle's pack overlaps another's unpack (a sender with several bundles in flight).
+    Host clock around a synchronisation of both streams; returns milliseconds."""
+    lib, check = h.lib, h.capi.check
+    second = C.c_void_p()
+    check(lib.axr_stream_create(C.byref(second)))
+    streams = (h.stream, second.value)
+    n = len(sets)
+    calls = [(s.pp, s.up, s.ptr, s.nbytes) for s in sets]
+
+    def step(i):
+        pp, up, ptr, nb = calls[i % n]
+        stream = streams[i % 2]
+        rc = lib.axr_pack(pp, ptr, nb, stream)
+        rc |= lib.axr_unpack(up, ptr, nb, stream)
+        if rc:
+            check(rc)
+
+    def drain():
+        for stream in streams:
+            check(lib.axr_stream_synchronize(stream))
+
+    for i in range(warmup):
+        step(i)
+    drain()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    drain()
+    ms = (time.perf_counter() - t0) * 1e3
+    check(lib.axr_stream_destroy(second))
+    return ms
+
+
 def make_c2_sets(h, count, seed=0):
     from execution_ucx_amd import workloads
     spec = workloads.mixed_bundle(seed=seed)
@@ -570,6 +605,9 @@ def main():
         # cache-resident rate of the same bundle
         ms1 = run_sets(h, sets[:1], args.steps, args.warmup)
         extras["c2_cache_resident_GBps"] = round(rate(P, ms1, args.steps), 1)
+        # not `value`: bundles in flight on two streams hide the gap between dependent launches
+        ms2 = run_sets_two_streams(h, sets, args.steps, args.warmup)
+        extras["c2_two_streams_GBps"] = round(rate(P, ms2, args.steps), 1)
         extras.update({k: round(v, 2) for k, v in end_to_end_us(h, spec).items()})
         del sets
         torch.cuda.empty_cache()
