@@ -147,6 +147,9 @@ Tunables& tunables();
 
 int fail(int status, const std::string& message);   // records thread-local message
 int check_hip(int hip_error, const char* what);     // 0 or AXR_ERR_HIP
+// True for a handle that axr_stream_destroy has destroyed (and no later
+// axr_stream_create has returned again).
+bool stream_retired(void* stream);
 int fail_nothrow(int status, const char* message) noexcept;
 
 // Every extern "C" entry point runs its body through this: no C++ exception

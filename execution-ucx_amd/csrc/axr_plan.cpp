@@ -211,16 +211,21 @@ void invalidate_tables(axr_plan* p) {
 
 // Wait until the device no longer reads the plan's tables.  No event is
 // recorded per launch (it would put a barrier packet between back-to-back
-// bundles); the streams used since the last call are drained instead, and if
-// one of them is gone the whole device is.
+// bundles); the streams used since the last call are drained instead.  A stream
+// that axr_stream_destroy has destroyed in the meantime is not touched again
+// (HIP dereferences the handle): hipStreamDestroy may return before the
+// stream's work has finished, so the whole device is drained for it.
 void quiesce(axr_plan* p) {
+  bool whole_device = false;
   for (hipStream_t s : p->busy_streams) {
-    if (hipStreamSynchronize(s) != hipSuccess) {
+    if (s && stream_retired(s)) {
+      whole_device = true;
+    } else if (hipStreamSynchronize(s) != hipSuccess) {
       (void)hipGetLastError();
-      (void)hipDeviceSynchronize();
-      break;
+      whole_device = true;
     }
   }
+  if (whole_device) (void)hipDeviceSynchronize();
   p->busy_streams.clear();
 }
 

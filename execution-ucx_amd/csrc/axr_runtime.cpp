@@ -9,6 +9,7 @@
 #include <mutex>
 #include <set>
 #include <unordered_map>
+#include <unordered_set>
 #include <utility>
 
 #include "axr_internal.h"
@@ -126,6 +127,21 @@ void table_block_release(TableBlock* block) {
   *block = TableBlock();
 }
 
+}  // namespace axr
+
+// Streams made by axr_stream_create, and the handles of those destroyed since.
+// A plan remembers the streams it ran on and drains them before its tables go
+// away; a handle whose stream is gone must not reach HIP again.
+namespace {
+std::mutex g_stream_mutex;
+std::unordered_set<void*> g_retired_streams;
+}  // namespace
+
+namespace axr {
+bool stream_retired(void* stream) {
+  std::lock_guard<std::mutex> lock(g_stream_mutex);
+  return g_retired_streams.count(stream) != 0;
+}
 }  // namespace axr
 
 using namespace axr;
@@ -437,6 +453,10 @@ static int stream_create_body(void** stream) {
   // Default priority on purpose; non-blocking so it does not serialise with the null stream.
   int rc = check_hip(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate");
   if (rc) return rc;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mutex);
+    g_retired_streams.erase(s);   // the runtime hands addresses out again
+  }
   *stream = s;
   return AXR_OK;
 }
@@ -446,6 +466,10 @@ int axr_stream_create(void** stream) {
 
 static int stream_destroy_body(void* stream) {
   if (!stream) return AXR_OK;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mutex);
+    g_retired_streams.insert(stream);
+  }
   return check_hip(hipStreamDestroy(static_cast<hipStream_t>(stream)), "hipStreamDestroy");
 }
 int axr_stream_destroy(void* stream) {

@@ -132,6 +132,11 @@ AXR_API int axr_device_synchronize(void);
 /* Compute units and bytes of device memory of the current device. */
 AXR_API int axr_device_info(int* compute_units, uint64_t* total_mem, uint64_t* free_mem);
 
+/* Non-blocking streams of default priority.  A plan drains the streams it ran on
+ * before its device tables are released or rewritten (axr_plan_free,
+ * axr_plan_bind and friends): a stream made here may be destroyed while such a
+ * plan is alive (the plan then waits for the whole device instead); a stream made
+ * with hipStreamCreate directly must outlive the plans that ran on it. */
 AXR_API int axr_stream_create(void** stream);
 AXR_API int axr_stream_destroy(void* stream);
 AXR_API int axr_stream_synchronize(void* stream);

@@ -818,6 +818,34 @@ def test_plan_reuse_rebind_and_streams(pkg, orc, gpu):
         pkg._capi.check(lib.axr_stream_destroy(s))
 
 
+def test_plan_outlives_a_stream_it_ran_on(pkg, orc, gpu):
+    """A plan drains the streams it ran on before its tables are rewritten or
+    released.  A stream destroyed with axr_stream_destroy in the meantime must not
+    be touched again: rebinding and freeing such a plan used to crash the process."""
+    lib = pkg._capi.load()
+    rng = np.random.default_rng(9)
+    a = [rand_bytes_tensor(rng, n, gpu) for n in (70000, 33, 4096)]
+    b = [rand_bytes_tensor(rng, n, gpu) for n in (70000, 33, 4096)]
+    want_a = orc.pack([tbytes(t) for t in a], 256)
+    want_b = orc.pack([tbytes(t) for t in b], 256)
+    for then in ("free", "rebind"):
+        plan = pkg.BundlePlan.create(a, align=256)
+        n = plan.payload_bytes
+        out = device_bytes(n, gpu)
+        s = C.c_void_p()
+        pkg._capi.check(lib.axr_stream_create(C.byref(s)))
+        plan.pack(out.data_ptr(), n, s.value)
+        pkg._capi.check(lib.axr_stream_synchronize(s))
+        assert np.array_equal(out.cpu().numpy()[:n], want_a)
+        pkg._capi.check(lib.axr_stream_destroy(s))
+        if then == "rebind":
+            plan.bind(b)
+            plan.pack(out.data_ptr(), n, None)
+            pkg._capi.check(lib.axr_device_synchronize())
+            assert np.array_equal(out.cpu().numpy()[:n], want_b)
+        plan.close()
+
+
 def test_pack_and_unpack_in_a_hip_graph(pkg, orc, gpu):
     """A prepared plan's pack and unpack are single kernel launches that stream
     capture can record.  The graph is replayed several times with eager work and
