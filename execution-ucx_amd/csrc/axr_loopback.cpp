@@ -11,6 +11,7 @@
 #include <memory>
 #include <mutex>
 #include <new>
+#include <set>
 
 #include "axr_internal.h"
 
@@ -48,6 +49,12 @@ bool host_type(int t) { return t == AXR_MEM_HOST || t == AXR_MEM_ROCM_MANAGED; }
 bool known_type(int t) { return host_type(t) || t == AXR_MEM_ROCM; }
 
 std::atomic<uint64_t> g_next_id{1};
+
+// Contexts that exist.  An endpoint is a plain pointer to its peer; a send looks the
+// peer up here (and delivers under this lock), so that a peer destroyed in the
+// meantime is an error and not a dangling pointer.
+std::mutex g_contexts_mu;
+std::set<const void*> g_contexts;
 
 }  // namespace
 
@@ -94,6 +101,11 @@ int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, u
   }
   m->key = g_next_id++;
   m->conn_id = conn_id;
+  std::lock_guard<std::mutex> alive(g_contexts_mu);
+  if (!g_contexts.count(peer)) {
+    m->request->done.store(-1);
+    return fail(AXR_ERR_INVALID, "the connection's peer context has been destroyed");
+  }
   std::lock_guard<std::mutex> lock(peer->mu);
   peer->arrived.push_back(std::move(m));
   return AXR_OK;
@@ -109,6 +121,10 @@ static int am_context_create_body(const char* name, size_t zcopy_thresh, axr_am_
   if (!c) return fail(AXR_ERR_NOMEM, "axr_am_context_create: out of host memory");
   c->name = name ? name : "";
   c->zcopy_thresh = zcopy_thresh ? zcopy_thresh : env_zcopy_thresh();
+  {
+    std::lock_guard<std::mutex> alive(g_contexts_mu);
+    g_contexts.insert(c);
+  }
   *ctx = c;
   return AXR_OK;
 }
@@ -118,6 +134,10 @@ int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_
 
 static int am_context_destroy_body(axr_am_context_t* ctx) {
   if (!ctx) return AXR_OK;
+  {
+    std::lock_guard<std::mutex> alive(g_contexts_mu);   // no delivery is under way past this
+    g_contexts.erase(ctx);
+  }
   {
     std::lock_guard<std::mutex> lock(ctx->mu);
     for (auto& m : ctx->arrived) m->request->done.store(-1);

@@ -395,7 +395,8 @@ typedef struct axr_am_message {
 /* zcopy_thresh 0 reads UCX_ZCOPY_THRESH, else 4096. */
 AXR_API int axr_am_context_create(const char* name, size_t zcopy_thresh, axr_am_context_t** ctx);
 AXR_API int axr_am_context_destroy(axr_am_context_t* ctx);
-/* Endpoint from `from` to `to`; *conn_id names it in axr_am_send*. */
+/* Endpoint from `from` to `to`; *conn_id names it in axr_am_send*.  Sending on it
+ * after `to` has been destroyed fails with AXR_ERR_INVALID. */
 AXR_API int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_id);
 /* *request identifies the send for axr_am_request_test. */
 AXR_API int axr_am_send(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* data,

@@ -116,6 +116,27 @@ def test_fifo_order_and_cancel(pkg, pair):
         assert np.array_equal(dst, src[i:i + 5000]) and client.test(reqs[i])
 
 
+def test_send_to_a_destroyed_peer_is_an_error(pkg):
+    """An endpoint outlives its peer context; sending on it fails cleanly (a closed
+    connection is an error_code in the reference, ucx_am_context.hpp:2318-2392) and
+    the request reads as failed."""
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    src = pattern(10000)
+    ok = client.send(conn, b"first", src.ctypes.data, 10000, memory_type=HOST)
+    server.close()                                           # the queued rendezvous send is cancelled
+    with pytest.raises(pkg.AxonRocmError):
+        client.test(ok)
+    with pytest.raises(pkg.AxonRocmError, match="destroyed"):
+        client.send(conn, b"second", src.ctypes.data, 10000, memory_type=HOST)
+    other = pkg.LoopbackAmContext("other")                   # the client itself still works
+    conn2 = client.connect(other)
+    client.send(conn2, b"third", src.ctypes.data, 16, memory_type=HOST)
+    assert other.recv_header().header == b"third"
+    client.close()
+    other.close()
+
+
 def test_unsupported_memory_type(pkg, pair):
     client, server, conn = pair
     src = pattern(10)
