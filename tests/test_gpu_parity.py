@@ -336,6 +336,77 @@ def random_torch_view(rng, parent, max_dims):
     return v
 
 
+def random_numpy_view(rng, parent):
+    """A view of `parent` with forward and backward steps and permuted dimensions."""
+    index = []
+    for n in parent.shape:
+        lo = int(rng.integers(0, n))
+        hi = int(rng.integers(lo + 1, n + 1))
+        step = int(rng.choice([1, 1, 2, 3, -1, -1, -2]))
+        index.append(slice(lo, hi, step) if step > 0 else slice(hi - 1, lo - 1 if lo else None, step))
+    v = parent[tuple(index)]
+    if rng.random() < 0.6:
+        v = v.transpose(*[int(i) for i in rng.permutation(parent.ndim)])
+    return v
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_views_with_negative_strides(pkg, orc, gpu, seed):
+    """numpy exports views that walk memory backwards (`a[::-1]`); torch never does, so
+    these are described by hand over a device copy of the same bytes.  Gather against
+    the oracle, then scatter into a poisoned twin and compare the whole twin."""
+    import torch
+    rng = np.random.default_rng(100 + seed)
+    dtypes = [(np.uint8, (1, 8, 1)), (np.int16, (0, 16, 1)), (np.float32, (2, 32, 1)),
+              (np.float64, (2, 64, 1)), (np.complex128, (5, 128, 1))]
+    memory = rng.integers(0, 256, size=1 << 23, dtype=np.uint8)
+    device = torch.from_numpy(memory).to(gpu)
+    base = memory.__array_interface__["data"][0]
+    for trial in range(10):
+        described, chunks, at = [], [], 0
+        for _ in range(int(rng.integers(1, 5))):
+            np_dt, dl_dt = dtypes[int(rng.integers(0, len(dtypes)))]
+            item = np.dtype(np_dt).itemsize
+            ndim = int(rng.integers(1, 5))
+            cap = 300 if ndim == 1 else (90 if ndim == 2 else (30 if ndim == 3 else 12))
+            shape = [int(x) for x in rng.integers(1, cap + 1, size=ndim)]
+            if rng.random() < 0.3:
+                shape = [min(n, 6) for n in shape[:-1]] + [int(rng.integers(100, 3000))]
+            nbytes = int(np.prod(shape)) * item
+            at = (at + 15) // 16 * 16 + int(rng.choice([0, 0, item]))
+            assert at + nbytes <= memory.size
+            v = random_numpy_view(rng, memory[at:at + nbytes].view(np_dt).reshape(shape))
+            start = v.__array_interface__["data"][0] - base
+            strides = tuple(st // item for st in v.strides)
+            described.append((start, dl_dt, tuple(v.shape), strides, item))
+            chunks.append(np.ascontiguousarray(v).view(np.uint8).reshape(-1))
+            at += nbytes
+
+        def views_over(tensor):
+            return [pkg.TensorView(data=tensor.data_ptr() + start, device_type=10, device_id=0, dtype=dl_dt,
+                                   shape=shape, strides=strides)
+                    for start, dl_dt, shape, strides, _ in described]
+        align = int(rng.choice([1, 64, 256]))
+        want = orc.pack(chunks, align)
+        plan = pkg.BundlePlan.create(views_over(device), align=align)
+        n = plan.payload_bytes
+        assert n == want.size
+        payload = device_bytes(n, gpu)
+        plan.pack(payload.data_ptr(), n)
+        torch.cuda.synchronize()
+        assert np.array_equal(payload.cpu().numpy()[:n], want), (seed, trial)
+        twin = device_bytes(memory.size, gpu, fill=0x77)
+        back = pkg.BundlePlan.from_header(plan.header).bind(views_over(twin))
+        back.unpack(payload.data_ptr(), n)
+        torch.cuda.synchronize()
+        expect = np.full(memory.size, 0x77, np.uint8)
+        for (start, _, shape, strides, item), c in zip(described, chunks):
+            orc.scatter_strided(c, expect, start, shape, strides, item)
+        assert np.array_equal(twin.cpu().numpy(), expect), (seed, trial)
+        plan.close()
+        back.close()
+
+
 @pytest.mark.parametrize("dtype_name", ["uint8", "bfloat16", "float32", "float64", "complex128"])
 def test_strided_gather_scatter_random(pkg, orc, gpu, dtype_name):
     import torch

@@ -44,7 +44,9 @@ def random_view(rng, parent):
     for n in parent.shape:
         lo = int(rng.integers(0, n))
         hi = int(rng.integers(lo + 1, n + 1))
-        index.append(slice(lo, hi, int(rng.choice([1, 1, 1, 2, 3]))))
+        step = int(rng.choice([1, 1, 1, 2, 3, -1, -2]))
+        # a negative step walks the same range backwards (numpy exports negative strides)
+        index.append(slice(lo, hi, step) if step > 0 else slice(hi - 1, lo - 1 if lo else None, step))
     v = parent[tuple(index)]
     if rng.random() < 0.7:
         v = v.transpose(*[int(i) for i in rng.permutation(parent.ndim)])
