@@ -15,7 +15,8 @@ from .dlpack import DLPackExport, TensorView, extract, extract_many
 from .loopback import AmMessage, LoopbackAmContext
 from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager
 from .pipeline import StreamedTransfer
-from .transfer import recv_tensors, send_tensors
+from .transfer import (classify_argument, flatten_arguments, recv_arguments, recv_tensors, regroup,
+                       send_arguments, send_tensors)
 
 __version__ = "0.1.0"
 

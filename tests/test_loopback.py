@@ -287,3 +287,91 @@ def test_send_recv_tensors_with_memory_policy(pkg, gpu):
             pkg.recv_tensors(server, memory_policy=lambda metas: [torch.zeros(1, device=gpu)], stream=stream)
         assert (bundle.payload_bytes >= 4096) == rndv
     assert pkg.recv_tensors(server) is None
+
+
+# ------------------------------------------------------------------ argument structure
+
+def test_arguments_are_classified_and_flattened_like_the_reference(pkg):
+    """ClassifyArg / add_tensor / add_nested_tensor_list
+    (bindings_runtime_helpers.hpp:262-330, 351-414): tensors in argument order, nested
+    lists flattened with their group sizes kept, empty inner lists allowed."""
+    t = [np.full(i + 1, i, np.float32) for i in range(8)]
+    args = [t[0], [t[1], t[2]], [[t[3]], [], [t[4], t[5]]], (t[6],), [], t[7]]
+    assert [pkg.classify_argument(a) for a in args] == [1, 2, 3, 2, 2, 1]
+    flat, structure = pkg.flatten_arguments(args)
+    assert [id(x) for x in flat] == [id(x) for x in t]                # argument order, depth first
+    assert structure == [(1, []), (2, [2]), (3, [1, 0, 2]), (2, [1]), (2, [0]), (1, [])]
+    from execution_ucx_amd import transfer
+    blob = transfer.encode_structure(structure)
+    assert blob[:4] == b"AXAG" and len(blob) == 8 + 6 * 5 + 4 * (1 + 3 + 1 + 1)
+    back, rest = transfer.decode_structure(blob + b"AXTBrest")
+    assert back == structure and rest == b"AXTBrest"
+    assert transfer.decode_structure(b"AXTBplain") == ([], b"AXTBplain")
+    again = pkg.regroup(structure, flat)
+    assert again[0] is t[0] and again[2] == [[t[3]], [], [t[4], t[5]]] and again[4] == [] and again[5] is t[7]
+    assert isinstance(again[3], list) and again[3][0] is t[6]
+    with pytest.raises(RuntimeError, match="Not enough tensors"):
+        pkg.regroup(structure, flat[:-2])
+    with pytest.raises(RuntimeError):
+        pkg.regroup(structure, flat + [t[0]])
+    with pytest.raises(ValueError):
+        transfer.decode_structure(blob[:-3])
+    with pytest.raises(ValueError):
+        transfer.decode_structure(b"AXAG" + (1).to_bytes(4, "little") + bytes([7]) + (0).to_bytes(4, "little"))
+
+    # what the reference refuses (or sends as plain parameters) is refused here
+    with pytest.raises(TypeError, match="Heterogeneous"):
+        pkg.classify_argument([[], t[1], [t[0]]])                    # met while scanning for a tensor
+    assert pkg.classify_argument([[t[0]], t[1]]) == 3                # the scan stops at the first tensor ...
+    with pytest.raises(TypeError, match="Heterogeneous"):
+        pkg.flatten_arguments([[[t[0]], t[1]]])                      # ... and flattening meets the stray one
+    with pytest.raises(TypeError, match="nested sequence"):
+        pkg.classify_argument([[1, 2], [3]])
+    with pytest.raises(TypeError):
+        pkg.classify_argument([[], []])                              # only empty inner lists: no tensors
+    with pytest.raises(TypeError):
+        pkg.classify_argument(3.5)
+    with pytest.raises(TypeError, match="DLManagedTensor"):
+        pkg.flatten_arguments([[t[0], "not a tensor"]])
+
+
+@pytest.mark.gpu
+def test_send_and_receive_nested_arguments(pkg, gpu):
+    """invoke(a, [b, c], [[d], [], [e, f]]) travels as ONE packed payload and comes back
+    with the same nesting, with and without a memory policy."""
+    import torch
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    g = torch.Generator(device="cpu").manual_seed(5)
+    t = [torch.randn(n, generator=g).to(gpu) for n in (3000, 17, 4096, 1, 999, 70000)]
+    t[2] = t[2].reshape(64, 64).t()                                   # a strided one in the middle
+    args = [t[0], [t[1], t[2]], [[t[3]], [], [t[4], t[5]]]]
+    for use_policy in (False, True):
+        outs = {}
+
+        def policy(metas):
+            outs["tensors"] = [torch.zeros(m.shape, dtype=torch.float32, device=gpu) for m in metas]
+            return outs["tensors"]
+
+        req, bundle = pkg.send_arguments(client, conn, args)
+        got = pkg.recv_arguments(server, memory_policy=policy if use_policy else None,
+                                 from_dlpack_fn=None if use_policy else torch.from_dlpack)
+        assert client.test(req)
+        torch.cuda.synchronize()
+        assert len(got) == 3 and len(got[1]) == 2 and [len(x) for x in got[2]] == [1, 0, 2]
+        flat = [got[0], *got[1], *[x for inner in got[2] for x in inner]]
+        for a, b in zip(flat, t):
+            assert tuple(a.shape) == tuple(b.shape)
+            assert torch.equal(a.reshape(-1).view(torch.uint8).cpu(), b.contiguous().reshape(-1).view(torch.uint8).cpu())
+        if use_policy:
+            assert all(x is y for x, y in zip(flat, outs["tensors"]))     # the policy's own objects
+        del got, flat
+        bundle.plan.close()
+        bundle.payload.release()
+    assert pkg.recv_arguments(server) is None
+    # a plain send_tensors message reads as one list argument
+    req, bundle = pkg.send_tensors(client, conn, t[:2])
+    got = pkg.recv_arguments(server, from_dlpack_fn=torch.from_dlpack)
+    assert len(got) == 1 and len(got[0]) == 2 and torch.equal(got[0][1], t[1])
+    client.close()
+    server.close()
