@@ -137,6 +137,8 @@ class LaunchInfo(C.Structure):
         ("table_bytes", C.c_uint32),
         ("host_copies", C.c_uint32),
         ("host_chunks", C.c_uint32),
+        ("inline_tables", C.c_uint32),
+        ("reserved", C.c_uint32),
     ]
 
 

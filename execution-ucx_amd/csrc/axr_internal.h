@@ -100,6 +100,16 @@ struct KernelArgs {
   uint32_t seg_shift;         // log2 of the tile-block size of wave_seg
 };
 
+// Tables of a small bundle handed to the kernel by value.  bytes[0..16) is a head
+// (a mark the kernel checks, then padding), the Seg array follows at kInlineTablesHead,
+// Dims and the tile-block index at the offsets the launch passes.
+constexpr uint32_t kInlineTableBytes = 3584;
+constexpr uint32_t kInlineTablesHead = 16;
+constexpr uint64_t kInlineTablesMark = 0x31454c4254525841ull;   // "AXRTBLE1"
+struct alignas(16) InlineTables {
+  uint8_t bytes[kInlineTableBytes];
+};
+
 struct LaunchConfig {
   uint32_t workgroups = 0;
   uint32_t tiles_per_wave = 0;
@@ -140,6 +150,8 @@ struct Tunables {
   int64_t transpose = 1;          // move transposed views as square blocks through LDS
   int64_t ragged_runs = 1;        // short runs of 16+ bytes that are no multiple of 16 move in
                                   // 16-byte granules (the last one overlapping) instead of narrower ones
+  int64_t inline_tables = 16384;  // bundles of up to this many tiles whose tables fit the kernel
+                                  // arguments are launched without a table upload; 0: never
 };
 Tunables& tunables();
 
@@ -169,6 +181,11 @@ int guarded(Body&& body) noexcept {
 
 int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& cfg,
                          void* stream);
+// Same launch with the tables inside the kernel arguments (default geometry only:
+// 2 KiB tiles, tensor side streaming, payload side cacheable, no die remapping).
+int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchConfig& cfg,
+                                const InlineTables& tables, uint32_t dims_at, uint32_t wave_at,
+                                void* stream);
 int launch_fill(void* dst, int value, size_t bytes, void* stream);
 
 // ---------------------------------------------------------------- runtime (axr_runtime.cpp)

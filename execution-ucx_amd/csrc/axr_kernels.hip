@@ -15,6 +15,8 @@
 // bundles without them run the small streaming kernels.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
+
 #include "axr_internal.h"
 
 namespace axr {
@@ -693,25 +695,13 @@ __device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_
   }
 }
 
-// At least four waves per SIMD (at most 128 VGPRs): the streaming instantiations
-// use far fewer, and the general ones sit just around that limit, where one
-// register too many would cost a quarter of the occupancy.
+// The whole pack or unpack of a bundle: every wavefront finds the segment of its
+// first tile through the tile-block index and walks forward from there.
 template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
-__global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
-    const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
-    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
-    uint32_t lds_per_wave, uint32_t nt_bits) {
-  // Scalar arguments (not one struct) so that the compiler can preload them
-  // into SGPRs at dispatch instead of fetching the kernarg segment first.
-  KernelArgs a;
-  a.segs = segs_arg;
-  a.dims = dims_arg;
-  a.wave_seg = wave_seg_arg;
-  a.payload = payload_arg;
-  a.ntiles = ntiles;
-  a.tiles_per_wave = tiles_per_wave;
-  a.xcd_remap = xcd_remap;
-  a.seg_shift = seg_shift;
+__device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
+                                            const AXR_CONST uint32_t* wave_seg, gbytes payload,
+                                            const KernelArgs& a, uint32_t lds_per_wave,
+                                            uint32_t nt_bits) {
   constexpr uint32_t kTile = ROWS * kRowBytes;
   const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
   const uint32_t lane_off = lane * kVecBytes;
@@ -726,11 +716,6 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   if (t >= a.ntiles) return;
   const uint32_t t_end =
       (a.ntiles - t > a.tiles_per_wave) ? t + a.tiles_per_wave : a.ntiles;
-  seg_table segs = reinterpret_cast<seg_table>(reinterpret_cast<uintptr_t>(a.segs));
-  dims_table dims = reinterpret_cast<dims_table>(reinterpret_cast<uintptr_t>(a.dims));
-  const AXR_CONST uint32_t* wave_seg =
-      reinterpret_cast<const AXR_CONST uint32_t*>(reinterpret_cast<uintptr_t>(a.wave_seg));
-  gbytes payload = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(a.payload));
   // The index has one entry per block of 2^seg_shift tiles (the planner sizes
   // blocks so that they rarely hold more than one segment); the loop below
   // walks forward from there to the segment of this wave's first tile.
@@ -799,6 +784,65 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
     }
     ++t;
   }
+}
+
+// Tables in device memory (uploaded once per plan).
+// At least four waves per SIMD (at most 128 VGPRs): the streaming instantiations
+// use far fewer, and the general ones sit just around that limit, where one
+// register too many would cost a quarter of the occupancy.
+template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
+__global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
+    const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
+    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
+    uint32_t lds_per_wave, uint32_t nt_bits) {
+  // Scalar arguments (not one struct) so that the compiler can preload them
+  // into SGPRs at dispatch instead of fetching the kernarg segment first.
+  KernelArgs a;
+  a.ntiles = ntiles;
+  a.tiles_per_wave = tiles_per_wave;
+  a.xcd_remap = xcd_remap;
+  a.seg_shift = seg_shift;
+  bundle_body<PACK, ROWS, NTT, NTP, ELEMENTS>(
+      reinterpret_cast<seg_table>(reinterpret_cast<uintptr_t>(segs_arg)),
+      reinterpret_cast<dims_table>(reinterpret_cast<uintptr_t>(dims_arg)),
+      reinterpret_cast<const AXR_CONST uint32_t*>(reinterpret_cast<uintptr_t>(wave_seg_arg)),
+      reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(payload_arg)), a, lds_per_wave, nt_bits);
+}
+
+// Tables of a small bundle travelling in the kernel arguments themselves: no
+// device block, no upload and nothing to keep alive after the launch.  The
+// kernarg segment holds the explicit arguments in order at their natural
+// alignment, so `tables` sits at kInlineTablesOffset; the kernel addresses it
+// there through the constant address space like the uploaded tables, and does
+// nothing unless the first word carries the mark the host wrote.
+struct InlineScalars {   // mirrors the argument list of bundle_kernel_inline
+  uint8_t* payload;
+  uint32_t ntiles, tiles_per_wave, xcd_remap, seg_shift, lds_per_wave, nt_bits, dims_at, wave_at;
+  InlineTables tables;
+};
+constexpr uint32_t kInlineTablesOffset = __builtin_offsetof(InlineScalars, tables);
+static_assert(kInlineTablesOffset == 48 && alignof(InlineTables) == 16, "kernarg layout");
+
+template <bool PACK, bool ELEMENTS>
+__global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel_inline(
+    uint8_t* payload_arg, uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap,
+    uint32_t seg_shift, uint32_t lds_per_wave, uint32_t nt_bits, uint32_t dims_at, uint32_t wave_at,
+    InlineTables tables) {
+  (void)tables;
+  const AXR_CONST uint8_t* base =
+      (const AXR_CONST uint8_t*)__builtin_amdgcn_kernarg_segment_ptr() + kInlineTablesOffset;
+  if (*reinterpret_cast<const AXR_CONST uint64_t*>(base) != kInlineTablesMark) return;
+  KernelArgs a;
+  a.ntiles = ntiles;
+  a.tiles_per_wave = tiles_per_wave;
+  a.xcd_remap = xcd_remap;
+  a.seg_shift = seg_shift;
+  // tensor side streaming, payload side cacheable: what small bundles use
+  bundle_body<PACK, 2, true, false, ELEMENTS>(
+      reinterpret_cast<seg_table>(base + kInlineTablesHead),
+      reinterpret_cast<dims_table>(base + kInlineTablesHead + dims_at),
+      reinterpret_cast<const AXR_CONST uint32_t*>(base + kInlineTablesHead + wave_at),
+      reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(payload_arg)), a, lds_per_wave, nt_bits);
 }
 
 __global__ __launch_bounds__(256) void fill_kernel(uint8_t* dst, uint8_t value, size_t bytes) {
@@ -979,6 +1023,39 @@ int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& 
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   return pack ? launch_dir<true>(args, cfg, s) : launch_dir<false>(args, cfg, s);
+}
+
+int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchConfig& cfg,
+                                const InlineTables& tables, uint32_t dims_at, uint32_t wave_at,
+                                void* stream) {
+  if (args.ntiles == 0 || cfg.workgroups == 0) return AXR_OK;
+  if (cfg.tile_rows != 2 || (cfg.nontemporal & 3u) != 1u || args.xcd_remap)
+    return fail(AXR_ERR_INVALID, "inline tables go with the default launch geometry only");
+  if (cfg.threads == 0 || cfg.threads % kWaveLanes ||
+      cfg.threads > (cfg.elements ? kMaxElementThreads : kMaxThreadsPerWorkgroup))
+    return fail(AXR_ERR_INVALID, "workgroup size does not fit the kernel");
+  if (static_cast<uint64_t>(cfg.lds_per_wave) * (cfg.threads / kWaveLanes) > 64u * 1024u)
+    return fail(AXR_ERR_INVALID, "workgroup needs more than 64 KiB of LDS");
+  const uint64_t covered = static_cast<uint64_t>(cfg.workgroups) * (cfg.threads / kWaveLanes) *
+                           cfg.tiles_per_wave;
+  if (covered < args.ntiles || args.tiles_per_wave != cfg.tiles_per_wave)
+    return fail(AXR_ERR_INVALID, "launch geometry does not cover the tile range");
+  if (std::memcmp(tables.bytes, &kInlineTablesMark, sizeof(kInlineTablesMark)) != 0)
+    return fail(AXR_ERR_INVALID, "inline tables lack their mark");
+  const dim3 grid(cfg.workgroups), block(cfg.threads);
+  const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * (cfg.threads / kWaveLanes) : 0u;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define AXR_INLINE_LAUNCH(PACK, EL)                                                              \
+  hipLaunchKernelGGL((bundle_kernel_inline<PACK, EL>), grid, block, lds_bytes, s, args.payload,   \
+                     args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift,            \
+                     cfg.lds_per_wave, cfg.nontemporal, dims_at, wave_at, tables)
+  if (pack) {
+    if (cfg.elements) AXR_INLINE_LAUNCH(true, true); else AXR_INLINE_LAUNCH(true, false);
+  } else {
+    if (cfg.elements) AXR_INLINE_LAUNCH(false, true); else AXR_INLINE_LAUNCH(false, false);
+  }
+#undef AXR_INLINE_LAUNCH
+  return check_hip(hipGetLastError(), "bundle kernel launch (inline tables)");
 }
 
 int launch_fill(void* dst, int value, size_t bytes, void* stream) {

@@ -338,6 +338,9 @@ static int tune_set_body(const char* key, int64_t value) {
     t.xcd_remap = value ? 1 : 0;
   } else if (k == "ragged_runs") {
     t.ragged_runs = value ? 1 : 0;
+  } else if (k == "inline_tables") {
+    if (value < 0 || value > (1 << 30)) return fail(AXR_ERR_INVALID, "inline_tables must be in [0, 2^30]");
+    t.inline_tables = value;
   } else if (k == "transpose") {
     t.transpose = value ? 1 : 0;
   } else {
@@ -363,6 +366,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "xcd_remap") *value = t.xcd_remap;
   else if (k == "transpose") *value = t.transpose;
   else if (k == "ragged_runs") *value = t.ragged_runs;
+  else if (k == "inline_tables") *value = t.inline_tables;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

@@ -285,7 +285,9 @@ AXR_API int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_byt
  * are resident.  Afterwards axr_pack / axr_unpack of this plan only launch one
  * kernel (no allocation, no copy, no host wait), so they may be recorded into a
  * HIP graph by stream capture; without it a capturing call fails with
- * AXR_ERR_INVALID.  While a graph that holds such a launch can still run, the
+ * AXR_ERR_INVALID, unless the bundle is small enough to carry its tables in the
+ * kernel arguments (axr_launch_info.inline_tables; such a launch is recorded
+ * whole and the plan may even be freed afterwards).  While a graph that holds such a launch can still run, the
  * plan must stay alive and must not be rebound, and the tensors and the payload
  * must stay where they are.  Bundles with kDLCPU tensors cannot be captured
  * (AXR_ERR_UNSUPPORTED).  No counterpart in the reference, whose payload never
@@ -302,6 +304,10 @@ typedef struct axr_launch_info {
   uint32_t table_bytes;    /* device table size                               */
   uint32_t host_copies;    /* contiguous pieces of kDLCPU tensors              */
   uint32_t host_chunks;    /* device copies that move them (pinned staging)    */
+  uint32_t inline_tables;  /* 1: the next launch carries the tables inside the
+                              kernel arguments (small bundle, first launch:
+                              no upload, no device block)                      */
+  uint32_t reserved;
 } axr_launch_info_t;
 AXR_API int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info);
 
@@ -336,8 +342,12 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * tensor side / bit 1 payload side), "payload_cache_bytes", "gather_run_bytes",
  * "xcd_remap", "transpose" (1: transposed views move as square blocks through
  * LDS; 0: element by element), "ragged_runs" (1: short strided runs whose
- * length is no multiple of 16 bytes still move in 16-byte granules).  Unknown
- * key -> AXR_ERR_INVALID. */
+ * length is no multiple of 16 bytes still move in 16-byte granules),
+ * "inline_tables" (the first launch of a bundle of at most this many tiles
+ * whose tables fit into 3.5 KiB carries the tables inside the kernel arguments:
+ * no table upload, nothing to wait for when the plan is freed; a plan that is
+ * launched again uploads its tables then; 0 switches that off; read at every
+ * axr_pack / axr_unpack).  Unknown key -> AXR_ERR_INVALID. */
 AXR_API int axr_tune_set(const char* key, int64_t value);
 AXR_API int axr_tune_get(const char* key, int64_t* value);
 

@@ -917,6 +917,70 @@ def test_plan_outlives_a_stream_it_ran_on(pkg, orc, gpu):
         plan.close()
 
 
+def test_small_bundles_with_tables_in_the_kernel_arguments(pkg, orc, gpu):
+    """Small bundles travel with their tables inside the kernel arguments; the same
+    bundles with that switched off use an uploaded table block.  Both must give the
+    oracle's bytes: plain tensors with pads, strided rows, short strided runs,
+    transposed views, and a mix with a host tensor.  A plan launched this way can be
+    freed at once and captured in a graph without axr_plan_prepare."""
+    import torch
+    rng = np.random.default_rng(55)
+
+    def rb(n):
+        return rand_bytes_tensor(rng, n, gpu)
+    mat = rb(2 * 96 * 80).view(torch.int16).reshape(96, 80)
+    rows = rb(4 * 40 * 1024).view(torch.float32).reshape(40, 1024)
+    cases = {
+        "plain": [rb(5000), rb(1), rb(70001), rb(0), rb(4096)],
+        "strided rows": [rows[:, :600], rb(33)],                      # 2400-byte runs: run tiles
+        "short runs": [rows[:, 5:45], mat[::2, 3:70]],                # element mode
+        "transposed": [mat.t(), rows[:, :64].t(), rb(100)],
+        "with a host tensor": [rb(3000), torch.from_numpy(rng.integers(0, 256, 5000, dtype=np.uint8)), rb(17)],
+    }
+    for name, tensors in cases.items():
+        want = orc.pack([tbytes(t) for t in tensors], 256)
+        for inline in (16384, 0):
+            pkg.tune(inline_tables=inline)
+            try:
+                plan = pkg.BundlePlan.create(tensors, align=256)
+                assert plan.launch_info()["inline_tables"] == (1 if inline else 0), name
+                n, header = plan.payload_bytes, plan.header
+                payload = device_bytes(n, gpu)
+                plan.pack(payload.data_ptr(), n)
+                plan.close()                                           # nothing to wait for when inline
+                torch.cuda.synchronize()
+                assert np.array_equal(payload.cpu().numpy()[:n], want), (name, inline)
+                outs = [torch.zeros(t.shape, dtype=t.dtype, device=t.device) for t in tensors]
+                back = pkg.BundlePlan.from_header(header).bind(outs)
+                assert back.launch_info()["inline_tables"] == (1 if inline else 0), name
+                back.unpack(payload.data_ptr(), n)
+                torch.cuda.synchronize()
+                back.close()
+                for o, t in zip(outs, tensors):
+                    assert np.array_equal(tbytes(o), tbytes(t)), (name, inline)
+            finally:
+                pkg.tune(inline_tables=16384)
+
+    # capture without prepare: the launch carries everything it needs
+    tensors = cases["short runs"] + cases["plain"]
+    want = orc.pack([tbytes(t) for t in tensors], 256)
+    plan = pkg.BundlePlan.create(tensors, align=256)
+    assert plan.launch_info()["inline_tables"] == 1
+    n = plan.payload_bytes
+    payload = device_bytes(n, gpu)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        plan.pack(payload.data_ptr(), n, side.cuda_stream)
+    plan.close()                                                       # the graph keeps its own copy
+    for _ in range(3):
+        payload.fill_(POISON)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(payload.cpu().numpy()[:n], want)
+
+
 def test_pack_and_unpack_in_a_hip_graph(pkg, orc, gpu):
     """A prepared plan's pack and unpack are single kernel launches that stream
     capture can record.  The graph is replayed several times with eager work and

@@ -321,6 +321,35 @@ def test_negative_and_many_strides(pkg):
     assert segs[3]["address"] - segs[0]["address"] == strides[0]
 
 
+def test_small_bundles_carry_their_tables_in_the_kernel_arguments(pkg):
+    """Tables of up to 3.5 KiB (minus a 16-byte head) and bundles of up to `inline_tables`
+    tiles with the default geometry need no device table block."""
+    def info(views, **tune):
+        if tune:
+            pkg.tune(**tune)
+        try:
+            return pkg.BundlePlan.create(views, align=256).launch_info()
+        finally:
+            pkg.tune(tile_rows=0, inline_tables=16384, nontemporal=-1)
+    few = [tv(pkg, 0x10000 * (i + 1), [5000]) for i in range(4)]
+    i = info(few)
+    assert i["inline_tables"] == 1 and i["table_bytes"] + 16 <= 3584
+    assert info(few, inline_tables=0)["inline_tables"] == 0
+    assert info(few, tile_rows=4)["inline_tables"] == 0            # another geometry: uploaded tables
+    assert info(few, nontemporal=3)["inline_tables"] == 0
+    assert info([tv(pkg, 0x10000, [3 * 2048])], inline_tables=2)["inline_tables"] == 0   # 3 tiles > 2
+    assert info([tv(pkg, 0x10000, [3 * 2048])], inline_tables=3)["inline_tables"] == 1
+    many = [tv(pkg, 0x1000 * (i + 1), [100]) for i in range(120)]  # 121 x 32 B of segments alone
+    assert info(many)["inline_tables"] == 0
+    assert info(many[:90])["inline_tables"] == 1
+    big = [tv(pkg, 0x10000000, [64 << 20])]                        # 32768 tiles
+    assert info(big)["inline_tables"] == 0
+    strided = [tv(pkg, 0x10000, [64, 64], strides=[1, 64], dtype=(2, 32, 1)),
+               tv(pkg, 0x90000, [100, 40], strides=[100, 1])]
+    assert info(strided)["inline_tables"] == 1                     # Dims records fit as well
+    assert info([tv(pkg, 0x10000, [0])])["inline_tables"] == 0     # nothing to launch
+
+
 def test_pads_fill_segments_and_host_copies(pkg):
     views = [tv(pkg, 0x10000, [100]),                       # device, pad 156
              tv(pkg, 0x20000, [0]),                         # empty: no segment
