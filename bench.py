@@ -291,6 +291,44 @@ def end_to_end_us(h, spec, steps=20):
             "round_trip_us": times[len(times) // 2] * 1e6}
 
 
+def fresh_small_round_trip(h, tensors=4, each=64 * 1024, steps=200):
+    """Wall time of plan -> pack -> sync -> plan-from-header -> bind -> unpack -> sync for a
+    fresh bundle of a few tensors (the size of a typical RPC argument list), C ABI only."""
+    from execution_ucx_amd.dlpack import TensorArray
+    lib, capi, torch = h.lib, h.capi, h.torch
+    src = [torch.randint(0, 255, (each,), dtype=torch.uint8, device="cuda") for _ in range(tensors)]
+    dst = [torch.zeros_like(t) for t in src]
+    sa, da = TensorArray.from_objects(src), TensorArray.from_objects(dst)
+    probe = h.pkg.BundlePlan.create(src, align=256)
+    nbytes, inline = probe.payload_bytes, probe.launch_info()["inline_tables"]
+    probe.close()
+    payload = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    times = []
+    for it in range(steps + 5):
+        h.sync()
+        t0 = time.perf_counter()
+        p = C.c_void_p()
+        capi.check(lib.axr_plan_create(sa.pointer(), sa.count, 256, 0, C.byref(p)))
+        hp, hn = C.c_void_p(), C.c_size_t()
+        capi.check(lib.axr_plan_header(p, C.byref(hp), C.byref(hn)))
+        capi.check(lib.axr_pack(p, payload.data_ptr(), nbytes, h.stream))
+        capi.check(lib.axr_stream_synchronize(h.stream))
+        r = C.c_void_p()
+        capi.check(lib.axr_plan_from_header(hp, hn.value, C.byref(r)))
+        capi.check(lib.axr_plan_bind(r, da.pointer(), da.count))
+        capi.check(lib.axr_unpack(r, payload.data_ptr(), nbytes, h.stream))
+        capi.check(lib.axr_stream_synchronize(h.stream))
+        t1 = time.perf_counter()
+        capi.check(lib.axr_plan_free(p))
+        capi.check(lib.axr_plan_free(r))
+        if it >= 5:
+            times.append(t1 - t0)
+    assert all(torch.equal(a, b) for a, b in zip(src, dst))
+    times.sort()
+    return {"tensors": tensors, "bytes_each": each, "round_trip_us": round(times[len(times) // 2] * 1e6, 2),
+            "tables_in_kernel_arguments": bool(inline)}
+
+
 def stream_c5(h, chunks=32):
     """8 GiB as 32 chunks of 64 pitched views through the two-stream pipeline."""
     from execution_ucx_amd import workloads
@@ -636,6 +674,7 @@ def main():
                                       "payload_bytes_P": tr[0].data_bytes, "steps": k5}
         del tr
         torch.cuda.empty_cache()
+        extras["fresh_small_bundle"] = fresh_small_round_trip(h)
         extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["loopback_iov_vs_bundle"] = iov_against_bundle(h, spec)
         extras["python_plan_us_per_1k_tensors"] = python_boundary(h, spec)
