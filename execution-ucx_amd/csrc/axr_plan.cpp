@@ -817,15 +817,22 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   if ((capturing ? !p->resident : p->launches == 0 && !p->uploaded) &&
       tables_fit_kernel_arguments(p)) {
     // Small bundle, first launch: the tables ride in the kernel arguments.  The launch
-    // owns its copy, so the plan keeps nothing alive for it and a capturing stream may
-    // record it.  A plan that is launched again is being reused: from the second launch
+    // owns its copy, so a capturing stream may record it.  A plan that is launched again is being reused: from the second launch
     // on it pays one upload and then the shorter argument list (a 3.5 KiB argument costs
     // 0.4 us per launch, the upload 4 us on the host and 4 us on the device, once).
     if (!p->inline_ready) fill_inline_tables(p);
+    rc = launch_bundle_kernel_inline(pack, a, p->cfg, *p->inline_tables,
+                                     static_cast<uint32_t>(p->dims_at),
+                                     static_cast<uint32_t>(p->wave_at), stream);
+    if (rc) return rc;
     ++p->launches;
-    return launch_bundle_kernel_inline(pack, a, p->cfg, *p->inline_tables,
-                                       static_cast<uint32_t>(p->dims_at),
-                                       static_cast<uint32_t>(p->wave_at), stream);
+    // The launch needs nothing of the plan any more, but callers rely on axr_plan_free and
+    // axr_plan_bind returning only when the plan's launches are done (they release the
+    // payload or the tensors next), so the stream is remembered all the same.
+    if (!capturing &&
+        std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+      p->busy_streams.push_back(stream);
+    return AXR_OK;
   }
   if (capturing && !p->resident)
     return fail(AXR_ERR_INVALID, "call axr_plan_prepare before capturing this plan in a graph");

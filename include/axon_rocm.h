@@ -234,6 +234,9 @@ typedef struct axr_plan axr_plan_t;
  * The plan copies shapes and strides; `tensors` may be freed on return. */
 AXR_API int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align,
                             uint32_t flags, axr_plan_t** plan);
+/* Returns when the plan's launches have finished on the streams they were given
+ * (launches recorded into a graph excepted), so the payload and the tensors may be
+ * released right after it. */
 AXR_API int axr_plan_free(axr_plan_t* plan);
 
 AXR_API int axr_plan_num_tensors(const axr_plan_t* plan, size_t* n);
@@ -287,7 +290,7 @@ AXR_API int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_byt
  * HIP graph by stream capture; without it a capturing call fails with
  * AXR_ERR_INVALID, unless the bundle is small enough to carry its tables in the
  * kernel arguments (axr_launch_info.inline_tables; such a launch is recorded
- * whole and the plan may even be freed afterwards).  While a graph that holds such a launch can still run, the
+ * whole and the plan may be freed afterwards).  While a graph that holds such a launch can still run, the
  * plan must stay alive and must not be rebound, and the tensors and the payload
  * must stay where they are.  Bundles with kDLCPU tensors cannot be captured
  * (AXR_ERR_UNSUPPORTED).  No counterpart in the reference, whose payload never
@@ -345,8 +348,8 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * length is no multiple of 16 bytes still move in 16-byte granules),
  * "inline_tables" (the first launch of a bundle of at most this many tiles
  * whose tables fit into 3.5 KiB carries the tables inside the kernel arguments:
- * no table upload, nothing to wait for when the plan is freed; a plan that is
- * launched again uploads its tables then; 0 switches that off; read at every
+ * no table block and no upload; a plan that is launched again uploads its
+ * tables then; 0 switches that off; read at every
  * axr_pack / axr_unpack).  Unknown key -> AXR_ERR_INVALID. */
 AXR_API int axr_tune_set(const char* key, int64_t value);
 AXR_API int axr_tune_get(const char* key, int64_t* value);

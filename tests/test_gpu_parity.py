@@ -947,7 +947,7 @@ def test_small_bundles_with_tables_in_the_kernel_arguments(pkg, orc, gpu):
                 n, header = plan.payload_bytes, plan.header
                 payload = device_bytes(n, gpu)
                 plan.pack(payload.data_ptr(), n)
-                plan.close()                                           # nothing to wait for when inline
+                plan.close()                                           # waits for the launch
                 torch.cuda.synchronize()
                 assert np.array_equal(payload.cpu().numpy()[:n], want), (name, inline)
                 outs = [torch.zeros(t.shape, dtype=t.dtype, device=t.device) for t in tensors]
