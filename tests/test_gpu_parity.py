@@ -374,7 +374,8 @@ def test_views_with_negative_strides(pkg, orc, gpu, seed):
                 shape = [min(n, 6) for n in shape[:-1]] + [int(rng.integers(100, 3000))]
             nbytes = int(np.prod(shape)) * item
             at = (at + 15) // 16 * 16 + int(rng.choice([0, 0, item]))
-            assert at + nbytes <= memory.size
+            if at + nbytes > memory.size:
+                break                                       # this trial has enough tensors
             v = random_numpy_view(rng, memory[at:at + nbytes].view(np_dt).reshape(shape))
             start = v.__array_interface__["data"][0] - base
             strides = tuple(st // item for st in v.strides)
@@ -386,6 +387,8 @@ def test_views_with_negative_strides(pkg, orc, gpu, seed):
             return [pkg.TensorView(data=tensor.data_ptr() + start, device_type=10, device_id=0, dtype=dl_dt,
                                    shape=shape, strides=strides)
                     for start, dl_dt, shape, strides, _ in described]
+        if not described:
+            continue
         align = int(rng.choice([1, 64, 256]))
         want = orc.pack(chunks, align)
         plan = pkg.BundlePlan.create(views_over(device), align=align)
