@@ -227,9 +227,19 @@ def _torch_exporter() -> tuple:
         return ()
     device = -1   # no GPU context: only host tensors can exist
     if torch.cuda.is_initialized():
-        if torch.cuda.current_stream() != torch.cuda.default_stream():
-            return ()
-        device = torch.cuda.current_device()
+        raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        get_device = getattr(torch._C, "_cuda_getDevice", None)
+        if raw_stream is not None and get_device is not None:
+            # the same two questions through torch's C entry points (0.3 us instead
+            # of 7 us, which matters for bundles of a few tensors); the default
+            # stream is the null handle
+            device = get_device()
+            if raw_stream(device) != 0:
+                return ()
+        else:
+            if torch.cuda.current_stream() != torch.cuda.default_stream():
+                return ()
+            device = torch.cuda.current_device()
     return (torch.Tensor, torch.utils.dlpack.to_dlpack, device)
 
 
