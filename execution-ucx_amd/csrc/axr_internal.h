@@ -150,6 +150,7 @@ struct Tunables {
   int64_t transpose = 1;          // move transposed views as square blocks through LDS
   int64_t ragged_runs = 1;        // short runs of 16+ bytes that are no multiple of 16 move in
                                   // 16-byte granules (the last one overlapping) instead of narrower ones
+  int64_t host_threads = 4;       // threads (the caller included) for host-side staging copies
   int64_t inline_tables = 16384;  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
 };
@@ -159,6 +160,16 @@ Tunables& tunables();
 
 int fail(int status, const std::string& message);   // records thread-local message
 int check_hip(int hip_error, const char* what);     // 0 or AXR_ERR_HIP
+// Host-side copies of the staging paths (pageable memory <-> pinned blocks).  One core
+// moves about 25 GB/s, less than the PCIe link; jobs of 2 MiB and more in total are cut
+// into byte-balanced shares for up to `host_threads` short-lived threads.
+struct HostCopyJob {
+  void* dst;
+  const void* src;
+  size_t bytes;
+};
+void host_copy(const HostCopyJob* jobs, size_t count);
+
 // True for a handle that axr_stream_destroy has destroyed (and no later
 // axr_stream_create has returned again).
 bool stream_retired(void* stream);

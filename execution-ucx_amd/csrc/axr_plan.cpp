@@ -706,11 +706,14 @@ int stage_acquire(HostStage* st) {
 // memory does).  Two blocks alternate.
 int move_host_tensors(axr_plan* p, bool pack, uint8_t* payload, hipStream_t stream) {
   const size_t nchunks = p->host_chunks.size();
-  auto pieces_out = [p](const HostChunk& c, const uint8_t* staged) {
+  std::vector<HostCopyJob> jobs;
+  auto pieces_out = [p, &jobs](const HostChunk& c, const uint8_t* staged) {
+    jobs.clear();
     for (uint32_t i = c.first; i < c.first + c.count; ++i) {
       const HostCopy& hc = p->host_copies[i];
-      std::memcpy(reinterpret_cast<void*>(hc.host), staged + (hc.offset - c.begin), hc.bytes);
+      jobs.push_back({reinterpret_cast<void*>(hc.host), staged + (hc.offset - c.begin), hc.bytes});
     }
+    host_copy(jobs.data(), jobs.size());
   };
   for (size_t k = 0; k < nchunks; ++k) {
     const HostChunk& c = p->host_chunks[k];
@@ -726,12 +729,14 @@ int move_host_tensors(axr_plan* p, bool pack, uint8_t* payload, hipStream_t stre
     const size_t span = static_cast<size_t>(c.end - c.begin);
     if (pack) {
       uint64_t at = c.begin;
+      jobs.clear();
       for (uint32_t i = c.first; i < c.first + c.count; ++i) {
         const HostCopy& hc = p->host_copies[i];
         if (hc.offset > at) std::memset(staged + (at - c.begin), 0, hc.offset - at);
-        std::memcpy(staged + (hc.offset - c.begin), reinterpret_cast<const void*>(hc.host), hc.bytes);
+        jobs.push_back({staged + (hc.offset - c.begin), reinterpret_cast<const void*>(hc.host), hc.bytes});
         at = hc.offset + hc.bytes;
       }
+      host_copy(jobs.data(), jobs.size());
       rc = check_hip(hipMemcpyAsync(payload + c.begin, staged, span, hipMemcpyDefault, stream),
                      "hipMemcpyAsync(host tensors -> payload)");
     } else {
