@@ -164,7 +164,8 @@ AXR_API int axr_mem_free(int memory_type, void* ptr, size_t bytes);
  * of ucx_cuda_memory_manager.hpp:62-78 extended with the pinned type.  ROCM to
  * HOST copies of 16 MiB and more go through two pinned staging blocks that up
  * to "host_threads" threads empty (the checkpoint writer's mr.memcpy(HOST, ...),
- * avro_serialization.cpp:478-523): 51 GB/s instead of 18 GB/s for 1 GiB. */
+ * avro_serialization.cpp:478-523): 51 GB/s instead of 18 GB/s for 1 GiB; HOST to
+ * ROCM copies of that size are staged the same way. */
 AXR_API int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t bytes);
 /* Same, enqueued on `stream`; pageable host memory makes it synchronous. */
 AXR_API int axr_memcpy_async(int dst_type, void* dst, int src_type, const void* src,

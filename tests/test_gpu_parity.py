@@ -1140,9 +1140,9 @@ def test_concurrent_host_threads(pkg, orc, gpu):
 # ------------------------------------------------------------------ memory resource
 
 def test_large_copy_to_pageable_host_memory(pkg, gpu):
-    """axr_memcpy from the device into pageable memory goes through pinned staging
-    blocks from 16 MiB on: three whole blocks and an odd tail, and the sizes around
-    the switch."""
+    """axr_memcpy between the device and pageable memory goes through pinned staging
+    blocks from 16 MiB on, in both directions: three whole blocks and an odd tail,
+    and the sizes around the switch."""
     import torch
     lib, capi = pkg._capi.load(), pkg._capi
     for n in ((16 << 20) - 1, 16 << 20, (24 << 20) + 12345, (40 << 20) + 7):
@@ -1151,6 +1151,12 @@ def test_large_copy_to_pageable_host_memory(pkg, gpu):
         capi.check(lib.axr_memcpy(capi.MEM_HOST, host.ctypes.data + 32, capi.MEM_ROCM, dev.data_ptr(), n))
         assert np.array_equal(host[32:32 + n], dev.cpu().numpy()), n
         assert (host[:32] == 0xEE).all() and (host[32 + n:] == 0xEE).all()
+        # and back from pageable memory, staged from the same size on
+        back = torch.full((n + 64,), 0x11, dtype=torch.uint8, device=gpu)
+        capi.check(lib.axr_memcpy(capi.MEM_ROCM, back.data_ptr() + 32, capi.MEM_HOST, host.ctypes.data + 32, n))
+        got = back.cpu().numpy()
+        assert np.array_equal(got[32:32 + n], host[32:32 + n]), n
+        assert (got[:32] == 0x11).all() and (got[32 + n:] == 0x11).all()
 
 
 def test_pool_and_copy_table(pkg, gpu):
