@@ -230,6 +230,94 @@ def decode_header(blob: bytes) -> Tuple[int, int, List[dict]]:
     return align, total, tensors
 
 
+# ---------------------------------------------------------------- argument structure
+
+def flatten_arguments(args: Sequence, is_tensor) -> Tuple[list, List[Tuple[str, List[int]]]]:
+    """Restatement of how the reference turns invoke() arguments into ONE tensor
+    stream (axon/python/src/bindings_runtime_helpers.hpp): ClassifyArg (:262-330)
+    decides per argument -- a tensor; a list/tuple whose first element is a tensor, or
+    an empty one (flat list); a list/tuple of lists/tuples where the first non-empty
+    inner one starts with a tensor (nested list) -- then add_tensor (:351-362) appends
+    single tensors and the elements of flat lists in order, and add_nested_tensor_list
+    (:387-414) appends every inner list's tensors in order and records one uint32
+    group size per inner list, empty ones included.  Pinned by the cases of the
+    reference's own test (axon/python/tests/test_numpy_rpc.py:271-298: a tuple of
+    tensors is a flat list, `[[], [t]]` is a nested list although its first inner list
+    is empty, `[]` is an empty flat list), by the description at :366-386 (all tensors
+    of every inner list in order, one count per inner list) and by the receiver's
+    regrouping loop (bindings_runtime_wrapper.cpp:183-228), which regroup_arguments
+    restates: flatten followed by regroup must give the arguments back.
+
+    Returns (tensors, [(kind, counts)]) with kind in "single" / "flat" / "nested".
+    """
+    tensors, structure = [], []
+    for arg in args:
+        if is_tensor(arg):
+            tensors.append(arg)
+            structure.append(("single", []))
+            continue
+        if not isinstance(arg, (list, tuple)):
+            raise TypeError("non-tensor argument")
+        if len(arg) == 0 or is_tensor(arg[0]):
+            tensors.extend(arg)
+            structure.append(("flat", [len(arg)]))
+            continue
+        found = False
+        for inner in arg:                       # the scan of ClassifyArg
+            if not isinstance(inner, (list, tuple)):
+                raise TypeError("heterogeneous sequence")
+            if len(inner) == 0:
+                continue
+            if not is_tensor(inner[0]):
+                raise TypeError("unsupported element inside nested sequence")
+            found = True
+            break
+        if not found:
+            raise TypeError("non-tensor argument")
+        sizes = []
+        for inner in arg:                       # add_nested_tensor_list
+            tensors.extend(inner)
+            sizes.append(len(inner))
+        structure.append(("nested", sizes))
+    return tensors, structure
+
+
+def regroup_arguments(structure: Sequence[Tuple[str, Sequence[int]]], tensors: Sequence) -> list:
+    """The receiver's loop (bindings_runtime_wrapper.cpp:183-228): consume the flat
+    tensor stream in order, `gsz` tensors per inner list."""
+    out, at = [], 0
+    for kind, counts in structure:
+        if kind == "single":
+            out.append(tensors[at])
+            at += 1
+        elif kind == "flat":
+            out.append(list(tensors[at:at + counts[0]]))
+            at += counts[0]
+        else:
+            outer = []
+            for gsz in counts:
+                outer.append(list(tensors[at:at + gsz]))
+                at += gsz
+            out.append(outer)
+    return out
+
+
+def encode_argument_structure(structure: Sequence[Tuple[str, Sequence[int]]]) -> bytes:
+    """Independent writer of the build's own framing of that structure (the reference
+    carries the group sizes as a cista VECTOR_UINT32 header parameter, unpinned like the
+    rest of its header): "AXAG", u32 argument count, then per argument u8 kind (1 single,
+    2 flat, 3 nested), u32 number of counts, the counts as u32 -- little-endian."""
+    code = {"single": 1, "flat": 2, "nested": 3}
+    blob = bytearray(b"AXAG")
+    blob += len(structure).to_bytes(4, "little")
+    for kind, counts in structure:
+        blob.append(code[kind])
+        blob += len(counts).to_bytes(4, "little")
+        for c in counts:
+            blob += int(c).to_bytes(4, "little")
+    return bytes(blob)
+
+
 # ---------------------------------------------------------------- CPU timing
 
 def time_pack_unpack(chunks: Sequence[np.ndarray], align: int = 1, threads: int = 1,

@@ -7,6 +7,8 @@ bundle_header_v1.json   tensor list + alignment -> header bytes (hex), by the
                         oracle's independent struct-based codec
 small_bundle_v1.json    seeded byte chunks -> packed payload (hex) for the tight
                         (align 1) and the 256-byte aligned layout
+argument_structure_v1.json  nested argument lists (tensors named by letters) -> flat
+                        tensor order, group sizes and the framing bytes (hex)
 kat_patterns.json       the closed-form patterns of the reference's own tests
                         (segment lengths and fill rule; expected = the running
                         pattern), so the data the reference tests hold is kept
@@ -52,6 +54,21 @@ def main():
         small["packed"][str(align)] = oracle.pack(chunks, align).tobytes().hex()
     with open(os.path.join(HERE, "small_bundle_v1.json"), "w") as f:
         json.dump(small, f, indent=1)
+
+    # the reference's own example first (bindings_runtime_helpers.hpp:364-386)
+    arg_cases = [
+        [[["a", "b"], ["c"]]],
+        ["a", ["b", "c"], [["d"], [], ["e", "f"]], ["g"], [], "h"],
+        [[[], [], ["a"]], [["b", "c", "d"]]],
+        [],
+    ]
+    out = []
+    for args in arg_cases:
+        flat, structure = oracle.flatten_arguments(args, lambda x: isinstance(x, str))
+        out.append({"args": args, "flat": flat, "structure": [[k, c] for k, c in structure],
+                    "blob_hex": oracle.encode_argument_structure(structure).hex()})
+    with open(os.path.join(HERE, "argument_structure_v1.json"), "w") as f:
+        json.dump(out, f, indent=1)
 
     kat = {
         "fill_rule": "byte k of the concatenated stream = k mod 256",

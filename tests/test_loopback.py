@@ -335,6 +335,49 @@ def test_arguments_are_classified_and_flattened_like_the_reference(pkg):
         pkg.flatten_arguments([[t[0], "not a tensor"]])
 
 
+def test_argument_structure_matches_the_oracle_and_the_fixture(pkg, orc):
+    """The package's flattening, framing and regrouping against the oracle's restatement
+    of the reference on random nestings, and against the committed fixture."""
+    import json
+    import os
+    from execution_ucx_amd import transfer
+    kinds = {1: "single", 2: "flat", 3: "nested"}
+    rng = np.random.default_rng(4)
+    mk = lambda: np.zeros(int(rng.integers(1, 5)), np.float32)
+    for _ in range(200):
+        args = []
+        for _ in range(int(rng.integers(0, 6))):
+            k = int(rng.integers(0, 3))
+            if k == 0:
+                args.append(mk())
+            elif k == 1:
+                args.append([mk() for _ in range(int(rng.integers(0, 4)))])
+            else:
+                inner = [[mk() for _ in range(int(rng.integers(0, 4)))] for _ in range(int(rng.integers(1, 4)))]
+                if not any(inner):
+                    inner.append([mk()])            # only empty inner lists hold no tensor at all
+                args.append(inner)
+        flat, structure = pkg.flatten_arguments(args)
+        oflat, ostructure = orc.flatten_arguments(args, lambda x: isinstance(x, np.ndarray))
+        assert [id(x) for x in flat] == [id(x) for x in oflat]
+        assert [(kinds[k], c) for k, c in structure] == ostructure
+        blob = transfer.encode_structure(structure)
+        assert blob == orc.encode_argument_structure(ostructure)
+        assert transfer.decode_structure(blob + b"AXTB")[0] == structure
+        back, oback = pkg.regroup(structure, flat), orc.regroup_arguments(ostructure, oflat)
+        same = lambda a, b: (a is b) if isinstance(a, np.ndarray) else (len(a) == len(b) and all(map(same, a, b)))
+        assert same(back, oback) and same(back, [list(a) if isinstance(a, tuple) else a for a in args])
+    here = os.path.dirname(os.path.abspath(__file__))
+    for c in json.load(open(os.path.join(here, "golden", "argument_structure_v1.json"))):
+        class Named(str):
+            __dlpack__ = None                        # stands in for a tensor
+        def named(x):
+            return Named(x) if isinstance(x, str) else [named(y) for y in x]
+        flat, structure = pkg.flatten_arguments(named(c["args"]))
+        assert [str(x) for x in flat] == c["flat"]
+        assert transfer.encode_structure(structure).hex() == c["blob_hex"]
+
+
 @pytest.mark.gpu
 def test_send_and_receive_nested_arguments(pkg, gpu):
     """invoke(a, [b, c], [[d], [], [e, f]]) travels as ONE packed payload and comes back

@@ -1,9 +1,13 @@
 """Pins the CPU oracle: the reference's own known-answer tests, the compiled
 reference (oracle/_ref, when built) and what the mathematics fixes."""
 import ctypes as C
+import json
+import os
 
 import numpy as np
 import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
 def pattern(n, start=0):
@@ -269,3 +273,32 @@ def test_header_roundtrip(orc):
     assert [t["nbytes"] for t in back] == [65536, 30, 0, 0]
     for a, b in zip(tensors, back):
         assert a["device"] == b["device"] and a["dtype"] == b["dtype"] and tuple(a["shape"]) == b["shape"]
+
+
+# ------------------------------------------------------------------ argument structure
+
+def test_argument_classification_cases_of_the_reference(orc):
+    """axon/python/tests/test_numpy_rpc.py:271-298: a tuple of tensors, a nested list
+    that starts with an empty inner list, and an empty outer list."""
+    t = np.ones((10,), dtype=np.float32)
+    is_tensor = lambda x: isinstance(x, np.ndarray)
+    assert orc.flatten_arguments([(t, t)], is_tensor)[1] == [("flat", [2])]
+    flat, structure = orc.flatten_arguments([[[], [t]]], is_tensor)
+    assert structure == [("nested", [0, 1])] and len(flat) == 1 and flat[0] is t
+    assert orc.flatten_arguments([[]], is_tensor) == ([], [("flat", [0])])
+    # flatten then regroup is the identity (lists and tuples both come back as lists)
+    args = [t, [t, t], [[t], [], [t, t]], []]
+    flat, structure = orc.flatten_arguments(args, is_tensor)
+    assert len(flat) == 6
+    back = orc.regroup_arguments(structure, flat)
+    assert back[0] is t and [len(x) for x in back[2]] == [1, 0, 2] and back[3] == []
+
+
+def test_argument_structure_fixture(orc):
+    cases = json.load(open(os.path.join(GOLDEN, "argument_structure_v1.json")))
+    assert cases[0]["flat"] == ["a", "b", "c"] and cases[0]["structure"] == [["nested", [2, 1]]]
+    for c in cases:
+        flat, structure = orc.flatten_arguments(c["args"], lambda x: isinstance(x, str))
+        assert flat == c["flat"] and [[k, n] for k, n in structure] == c["structure"]
+        assert orc.encode_argument_structure(structure).hex() == c["blob_hex"]
+        assert orc.regroup_arguments(structure, flat) == c["args"]
