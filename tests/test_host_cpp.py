@@ -36,3 +36,36 @@ def test_host_layer_on_device(gpu):
     out = subprocess.run([SELFTEST], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "host_selftest ok" in out.stdout
+
+
+def test_planner_and_header_codec_under_sanitizers(tmp_path):
+    """tests/cpp/plan_fuzz.cpp against a planner compiled with AddressSanitizer and
+    UBSan (host code only; the kernels' object file is linked as built): random tensor
+    descriptors through every inspection call, and mutated headers through the
+    decoder, which must refuse them or accept only what re-encodes to the same bytes."""
+    pkgdir = os.path.join(ROOT, "execution-ucx_amd")
+    objs = [os.path.join(pkgdir, "build", n) for n in
+            ("axr_runtime.cpp.o", "axr_loopback.cpp.o", "axr_kernels.hip.o")]
+    hipcc, clang = "/opt/rocm/bin/hipcc", "/opt/rocm/llvm/bin/clang++"
+    if not all(os.path.exists(p) for p in objs + [hipcc, clang]):
+        pytest.skip("needs the library's object files (make -C execution-ucx_amd) and the ROCm compilers")
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(pkgdir, "csrc")]
+    san = ["-fsanitize=address", "-fsanitize=undefined", "-fno-sanitize-recover=undefined"]
+    plan_o, fuzz_o, exe = (str(tmp_path / n) for n in ("axr_plan.o", "plan_fuzz.o", "plan_fuzz"))
+    host_san = [x for flag in san for x in ("-Xarch_host", flag)]
+    steps = [
+        [hipcc, "--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-fPIC", *host_san,
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", *inc,
+         "-x", "hip", "-c", os.path.join(pkgdir, "csrc", "axr_plan.cpp"), "-o", plan_o],
+        [clang, "-O1", "-g", "-std=c++17", *san, *inc, "-c",
+         os.path.join(ROOT, "tests", "cpp", "plan_fuzz.cpp"), "-o", fuzz_o],
+        [hipcc, "--offload-arch=gfx950", *san[:2], "-fno-gpu-sanitize", fuzz_o, plan_o, *objs,
+         "-o", exe, "-lpthread"],
+    ]
+    for cmd in steps:
+        out = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        assert out.returncode == 0, out.stderr[-3000:]
+    out = subprocess.run([exe, "7", "1200"], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, (out.stdout + out.stderr)[-3000:]
+    assert "plan_fuzz ok" in out.stdout
