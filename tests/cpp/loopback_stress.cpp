@@ -1,0 +1,136 @@
+// Thread-safety stress of the loopback active-message context on host memory (no GPU),
+// meant to be built with ThreadSanitizer (tests/test_host_cpp.py does that): several
+// sender threads, each on a connection of its own, push eager and rendezvous messages
+// at one server context while a receiver thread drains it and checks every payload,
+// and another thread creates, connects and destroys unrelated contexts.  The reference's
+// context is reached from any thread with the work hopping to the context thread
+// (ucx_context/ucx_am_context/ucx_am_context.hpp:2318-2392); here a mutex per context
+// stands in for that hop.  Prints "loopback_stress ok <messages>" and exits 0.
+#include <atomic>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#include "axon_rocm.h"
+
+namespace {
+
+constexpr int kSenders = 4;
+constexpr int kPerSender = 400;
+
+void die(const char* what, int rc) {
+  std::fprintf(stderr, "loopback_stress: %s -> %d (%s)\n", what, rc, axr_last_error());
+  std::exit(1);
+}
+
+struct Tag {   // the AM header of every message
+  uint32_t sender, seq, bytes, pad;
+};
+
+uint8_t byte_of(uint32_t sender, uint32_t seq, size_t i) {
+  return static_cast<uint8_t>(sender * 131u + seq * 7u + i);
+}
+
+}  // namespace
+
+int main() {
+  axr_am_context_t* server = nullptr;
+  if (int rc = axr_am_context_create("server", 4096, &server)) die("create server", rc);
+  std::atomic<int> received{0};
+  std::atomic<bool> stop_churn{false};
+
+  std::vector<std::thread> threads;
+  for (int s = 0; s < kSenders; ++s) {
+    threads.emplace_back([s, server] {
+      axr_am_context_t* client = nullptr;
+      if (int rc = axr_am_context_create("client", 4096, &client)) die("create client", rc);
+      uint64_t conn = 0;
+      if (int rc = axr_am_connect(client, server, &conn)) die("connect", rc);
+      // rendezvous sources must stay valid until the request completes
+      std::vector<std::vector<uint8_t>> live(kPerSender);
+      std::vector<uint64_t> requests(kPerSender);
+      for (int q = 0; q < kPerSender; ++q) {
+        const uint32_t bytes = (q % 3 == 0) ? 8192u + static_cast<uint32_t>(q) : static_cast<uint32_t>(q % 200);
+        live[q].resize(bytes);
+        for (size_t i = 0; i < bytes; ++i) live[q][i] = byte_of(s, q, i);
+        Tag tag{static_cast<uint32_t>(s), static_cast<uint32_t>(q), bytes, 0};
+        axr_am_data_t d;
+        std::memset(&d, 0, sizeof(d));
+        d.header.data = &tag;
+        d.header.size = sizeof(tag);
+        d.buffer.data = bytes ? live[q].data() : nullptr;
+        d.buffer.size = bytes;
+        d.buffer_type = AXR_MEM_HOST;
+        if (int rc = axr_am_send(client, conn, &d, nullptr, &requests[q])) die("send", rc);
+      }
+      for (int q = 0; q < kPerSender; ++q) {
+        int done = 0;
+        while (!done) {
+          if (int rc = axr_am_request_test(client, requests[q], &done)) die("request_test", rc);
+          if (done < 0) die("request failed", done);
+          if (!done) std::this_thread::yield();
+        }
+      }
+      if (int rc = axr_am_context_destroy(client)) die("destroy client", rc);
+    });
+  }
+  threads.emplace_back([server, &received] {
+    std::vector<uint32_t> next(kSenders, 0);
+    std::vector<uint8_t> buf(16384);
+    while (received.load() < kSenders * kPerSender) {
+      axr_am_message_t m;
+      const int rc = axr_am_recv_header(server, &m);
+      if (rc == AXR_ERR_NO_MESSAGE) {
+        std::this_thread::yield();
+        continue;
+      }
+      if (rc) die("recv_header", rc);
+      Tag tag;
+      if (m.header.size != sizeof(tag)) die("header size", -1);
+      std::memcpy(&tag, m.header.data, sizeof(tag));
+      if (tag.sender >= static_cast<uint32_t>(kSenders) || tag.seq != next[tag.sender]++) die("order per connection", -1);
+      if (m.data_length != tag.bytes) die("length", -1);
+      const uint8_t* got = nullptr;
+      if (m.is_rndv) {
+        if (int rc2 = axr_am_recv_buffer(server, m.key, AXR_MEM_HOST, buf.data(), buf.size(), nullptr)) die("recv_buffer", rc2);
+        got = buf.data();
+      } else {
+        got = static_cast<const uint8_t*>(m.eager_data.data);
+      }
+      for (size_t i = 0; i < tag.bytes; ++i)
+        if (got[i] != byte_of(tag.sender, tag.seq, i)) die("payload", -1);
+      if (!m.is_rndv) {
+        if (int rc2 = axr_am_message_release(server, m.key)) die("release", rc2);
+      }
+      received.fetch_add(1);
+    }
+  });
+  threads.emplace_back([&stop_churn] {   // unrelated contexts come and go
+    while (!stop_churn.load()) {
+      axr_am_context_t *a = nullptr, *b = nullptr;
+      if (int rc = axr_am_context_create("a", 0, &a)) die("create a", rc);
+      if (int rc = axr_am_context_create("b", 0, &b)) die("create b", rc);
+      uint64_t conn = 0;
+      if (int rc = axr_am_connect(a, b, &conn)) die("connect a b", rc);
+      if (int rc = axr_am_context_destroy(b)) die("destroy b", rc);
+      uint32_t word = 1;
+      axr_am_data_t d;
+      std::memset(&d, 0, sizeof(d));
+      d.header.data = &word;
+      d.header.size = sizeof(word);
+      d.buffer_type = AXR_MEM_HOST;
+      uint64_t req = 0;
+      if (axr_am_send(a, conn, &d, nullptr, &req) != AXR_ERR_INVALID) die("send to a destroyed peer", -1);
+      if (int rc = axr_am_context_destroy(a)) die("destroy a", rc);
+    }
+  });
+  for (size_t i = 0; i + 1 < threads.size(); ++i) threads[i].join();
+  stop_churn.store(true);
+  threads.back().join();
+  if (int rc = axr_am_context_destroy(server)) die("destroy server", rc);
+  std::printf("loopback_stress ok %d\n", received.load());
+  return 0;
+}

@@ -69,3 +69,34 @@ def test_planner_and_header_codec_under_sanitizers(tmp_path):
     out = subprocess.run([exe, "7", "1200"], capture_output=True, text=True, timeout=600)
     assert out.returncode == 0, (out.stdout + out.stderr)[-3000:]
     assert "plan_fuzz ok" in out.stdout
+
+
+def test_loopback_context_under_thread_sanitizer(tmp_path):
+    """tests/cpp/loopback_stress.cpp with the loopback context and the runtime shim
+    compiled with ThreadSanitizer (host code only, host memory only): four senders, one
+    receiver and a thread that creates and destroys contexts, all at once."""
+    pkgdir = os.path.join(ROOT, "execution-ucx_amd")
+    objs = [os.path.join(pkgdir, "build", n) for n in ("axr_plan.cpp.o", "axr_kernels.hip.o")]
+    hipcc, clang = "/opt/rocm/bin/hipcc", "/opt/rocm/llvm/bin/clang++"
+    if not all(os.path.exists(p) for p in objs + [hipcc, clang]):
+        pytest.skip("needs the library's object files (make -C execution-ucx_amd) and the ROCm compilers")
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(pkgdir, "csrc")]
+    built = []
+    for name in ("axr_loopback", "axr_runtime"):
+        built.append(str(tmp_path / (name + ".o")))
+        cmd = [hipcc, "--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-fPIC",
+               "-Xarch_host", "-fsanitize=thread", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", *inc,
+               "-x", "hip", "-c", os.path.join(pkgdir, "csrc", name + ".cpp"), "-o", built[-1]]
+        out = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        assert out.returncode == 0, out.stderr[-3000:]
+    stress_o, exe = str(tmp_path / "loopback_stress.o"), str(tmp_path / "loopback_stress")
+    for cmd in ([clang, "-O1", "-g", "-std=c++17", "-fsanitize=thread", *inc, "-c",
+                 os.path.join(ROOT, "tests", "cpp", "loopback_stress.cpp"), "-o", stress_o],
+                [hipcc, "--offload-arch=gfx950", "-fsanitize=thread", "-fno-gpu-sanitize", stress_o, *built, *objs,
+                 "-o", exe, "-lpthread"]):
+        out = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        assert out.returncode == 0, out.stderr[-3000:]
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0 and "ThreadSanitizer" not in out.stderr, (out.stdout + out.stderr)[-4000:]
+    assert "loopback_stress ok 1600" in out.stdout
