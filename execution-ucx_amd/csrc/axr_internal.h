@@ -6,6 +6,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <new>
 #include <string>
 #include <vector>
@@ -124,34 +125,35 @@ struct LaunchConfig {
 
 // ---------------------------------------------------------------- tunables
 
+// Read by planning threads while axr_tune_set may write: every knob is an atomic.
 struct Tunables {
   // Tile = tile_rows KiB moved by one wavefront.  0 picks the smallest of
   // 2, 4, 8, 16 that keeps the bundle within max_tiles tiles (and one tile per
   // run for bundles of short strided runs): small tiles and a grid of one tile
   // per wave measured fastest on MI355X (the hardware dispatcher balances the
   // load); larger tiles only bound the grid for multi-GiB bundles.
-  int64_t tile_rows = 0;
-  int64_t max_tiles = 1 << 20;
-  int64_t max_waves = 1 << 20;    // beyond this many tiles a wave takes several
-  int64_t threads = 0;            // workgroup size; 0 = 256 below 65,536 tiles (fewer dispatches
+  std::atomic<int64_t> tile_rows{0};
+  std::atomic<int64_t> max_tiles{1 << 20};
+  std::atomic<int64_t> max_waves{1 << 20};    // beyond this many tiles a wave takes several
+  std::atomic<int64_t> threads{0};            // workgroup size; 0 = 256 below 65,536 tiles (fewer dispatches
                                   // for short kernels), 128 above (finer balance at the tail)
   // Non-temporal hint: bit 0 tensor-side accesses, bit 1 payload-side accesses;
   // -1 = automatic: tensors always stream (read or written once), the payload
   // streams only when it is larger than payload_cache_bytes.  A smaller payload
   // is written with ordinary stores so that it is still in the 256 MB
   // last-level cache when the consumer (unpack, or the transport's copy) reads it.
-  int64_t nontemporal = -1;
-  int64_t payload_cache_bytes = 256ll << 20;
+  std::atomic<int64_t> nontemporal{-1};
+  std::atomic<int64_t> payload_cache_bytes{256ll << 20};
   // Strided runs shorter than this use element mode when they are multiples of
   // 16 bytes; other runs of 16 bytes or more up to five eighths of it (ragged
   // granules), anything else up to an eighth (measured crossovers).
-  int64_t gather_run_bytes = 2048;
-  int64_t xcd_remap = 0;          // contiguous wave ranges per die (measured slower)
-  int64_t transpose = 1;          // move transposed views as square blocks through LDS
-  int64_t ragged_runs = 1;        // short runs of 16+ bytes that are no multiple of 16 move in
+  std::atomic<int64_t> gather_run_bytes{2048};
+  std::atomic<int64_t> xcd_remap{0};          // contiguous wave ranges per die (measured slower)
+  std::atomic<int64_t> transpose{1};          // move transposed views as square blocks through LDS
+  std::atomic<int64_t> ragged_runs{1};        // short runs of 16+ bytes that are no multiple of 16 move in
                                   // 16-byte granules (the last one overlapping) instead of narrower ones
-  int64_t host_threads = 4;       // threads (the caller included) for host-side staging copies
-  int64_t inline_tables = 16384;  // bundles of up to this many tiles whose tables fit the kernel
+  std::atomic<int64_t> host_threads{4};       // threads (the caller included) for host-side staging copies
+  std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
 };
 Tunables& tunables();
