@@ -74,12 +74,17 @@ int device_compute_units(int* cus) {
 //
 // Plan tables are staged in pinned host memory and copied to a device block
 // with one async copy.  Both halves are recycled through a size-bucketed
-// free list so that steady-state planning performs no driver allocation.
+// free list so that steady-state planning performs no driver allocation.  The
+// list keeps at most kTableCacheBytes per half; what is released beyond that
+// goes back to the driver, so a burst of thousands of live plans does not pin
+// its peak forever.
 
 namespace {
+constexpr size_t kTableCacheBytes = 256u << 20;
 struct TableCache {
   std::mutex mu;
   std::multimap<std::pair<int, size_t>, TableBlock> free_blocks;
+  size_t cached_bytes = 0;
 };
 TableCache& table_cache() {
   static TableCache* c = new TableCache();   // leaked on purpose: outlives static dtors
@@ -104,6 +109,7 @@ int table_block_acquire(size_t bytes, TableBlock* block) {
     if (it != c.free_blocks.end()) {
       *block = it->second;
       c.free_blocks.erase(it);
+      c.cached_bytes -= want;
       return AXR_OK;
     }
   }
@@ -124,8 +130,18 @@ int table_block_acquire(size_t bytes, TableBlock* block) {
 void table_block_release(TableBlock* block) {
   if (!block->host) return;
   TableCache& c = table_cache();
-  std::lock_guard<std::mutex> lock(c.mu);
-  c.free_blocks.emplace(std::make_pair(block->device_id, block->bytes), *block);
+  {
+    std::lock_guard<std::mutex> lock(c.mu);
+    if (c.cached_bytes + block->bytes <= kTableCacheBytes) {
+      c.free_blocks.emplace(std::make_pair(block->device_id, block->bytes), *block);
+      c.cached_bytes += block->bytes;
+      *block = TableBlock();
+      return;
+    }
+  }
+  // callers release a block only when nothing on the device reads it any more
+  (void)hipHostFree(block->host);
+  (void)hipFree(block->device);
   *block = TableBlock();
 }
 

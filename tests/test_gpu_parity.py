@@ -892,6 +892,34 @@ def test_plan_reuse_rebind_and_streams(pkg, orc, gpu):
         pkg._capi.check(lib.axr_stream_destroy(s))
 
 
+def test_block_cache_gives_memory_back_after_a_burst(pkg, orc, gpu):
+    """Forty live plans with host tensors hold an 8 MiB pinned staging block each (320 MiB,
+    more than the 256 MiB the recycling list keeps); freeing them returns the excess to the
+    driver, and planning goes on as before."""
+    import torch
+    rng = np.random.default_rng(3)
+    host = [rng.integers(0, 256, size=70000, dtype=np.uint8) for _ in range(3)]
+    dev = rand_bytes_tensor(rng, 5000, gpu)
+    tensors = [host[0], dev, host[1], host[2]]
+    want = orc.pack([np.ascontiguousarray(t).reshape(-1) if isinstance(t, np.ndarray) else tbytes(t)
+                     for t in tensors], 256)
+    plans, payloads = [], []
+    for _ in range(40):
+        plan = pkg.BundlePlan.create(tensors, align=256)
+        buf = device_bytes(plan.payload_bytes, gpu)
+        plan.pack(buf.data_ptr(), plan.payload_bytes)
+        plans.append(plan)
+        payloads.append(buf)
+    torch.cuda.synchronize()
+    for plan, buf in zip(plans, payloads):
+        assert np.array_equal(buf.cpu().numpy()[:plan.payload_bytes], want)
+        plan.close()
+    for _ in range(3):                                       # blocks come from the list again
+        got, plan, _ = run_pack(pkg, tensors, 256, gpu)
+        assert np.array_equal(got, want)
+        plan.close()
+
+
 def test_plan_outlives_a_stream_it_ran_on(pkg, orc, gpu):
     """A plan drains the streams it ran on before its tables are rewritten or
     released.  A stream destroyed with axr_stream_destroy in the meantime must not
