@@ -131,6 +131,7 @@ struct axr_plan {
   size_t dims_at = 0, wave_at = 0;
   bool uploaded = false;
   bool resident = false;             // upload known to be complete (axr_plan_prepare)
+  size_t stage_bytes = 0;            // longest host chunk: size of the staging blocks
   std::unique_ptr<InlineTables> inline_tables;   // the tables as a kernel argument (small bundles)
   bool inline_ready = false;
   uint64_t launches = 0;             // kernel launches since the tables were built
@@ -585,6 +586,9 @@ int build_tables(axr_plan* p) {
     }
     p->host_chunks.push_back({i, 1, hc.offset, hc.offset + hc.bytes});
   }
+  p->stage_bytes = 0;
+  for (const HostChunk& c : p->host_chunks)
+    p->stage_bytes = std::max<size_t>(p->stage_bytes, static_cast<size_t>(c.end - c.begin));
   p->ntiles = static_cast<uint32_t>(b.tiles);
   Seg sentinel;
   std::memset(&sentinel, 0, sizeof(sentinel));
@@ -685,9 +689,14 @@ int stage_ready(HostStage* st) {   // block until the staging block's last devic
   return check_hip(hipEventSynchronize(st->ready), "hipEventSynchronize(staging)");
 }
 
-int stage_acquire(HostStage* st) {
+int stage_acquire(HostStage* st, size_t bytes) {
+  if (st->block.host && st->block.bytes < bytes) {   // a rebound plan with longer chunks
+    int rc = stage_ready(st);
+    if (rc) return rc;
+    table_block_release(&st->block);
+  }
   if (!st->block.host) {
-    int rc = table_block_acquire(kStageBytes, &st->block);
+    int rc = table_block_acquire(bytes, &st->block);
     if (rc) return rc;
   }
   if (!st->ready) {
@@ -723,10 +732,11 @@ int move_host_tensors(axr_plan* p, bool pack, uint8_t* payload, hipStream_t stre
       if (rc) return rc;
       pieces_out(p->host_chunks[k - 2], static_cast<const uint8_t*>(st->block.host));
     }
-    int rc = stage_acquire(st);
+    const size_t span = static_cast<size_t>(c.end - c.begin);
+    // a block as long as the plan's longest chunk (8 MiB at most), not 8 MiB for all
+    int rc = stage_acquire(st, p->stage_bytes);
     if (rc) return rc;
     uint8_t* staged = static_cast<uint8_t*>(st->block.host);
-    const size_t span = static_cast<size_t>(c.end - c.begin);
     if (pack) {
       uint64_t at = c.begin;
       jobs.clear();

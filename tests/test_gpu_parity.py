@@ -893,12 +893,12 @@ def test_plan_reuse_rebind_and_streams(pkg, orc, gpu):
 
 
 def test_block_cache_gives_memory_back_after_a_burst(pkg, orc, gpu):
-    """Forty live plans with host tensors hold an 8 MiB pinned staging block each (320 MiB,
-    more than the 256 MiB the recycling list keeps); freeing them returns the excess to the
-    driver, and planning goes on as before."""
+    """Forty live plans with 9 MiB of host tensors hold two pinned staging blocks each (4 and
+    8 MiB: 480 MiB, more than the 256 MiB the recycling list keeps); freeing them returns the
+    excess to the driver, and planning goes on as before."""
     import torch
     rng = np.random.default_rng(3)
-    host = [rng.integers(0, 256, size=70000, dtype=np.uint8) for _ in range(3)]
+    host = [rng.integers(0, 256, size=3 << 20, dtype=np.uint8) for _ in range(3)]
     dev = rand_bytes_tensor(rng, 5000, gpu)
     tensors = [host[0], dev, host[1], host[2]]
     want = orc.pack([np.ascontiguousarray(t).reshape(-1) if isinstance(t, np.ndarray) else tbytes(t)
