@@ -229,7 +229,7 @@ typedef struct axr_plan axr_plan_t;
  * they are packed as their C-order element sequence; the reference would
  * ship the first nbytes of storage instead (dlpack_helpers.cpp:776-780).
  * Every tensor must be device-accessible (kDLROCM / kDLROCMHost) or kDLCPU;
- * kDLCPU tensors travel through pinned staging blocks of 8 MiB: neighbouring
+ * kDLCPU tensors travel through pinned staging blocks of up to 8 MiB: neighbouring
  * pieces share one device copy per block; axr_pack returns once the host
  * tensors have been read, axr_unpack once they hold their data (the device
  * tensors of the same bundle still complete asynchronously on the stream).
