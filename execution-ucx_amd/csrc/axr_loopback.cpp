@@ -162,7 +162,8 @@ int axr_am_connect(axr_am_context_t* from, axr_am_context_t* to, uint64_t* conn_
   return guarded([&] { return am_connect_body(from, to, conn_id); });
 }
 
-static int am_send_body(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* d, void* stream, uint64_t* request) {
+static int am_send_body(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_data_t* d,
+                        void* stream, uint64_t* request) {
   if (!ctx || !d) return fail(AXR_ERR_INVALID, "axr_am_send: null argument");
   if (!d->header.data || d->header.size == 0)
     return fail(AXR_ERR_INVALID, "axr_am_send: the header must not be empty");
@@ -201,7 +202,8 @@ int axr_am_send(axr_am_context_t* ctx,
   return guarded([&] { return am_send_body(ctx, conn_id, d, stream, request); });
 }
 
-static int am_send_iov_body(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* d, void* stream, uint64_t* request) {
+static int am_send_iov_body(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* d,
+                            void* stream, uint64_t* request) {
   if (!ctx || !d) return fail(AXR_ERR_INVALID, "axr_am_send_iov: null argument");
   if (!d->header.data || d->header.size == 0)
     return fail(AXR_ERR_INVALID, "axr_am_send_iov: the header must not be empty");
@@ -327,7 +329,8 @@ static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_bu
   return rc;
 }
 
-static int am_recv_buffer_body(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst, size_t dst_bytes, void* stream) {
+static int am_recv_buffer_body(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
+                               size_t dst_bytes, void* stream) {
   if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null context");
   if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer: null buffer");
   axr_buffer_t one{dst, dst_bytes};
@@ -342,7 +345,8 @@ int axr_am_recv_buffer(axr_am_context_t* ctx,
   return guarded([&] { return am_recv_buffer_body(ctx, key, dst_type, dst, dst_bytes, stream); });
 }
 
-static int am_recv_buffer_async_body(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst, size_t dst_bytes, void* stream) {
+static int am_recv_buffer_async_body(axr_am_context_t* ctx, uint64_t key, int dst_type, void* dst,
+                                     size_t dst_bytes, void* stream) {
   if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_async: null context");
   if (!dst && dst_bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_async: null buffer");
   axr_buffer_t one{dst, dst_bytes};
@@ -354,10 +358,13 @@ int axr_am_recv_buffer_async(axr_am_context_t* ctx,
                              void* dst,
                              size_t dst_bytes,
                              void* stream) {
-  return guarded([&] { return am_recv_buffer_async_body(ctx, key, dst_type, dst, dst_bytes, stream); });
+  return guarded([&] { return am_recv_buffer_async_body(ctx, key, dst_type, dst, dst_bytes,
+                 stream); });
 }
 
-static int am_recv_buffer_iov_body(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_buffer_t* buffer_vec, size_t buffer_count, void* stream) {
+static int am_recv_buffer_iov_body(axr_am_context_t* ctx, uint64_t key, int dst_type,
+                                   const axr_buffer_t* buffer_vec, size_t buffer_count,
+                                   void* stream) {
   if (!ctx || !buffer_vec || buffer_count == 0)
     return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_iov: null or empty buffer vector");
   for (size_t i = 0; i < buffer_count; ++i) {
@@ -372,7 +379,8 @@ int axr_am_recv_buffer_iov(axr_am_context_t* ctx,
                            const axr_buffer_t* buffer_vec,
                            size_t buffer_count,
                            void* stream) {
-  return guarded([&] { return am_recv_buffer_iov_body(ctx, key, dst_type, buffer_vec, buffer_count, stream); });
+  return guarded([&] { return am_recv_buffer_iov_body(ctx, key, dst_type, buffer_vec, buffer_count,
+                 stream); });
 }
 
 static int am_message_release_body(axr_am_context_t* ctx, uint64_t key) {

@@ -832,9 +832,10 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   if ((capturing ? !p->resident : p->launches == 0 && !p->uploaded) &&
       tables_fit_kernel_arguments(p)) {
     // Small bundle, first launch: the tables ride in the kernel arguments.  The launch
-    // owns its copy, so a capturing stream may record it.  A plan that is launched again is being reused: from the second launch
-    // on it pays one upload and then the shorter argument list (a 3.5 KiB argument costs
-    // 0.4 us per launch, the upload 4 us on the host and 4 us on the device, once).
+    // owns its copy, so a capturing stream may record it.  A plan that is launched again
+    // is being reused: from the second launch on it pays one upload and then the shorter
+    // argument list (a 3.5 KiB argument costs 0.4 us per launch, the upload 4 us on the
+    // host and 4 us on the device, once).
     if (!p->inline_ready) fill_inline_tables(p);
     rc = launch_bundle_kernel_inline(pack, a, p->cfg, *p->inline_tables,
                                      static_cast<uint32_t>(p->dims_at),
@@ -904,7 +905,8 @@ int axr_tensor_nbytes(const axr_tensor_t* t, uint64_t* nbytes) {
   return guarded([&] { return tensor_nbytes_body(t, nbytes); });
 }
 
-static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t align, uint32_t flags, axr_plan_t** plan) {
+static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t align, uint32_t flags,
+                            axr_plan_t** plan) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_create: null result");
   *plan = nullptr;
   if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_create: null tensor array");
@@ -1137,7 +1139,8 @@ int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {
   return guarded([&] { return plan_bind_body(plan, tensors, n); });
 }
 
-static int plan_split_body(const axr_plan_t* plan, void* payload, size_t payload_bytes, axr_buffer_t* views) {
+static int plan_split_body(const axr_plan_t* plan, void* payload, size_t payload_bytes,
+                           axr_buffer_t* views) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_split: null plan");
   if (plan->payload_bytes > payload_bytes)
     return fail(AXR_ERR_LENGTH, "Total size of chunks exceeds buffer size");
@@ -1211,7 +1214,8 @@ int axr_plan_launch_info(axr_plan_t* plan, axr_launch_info_t* info) {
   return guarded([&] { return plan_launch_info_body(plan, info); });
 }
 
-static int plan_segments_body(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity, size_t* count) {
+static int plan_segments_body(axr_plan_t* plan, axr_segment_info_t* out, size_t capacity,
+                              size_t* count) {
   if (!plan || !count) return fail(AXR_ERR_INVALID, "axr_plan_segments: null argument");
   int rc = build_tables(plan);
   if (rc) return rc;

@@ -826,7 +826,8 @@ int axr_memcpy(int dst_type, void* dst, int src_type, const void* src, size_t by
   return guarded([&] { return memcpy_body(dst_type, dst, src_type, src, bytes); });
 }
 
-static int memcpy_async_body(int dst_type, void* dst, int src_type, const void* src, size_t bytes, void* stream) {
+static int memcpy_async_body(int dst_type, void* dst, int src_type, const void* src, size_t bytes,
+                             void* stream) {
   if (bytes == 0) return AXR_OK;
   if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_memcpy_async: null pointer");
   hipMemcpyKind kind;
@@ -910,7 +911,8 @@ int axr_pool_default(axr_pool_t** pool) {
   return guarded([&] { return pool_default_body(pool); });
 }
 
-static int pool_set_registrar_body(axr_pool_t* pool, axr_register_fn reg, axr_unregister_fn unreg, void* user) {
+static int pool_set_registrar_body(axr_pool_t* pool, axr_register_fn reg, axr_unregister_fn unreg,
+                                   void* user) {
   if (!pool) return fail(AXR_ERR_INVALID, "axr_pool_set_registrar: null pool");
   std::lock_guard<std::mutex> lock(pool->mu);
   if (!pool->slabs.empty())
@@ -927,7 +929,8 @@ int axr_pool_set_registrar(axr_pool_t* pool,
   return guarded([&] { return pool_set_registrar_body(pool, reg, unreg, user); });
 }
 
-static int pool_alloc_body(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr, void** mem_h) {
+static int pool_alloc_body(axr_pool_t* pool, size_t bytes, size_t alignment, void** ptr,
+                           void** mem_h) {
   if (!pool || !ptr) return fail(AXR_ERR_INVALID, "axr_pool_alloc: null argument");
   *ptr = nullptr;
   if (mem_h) *mem_h = nullptr;
