@@ -911,6 +911,7 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   *plan = nullptr;
   if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_create: null tensor array");
   if (n > 0xffffffffull) return fail(AXR_ERR_INVALID, "axr_plan_create: too many tensors");
+  if (flags != 0) return fail(AXR_ERR_INVALID, "axr_plan_create: flags are reserved and must be 0");
   int rc = check_align(align);
   if (rc) return rc;
   axr_plan* p = new (std::nothrow) axr_plan();

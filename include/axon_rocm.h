@@ -233,7 +233,8 @@ typedef struct axr_plan axr_plan_t;
  * pieces share one device copy per block; axr_pack returns once the host
  * tensors have been read, axr_unpack once they hold their data (the device
  * tensors of the same bundle still complete asynchronously on the stream).
- * The plan copies shapes and strides; `tensors` may be freed on return. */
+ * The plan copies shapes and strides; `tensors` may be freed on return.
+ * `flags` is reserved and must be 0 (AXR_ERR_INVALID otherwise). */
 AXR_API int axr_plan_create(const axr_tensor_t* tensors, size_t n, uint32_t align,
                             uint32_t flags, axr_plan_t** plan);
 /* Returns when the plan's launches have finished on the streams they were given

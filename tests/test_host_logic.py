@@ -80,6 +80,19 @@ def test_tunables(pkg):
         pkg.tune(no_such_knob=1)
 
 
+def test_plan_create_refuses_what_it_does_not_know(pkg):
+    lib = pkg._capi.load()
+    arr = pkg.dlpack.TensorArray([tv(pkg, 0x1000, [16])])
+    h = C.c_void_p()
+    assert lib.axr_plan_create(arr.pointer(), 1, 256, 1, C.byref(h)) == pkg._capi.AXR_ERR_INVALID   # reserved flags
+    assert not h.value
+    assert lib.axr_plan_create(arr.pointer(), 1, 3, 0, C.byref(h)) == pkg._capi.AXR_ERR_INVALID     # alignment
+    assert lib.axr_plan_create(None, 1, 256, 0, C.byref(h)) == pkg._capi.AXR_ERR_INVALID
+    assert lib.axr_plan_create(arr.pointer(), 1, 256, 0, None) == pkg._capi.AXR_ERR_INVALID
+    assert lib.axr_plan_create(None, 0, 256, 0, C.byref(h)) == 0 and h.value                     # an empty bundle
+    assert lib.axr_plan_free(h) == 0
+
+
 # ------------------------------------------------------------------ size rule and layout
 
 def test_nbytes_rule_matches_oracle(pkg, orc):
