@@ -17,7 +17,7 @@ from dataclasses import dataclass
 from typing import Any, Callable, List, Optional, Sequence, Tuple
 
 from . import _capi
-from .dlpack import DLPackExport, TensorArray, TensorView, extract_many
+from .dlpack import DLPackExport, TensorArray, TensorView
 from .memory import DevicePool, PoolBuffer
 
 

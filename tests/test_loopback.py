@@ -216,7 +216,6 @@ def test_device_iov_equals_packed_bundle(pkg, orc, gpu):
 def test_device_eager_and_process_reply(pkg, gpu):
     """Small device payload goes eager through host memory; the send -> process ->
     reply round trip of ucx_am_context_test.cpp:1893-1944 with the halving kernel."""
-    import ctypes as C
     import torch
     client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
     c2s, s2c = client.connect(server), server.connect(client)
