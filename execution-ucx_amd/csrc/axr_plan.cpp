@@ -73,7 +73,8 @@ T get(const uint8_t* p) {
   return x;
 }
 
-uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+// `a` is a power of two everywhere (check_align, table sections): no division per tensor
+uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) & ~(a - 1); }
 
 bool mul_overflow(uint64_t a, uint64_t b, uint64_t* out) {
   return __builtin_mul_overflow(a, b, out);
@@ -306,7 +307,8 @@ uint64_t element_mode_limit(uint64_t run_bytes) {
 
 struct Builder {
   axr_plan* p;
-  uint32_t tile_bytes;
+  uint32_t tile_bytes;    // rows * 1 KiB with rows a power of two
+  uint32_t tile_shift;    // log2(tile_bytes)
   uint64_t tiles = 0;
 
   int add_seg(uint32_t tensor, uint64_t ptr, uint64_t off, uint64_t run_bytes, uint64_t ntile,
@@ -330,7 +332,7 @@ struct Builder {
   int add_strided(uint32_t tensor, uint64_t ptr, uint64_t off, const uint64_t* ext,
                   const int64_t* str, size_t nd, uint64_t run_bytes) {
     if (nd == 0) {
-      return add_seg(tensor, ptr, off, run_bytes, (run_bytes + tile_bytes - 1) / tile_bytes, 0);
+      return add_seg(tensor, ptr, off, run_bytes, (run_bytes + tile_bytes - 1) >> tile_shift, 0);
     }
     uint64_t inner_runs = 1;
     for (size_t d = 1; d < nd; ++d) inner_runs *= ext[d];
@@ -533,7 +535,7 @@ int build_tables(axr_plan* p) {
                static_cast<uint64_t>(tn.max_tiles))
       rows *= 2;
   }
-  Builder b{p, rows * kRowBytes};
+  Builder b{p, rows * kRowBytes, static_cast<uint32_t>(__builtin_ctz(rows * kRowBytes))};
   p->segs.reserve(p->tensors.size() + 1);
   p->seg_tensor.reserve(p->tensors.size());
 
