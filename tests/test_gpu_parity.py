@@ -953,7 +953,7 @@ def test_small_bundles_with_tables_in_the_kernel_arguments(pkg, orc, gpu):
     bundles with that switched off use an uploaded table block.  Both must give the
     oracle's bytes: plain tensors with pads, strided rows, short strided runs,
     transposed views, and a mix with a host tensor.  A plan launched this way can be
-    freed at once and captured in a graph without axr_plan_prepare."""
+    captured in a graph without axr_plan_prepare, and freed once the capture has ended."""
     import torch
     rng = np.random.default_rng(55)
 
