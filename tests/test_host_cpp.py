@@ -100,3 +100,34 @@ def test_loopback_context_under_thread_sanitizer(tmp_path):
     out = subprocess.run([exe], capture_output=True, text=True, timeout=600)
     assert out.returncode == 0 and "ThreadSanitizer" not in out.stderr, (out.stdout + out.stderr)[-4000:]
     assert "loopback_stress ok 1600" in out.stdout
+
+
+def test_host_copy_helper_under_sanitizers(tmp_path):
+    """tests/cpp/host_copy_check.cpp: the threaded copy of the staging paths against plain
+    memcpy for random piece lists and 1 to 16 threads, with the runtime shim compiled with
+    AddressSanitizer and UBSan (host code only, no GPU)."""
+    pkgdir = os.path.join(ROOT, "execution-ucx_amd")
+    objs = [os.path.join(pkgdir, "build", n) for n in
+            ("axr_plan.cpp.o", "axr_loopback.cpp.o", "axr_kernels.hip.o")]
+    hipcc, clang = "/opt/rocm/bin/hipcc", "/opt/rocm/llvm/bin/clang++"
+    if not all(os.path.exists(p) for p in objs + [hipcc, clang]):
+        pytest.skip("needs the library's object files (make -C execution-ucx_amd) and the ROCm compilers")
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", os.path.join(pkgdir, "csrc")]
+    runtime_o, check_o, exe = (str(tmp_path / n) for n in ("axr_runtime.o", "host_copy_check.o", "host_copy_check"))
+    steps = [
+        [hipcc, "--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-fPIC",
+         "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", *inc,
+         "-x", "hip", "-c", os.path.join(pkgdir, "csrc", "axr_runtime.cpp"), "-o", runtime_o],
+        [clang, "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", *inc, "-c",
+         os.path.join(ROOT, "tests", "cpp", "host_copy_check.cpp"), "-o", check_o],
+        [hipcc, "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined", "-fno-gpu-sanitize",
+         check_o, runtime_o, *objs, "-o", exe, "-lpthread"],
+    ]
+    for cmd in steps:
+        out = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        assert out.returncode == 0, out.stderr[-3000:]
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, (out.stdout + out.stderr)[-3000:]
+    assert "host_copy_check ok" in out.stdout
