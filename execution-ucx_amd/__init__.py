@@ -8,7 +8,8 @@ nothing here computes on the CPU.
 from . import _capi
 from ._capi import (AxonRocmError, HeaderError, LengthError, MismatchError, NoDeviceError,
                     NoMessageError, NotImplementedForEager, UnsupportedMemoryError)
-from .bundle import BundlePlan, PackedBundle, TensorMeta, bundle_to_host, pack_bundle, unpack_bundle
+from .bundle import (BundlePlan, DLDataType, DLDevice, PackedBundle, TensorMeta, bundle_to_host, pack_bundle,
+                     unpack_bundle)
 from .device import (CpuDevice, Device, DeviceType, RocmDevice, auto_detect, cpu, device_count,
                      rocm)
 from .dlpack import DLPackExport, TensorView, extract, extract_many

@@ -14,25 +14,47 @@ from __future__ import annotations
 
 import ctypes as C
 from dataclasses import dataclass
-from typing import Any, Callable, List, Optional, Sequence, Tuple
+from typing import Any, Callable, List, NamedTuple, Optional, Sequence, Tuple
 
 from . import _capi
 from .dlpack import DLPackExport, TensorArray, TensorView
 from .memory import DevicePool, PoolBuffer
 
 
+class DLDevice(NamedTuple):
+    """``meta.device`` of the reference's Python TensorMeta: ``device_type`` (an int, so
+    that raw values survive) and ``device_id``
+    (axon/python/tests/test_types_enums.py:171-207).  Still a plain 2-tuple."""
+
+    device_type: int = 1
+    device_id: int = 0
+
+
+class DLDataType(NamedTuple):
+    """``meta.dtype``: ``code``, ``bits``, ``lanes``.  Still a plain 3-tuple."""
+
+    code: int = 2
+    bits: int = 32
+    lanes: int = 1
+
+
 @dataclass(frozen=True)
 class TensorMeta:
-    """Fields of the reference's TensorMeta (rpc_core/utils/tensor_meta.hpp:77-82)
-    as carried by the bundle header, plus the packed offset and size."""
+    """Fields of the reference's TensorMeta (rpc_core/utils/tensor_meta.hpp:77-82) under
+    the names its Python binding gives them (``device.device_type``, ``dtype.bits``,
+    ``shape``, ``strides`` ...), so that a memory policy written for the reference reads
+    them unchanged, plus the packed offset and size.  ``strides`` is always empty: packed
+    tensors are compact (the reference leaves it empty for compact tensors as well,
+    axon/python/src/dlpack_helpers.cpp:713-719).  Sequences are tuples, not lists."""
 
-    device: Tuple[int, int]
-    ndim: int
-    dtype: Tuple[int, int, int]
-    byte_offset: int
-    shape: Tuple[int, ...]
-    offset: int
-    nbytes: int
+    device: DLDevice = DLDevice()
+    ndim: int = 0
+    dtype: DLDataType = DLDataType()
+    byte_offset: int = 0
+    shape: Tuple[int, ...] = ()
+    strides: Tuple[int, ...] = ()
+    offset: int = 0
+    nbytes: int = 0
 
 
 def _stream_handle(stream) -> Optional[int]:
@@ -119,8 +141,8 @@ class BundlePlan:
         for i in range(len(offs)):
             _capi.check(self._lib.axr_plan_tensor_meta(self._h, i, C.byref(t)))
             out.append(TensorMeta(
-                device=(t.device_type, t.device_id), ndim=t.ndim,
-                dtype=(t.dtype_code, t.dtype_bits, t.dtype_lanes), byte_offset=0,
+                device=DLDevice(t.device_type, t.device_id), ndim=t.ndim,
+                dtype=DLDataType(t.dtype_code, t.dtype_bits, t.dtype_lanes), byte_offset=0,
                 shape=tuple(t.shape[d] for d in range(t.ndim)), offset=offs[i], nbytes=sizes[i]))
         return out
 

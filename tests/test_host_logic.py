@@ -80,6 +80,25 @@ def test_tunables(pkg):
         pkg.tune(no_such_knob=1)
 
 
+def test_tensor_meta_reads_like_the_reference_binding(pkg):
+    """axon/python/tests/test_types_enums.py:171-207: default-constructible, fields device
+    (device_type, device_id as ints), ndim, dtype (code, bits, lanes), byte_offset, shape,
+    strides -- what a memory policy written for the reference touches."""
+    meta = pkg.TensorMeta()
+    for field in ("device", "ndim", "dtype", "byte_offset", "shape", "strides"):
+        assert hasattr(meta, field)
+    assert meta.ndim == 0 and meta.byte_offset == 0
+    assert isinstance(meta.device, pkg.DLDevice) and isinstance(meta.dtype, pkg.DLDataType)
+    assert isinstance(meta.device.device_type, int) and isinstance(meta.device.device_id, int)
+    assert all(hasattr(meta.dtype, f) for f in ("code", "bits", "lanes"))
+    plan = pkg.BundlePlan.create([tv(pkg, 0x1000, [3, 5], dtype=(4, 16, 1))], align=64)
+    m = plan.metas()[0]
+    assert (m.device.device_type, m.device.device_id, m.ndim) == (10, 0, 2)
+    assert (m.dtype.code, m.dtype.bits, m.dtype.lanes) == (4, 16, 1) and m.dtype == (4, 16, 1)
+    assert tuple(m.shape) == (3, 5) and list(m.strides) == [] and m.byte_offset == 0
+    assert np.zeros(tuple(m.shape)).shape == (3, 5)          # the way policies use it
+
+
 def test_plan_create_refuses_what_it_does_not_know(pkg):
     lib = pkg._capi.load()
     arr = pkg.dlpack.TensorArray([tv(pkg, 0x1000, [16])])
