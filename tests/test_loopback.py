@@ -417,3 +417,43 @@ def test_send_and_receive_nested_arguments(pkg, gpu):
     assert len(got) == 1 and len(got[0]) == 2 and torch.equal(got[0][1], t[1])
     client.close()
     server.close()
+
+
+@pytest.mark.gpu
+def test_memory_policy_with_tracked_numpy_arrays(pkg, gpu):
+    """The reference's memory-policy test (axon/python/tests/test_server_memory_policy.py:
+    9-66, test_invoke_memory_policy.py:9-40): the policy gets a list of metas, allocates an
+    ndarray subclass per meta from `tuple(meta.shape)`, returns the object itself for one
+    meta and a list otherwise; the handler must see those very objects, filled."""
+    import torch
+
+    class TrackedArray(np.ndarray):
+        pass
+    created = {}
+
+    def custom_policy(meta_list):
+        assert isinstance(meta_list, list) and len(meta_list) > 0
+        results = []
+        for meta in meta_list:
+            assert meta.dtype.bits == 32 and meta.dtype.code == 2 and meta.device.device_type == 10
+            arr = np.zeros(tuple(meta.shape), dtype=np.float32).view(TrackedArray)
+            created[id(arr)] = True
+            results.append(arr)
+        return results[0] if len(results) == 1 else results
+
+    client, server = pkg.LoopbackAmContext("client"), pkg.LoopbackAmContext("server")
+    conn = client.connect(server)
+    for tensors in ([torch.ones(1024, 1024, device=gpu)],                      # 4 MiB: rendezvous
+                    [torch.ones(300, device=gpu), torch.full((7, 9), 1.0, device=gpu)]):
+        created.clear()
+        req, bundle = pkg.send_tensors(client, conn, tensors)
+        got = pkg.recv_tensors(server, memory_policy=custom_policy)
+        assert client.test(req)
+        assert len(got) == len(tensors)
+        for arr, t in zip(got, tensors):
+            assert isinstance(arr, TrackedArray) and id(arr) in created
+            assert arr.shape == tuple(t.shape) and np.allclose(arr, 1.0)
+        bundle.plan.close()
+        bundle.payload.release()
+    client.close()
+    server.close()
