@@ -258,9 +258,13 @@ def unpack_bundle(header: bytes, payload: Any, payload_bytes: Optional[int] = No
     pieces = plan.split(ptr, size)
     metas = plan.metas()
     owner = payload  # every view keeps the payload block alive
+    # the views live where the payload does: on the receiver's current device, whatever
+    # ordinal the sender's tensors had (the reference writes 0, dlpack_helpers.cpp:82-114)
+    device = C.c_int(0)
+    _capi.check(_capi.load().axr_device_get(C.byref(device)))
     results = []
     for (p, n), m in zip(pieces, metas):
-        exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLROCM, m.device[1],
+        exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLROCM, device.value,
                            release=(lambda keep=owner: None))
         results.append(from_dlpack_fn(exp) if from_dlpack_fn else exp)
     plan.close()
