@@ -304,16 +304,29 @@ class DLPackExport:
         self._device = (device_type, device_id)
         self._release = release
         self._consumed = False
+        self._exported = False     # a capsule went out: its deleter releases the memory
 
     def __dlpack_device__(self):
         return self._device
 
     def __dlpack__(self, stream=None, max_version=None, dl_device=None, copy=None):
+        # checks, their order and the exception types follow the reference's wrapper
+        # (axon/python/src/dlpack_helpers.hpp:106-155): consumed first (and for good,
+        # even when a later check raises), then the stream rule for host memory, then
+        # the target device, then copy
         if self._consumed:
-            raise RuntimeError("DLPack capsule can only be consumed once")
-        if copy:
-            raise BufferError("this producer cannot copy")
+            raise RuntimeError("DLPack capsule has already been consumed. "
+                               "__dlpack__() can only be called once per capsule.")
         self._consumed = True
+        if self._device[0] == _capi.kDLCPU and stream is not None:
+            raise ValueError("stream must be None for CPU device (kDLCPU)")
+        if dl_device is not None and int(dl_device[0]) != self._device[0]:
+            if copy is not None and not copy:
+                raise RuntimeError("Cross-device export requires copy=True or copy=None, "
+                                   "but copy=False was specified")
+            raise RuntimeError("Cross-device DLPack export is not yet supported")
+        if copy:
+            raise RuntimeError("copy=True is not supported; this implementation is zero-copy only")
         nd = len(self._shape)
         shape = (C.c_int64 * max(nd, 1))(*self._shape)
         managed = _ManagedTensor()
@@ -330,10 +343,11 @@ class DLPackExport:
         managed.manager_ctx = key
         managed.deleter = _managed_deleter
         _live_exports[key] = (managed, shape, self, self._release)
+        self._exported = True
         return _py.PyCapsule_New(C.addressof(managed), _NAME, _capsule_destructor)
 
     def __del__(self):
-        if not self._consumed and self._release is not None:
+        if not self._exported and self._release is not None:
             release, self._release = self._release, None
             release()
 

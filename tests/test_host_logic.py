@@ -454,6 +454,30 @@ def test_dlpack_export_single_consume(pkg):
     del exp2
     gc.collect()
     assert released == [1, 2]
+    # argument checks of the reference's wrapper (axon/python/src/dlpack_helpers.hpp:106-155):
+    # each refusal still consumes the capsule, and the memory is released with the wrapper
+    def fresh(tag, device_type=1):
+        return pkg.DLPackExport(src.ctypes.data, 160, (1, 8, 1), device_type, 0,
+                                release=lambda: released.append(tag))
+    for tag, kwargs, device_type, error, text in (
+            (3, {"stream": 0}, 1, ValueError, "stream must be None for CPU"),
+            (4, {"dl_device": (10, 0)}, 1, RuntimeError, "not yet supported"),
+            (5, {"dl_device": (10, 0), "copy": False}, 1, RuntimeError, "copy=False was specified"),
+            (6, {"copy": True}, 1, RuntimeError, "zero-copy only"),
+            (7, {"copy": True, "stream": 0}, 10, RuntimeError, "zero-copy only")):
+        exp = fresh(tag, device_type)
+        with pytest.raises(error, match=text):
+            exp.__dlpack__(**kwargs)
+        with pytest.raises(RuntimeError, match="already been consumed"):
+            exp.__dlpack__()
+        del exp
+        gc.collect()
+        assert released[-1] == tag
+    ok = fresh(8)
+    capsule = ok.__dlpack__(stream=None, max_version=(1, 0), dl_device=(1, 0), copy=False)   # all accepted
+    del capsule, ok
+    gc.collect()
+    assert released[-1] == 8
 
 
 def test_device_objects(pkg):
