@@ -122,6 +122,12 @@ def _read(dl: _capi.Tensor, owner: Any) -> TensorView:
     )
 
 
+class NotDLPackError(TypeError, RuntimeError):
+    """An object that is no DLPack producer.  The reference raises RuntimeError here
+    (axon/python/src/dlpack_helpers.cpp:153-155); TypeError is what Python code expects:
+    this is both."""
+
+
 def extract(obj: Any) -> TensorView:
     """Describe ``obj`` (anything with ``__dlpack__``, or a capsule)."""
     if isinstance(obj, TensorView):
@@ -138,9 +144,9 @@ def extract(obj: Any) -> TensorView:
         ptr = _py.PyCapsule_GetPointer(capsule, _NAME_VERSIONED)
         managed = C.cast(ptr, C.POINTER(_ManagedTensorVersioned)).contents
         return _read(managed.dl_tensor, (capsule, obj))
-    raise TypeError(
-        "object does not provide a DLPack capsule named 'dltensor' "
-        f"(got {type(obj).__name__})"
+    raise NotDLPackError(
+        f"Invalid dlpack object {obj!r} when extracting: missing __dlpack__ method "
+        "or a capsule not named 'dltensor'"
     )
 
 
