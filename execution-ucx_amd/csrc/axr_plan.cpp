@@ -148,16 +148,22 @@ struct axr_plan {
 
 namespace {
 
-void compute_layout(axr_plan* p) {
-  uint64_t off = 0, data = 0;
+// False when an offset or the payload size does not fit 64 bits (a crafted header,
+// or a tensor list whose sizes add up past 2^64): nothing is laid out then.
+bool compute_layout(axr_plan* p) {
+  uint64_t off = 0, data = 0, end = 0;
+  const uint64_t mask = static_cast<uint64_t>(p->align) - 1;
   for (auto& t : p->tensors) {
-    off = align_up(off, p->align);
+    if (__builtin_add_overflow(off, mask, &off)) return false;
+    off &= ~mask;
     t.offset = off;
-    off += t.nbytes;
-    data += t.nbytes;
+    if (__builtin_add_overflow(off, t.nbytes, &off)) return false;
+    end = off;
+    data += t.nbytes;   // at most `off`, which did not overflow
   }
-  p->payload_bytes = p->tensors.empty() ? 0 : p->tensors.back().offset + p->tensors.back().nbytes;
+  p->payload_bytes = end;
   p->data_bytes = data;
+  return true;
 }
 
 void encode_header(axr_plan* p) {
@@ -931,7 +937,10 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
       return rc;
     }
   }
-  compute_layout(p);
+  if (!compute_layout(p)) {
+    delete p;
+    return fail(AXR_ERR_INVALID, "axr_plan_create: bundle size overflows 64 bits");
+  }
   encode_header(p);
   p->bound = true;
   *plan = p;
@@ -1090,8 +1099,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   }
   std::vector<uint64_t> sent(n);
   for (uint32_t i = 0; i < n; ++i) sent[i] = p->tensors[i].offset;
-  compute_layout(p);
-  bool ok = p->payload_bytes == payload;
+  bool ok = compute_layout(p) && p->payload_bytes == payload;
   for (uint32_t i = 0; i < n && ok; ++i) ok = sent[i] == p->tensors[i].offset;
   if (!ok) {
     delete p;

@@ -176,6 +176,38 @@ int main(int argc, char** argv) {
     }
     axr_plan_free(plan);
   }
+  {   // sizes that wrap 64 bits: refused at creation and in a crafted header
+    int64_t huge = int64_t(1) << 62;
+    axr_tensor_t t[2];
+    std::memset(t, 0, sizeof(t));
+    for (axr_tensor_t& x : t) {
+      x.data = reinterpret_cast<void*>(0x1000);
+      x.device_type = 10;
+      x.ndim = 1;
+      x.dtype_code = 1;
+      x.dtype_bits = 16;
+      x.dtype_lanes = 1;
+      x.shape = &huge;
+    }
+    axr_plan_t* p = nullptr;
+    if (axr_plan_create(t, 2, 1, 0, &p) != AXR_ERR_INVALID || p) die("wrapping sizes accepted", -1);
+    uint8_t h[24 + 2 * 48];
+    const uint32_t magic = 0x42545841u, n = 2, align = 1;
+    const uint16_t version = 1, flags = 0;
+    const uint64_t payload = 0, nbytes = uint64_t(1) << 63, zero = 0;
+    uint8_t* w = h;
+    auto emit = [&w](const void* src, size_t len) { std::memcpy(w, src, len); w += len; };
+    emit(&magic, 4); emit(&version, 2); emit(&flags, 2); emit(&n, 4); emit(&align, 4); emit(&payload, 8);
+    for (int i = 0; i < 2; ++i) {
+      const uint64_t off = i ? nbytes : 0;
+      const int32_t dev = 10, id = 0, ndim = 1;
+      const uint8_t code = 1, bits = 16;
+      const uint16_t lanes = 1;
+      emit(&off, 8); emit(&nbytes, 8); emit(&dev, 4); emit(&id, 4); emit(&ndim, 4);
+      emit(&code, 1); emit(&bits, 1); emit(&lanes, 2); emit(&zero, 8); emit(&huge, 8);
+    }
+    if (axr_plan_from_header(h, sizeof(h), &p) != AXR_ERR_HEADER || p) die("wrapping header accepted", -1);
+  }
   std::printf("plan_fuzz ok: %ld plans, %ld with tables, %ld mutated headers decoded, %ld of them valid\n",
               plans, tables, decodes, accepted);
   return 0;

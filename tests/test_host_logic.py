@@ -643,3 +643,28 @@ def test_empty_and_extreme_bundles(pkg, orc):
     # a null data pointer is only acceptable for an empty tensor
     with pytest.raises(pkg.AxonRocmError):
         pkg.BundlePlan.create([tv(pkg, 0, [8])], align=1)
+    # sizes that each fit 64 bits but add up past 2^64 are refused as well
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.create([tv(pkg, 0x1000, [2 ** 62], dtype=(1, 16, 1))] * 2, align=1)
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.create([tv(pkg, 0x1000, [2 ** 63 - 4], dtype=(1, 16, 1)), tv(pkg, 0x1000, [1])],
+                              align=16)
+
+
+def test_header_whose_sizes_wrap_64_bits_is_refused(pkg):
+    """Two tensors of 2^63 bytes each: offset 0 and 2^63, payload 2^64 = 0 after
+    wrapping.  Such a header must not decode into views that lie outside the payload."""
+    import struct
+    n, align, payload = 2, 1, 0
+    h = struct.pack("<IHHIIQ", 0x42545841, 1, 0, n, align, payload)
+    for off in (0, 2 ** 63):
+        h += struct.pack("<QQiiiBBHQq", off, 2 ** 63, 10, 0, 1, 1, 16, 1, 0, 2 ** 62)
+    with pytest.raises(pkg.AxonRocmError) as e:
+        pkg.BundlePlan.from_header(h)
+    assert e.value.status == pkg._capi.AXR_ERR_HEADER
+    # the align-up step can wrap too: offset 2^64 - 8 rounded up to 16
+    h = struct.pack("<IHHIIQ", 0x42545841, 1, 0, 2, 16, 1)
+    h += struct.pack("<QQiiiBBHQq", 0, 2 ** 64 - 8, 10, 0, 1, 1, 16, 1, 0, 2 ** 63 - 4)
+    h += struct.pack("<QQiiiBBHQq", 0, 1, 10, 0, 1, 1, 8, 1, 0, 1)
+    with pytest.raises(pkg.AxonRocmError):
+        pkg.BundlePlan.from_header(h)
