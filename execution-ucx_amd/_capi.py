@@ -241,6 +241,7 @@ PROTOTYPES = {
     "axr_pack": (C.c_int, [_vp, _vp, _sz, _vp]),
     "axr_unpack": (C.c_int, [_vp, _vp, _sz, _vp]),
     "axr_plan_prepare": (C.c_int, [_vp, _vp]),
+    "axr_pack_noalloc": (C.c_int, [_vp, _vp, _sz, _vp]),
     "axr_plan_launch_info": (C.c_int, [_vp, C.POINTER(LaunchInfo)]),
     "axr_plan_segments": (C.c_int, [_vp, C.POINTER(SegmentInfo), _sz, C.POINTER(_sz)]),
     "axr_tune_set": (C.c_int, [C.c_char_p, C.c_int64]),

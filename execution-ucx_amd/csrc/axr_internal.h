@@ -200,6 +200,11 @@ int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchC
                                 const InlineTables& tables, uint32_t dims_at, uint32_t wave_at,
                                 void* stream);
 int launch_fill(void* dst, int value, size_t bytes, void* stream);
+// Device address, on the current device, of the kStaticTableBytes bytes that hold the
+// tables of axr_pack_noalloc (a __device__ array of the code object: never allocated,
+// shared by every call on that device).
+constexpr size_t kStaticTableBytes = 1u << 20;
+int static_table_area(void** ptr);
 
 // ---------------------------------------------------------------- runtime (axr_runtime.cpp)
 

@@ -1058,6 +1058,41 @@ int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchC
   return check_hip(hipGetLastError(), "bundle kernel launch (inline tables)");
 }
 
+// ---------------------------------------------------------------- static table area
+//
+// Device memory for the tables of axr_pack_noalloc: part of the code object, so no
+// call ever allocates it.  Every device the library runs on holds its own copy at its
+// own address until the process ends.  `scratch` below is only the host-side handle of
+// the symbol; the device address comes from hipGetSymbolAddress, once per device, and
+// that address is what copies and kernel arguments use.
+static __device__ __align__(256) uint8_t scratch[kStaticTableBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<uint8_t*> g_scratch_address[kMaxDevices];
+}  // namespace
+
+int static_table_area(void** ptr) {
+  int device = -1;
+  int rc = check_hip(hipGetDevice(&device), "hipGetDevice");
+  if (rc) return rc;
+  if (device < 0 || device >= kMaxDevices)
+    return fail(AXR_ERR_UNSUPPORTED, "device ordinal beyond the static table area's registry");
+  uint8_t* address = g_scratch_address[device].load(std::memory_order_acquire);
+  if (!address) {
+    // the current device is `device`: the lookup answers for that device's copy.  Two
+    // threads racing here obtain the same address.
+    void* found = nullptr;
+    rc = check_hip(hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(static table area)");
+    if (rc) return rc;
+    if (!found) return fail(AXR_ERR_HIP, "hipGetSymbolAddress returned no address");
+    address = static_cast<uint8_t*>(found);
+    g_scratch_address[device].store(address, std::memory_order_release);
+  }
+  *ptr = address;
+  return AXR_OK;
+}
+
 int launch_fill(void* dst, int value, size_t bytes, void* stream) {
   if (bytes == 0) return AXR_OK;
   hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(bytes / 16 + 1, 1u << 16)), dim3(256), 0,

@@ -1184,6 +1184,90 @@ int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes, void
   return guarded([&] { return unpack_body(plan, payload, payload_bytes, stream); });
 }
 
+// axr_pack for callers that must not allocate device memory.  The tables ride in the
+// kernel arguments when they fit; otherwise they are copied, on `stream`, into the static
+// table area of the current device and the same kernel as axr_pack reads them there.
+static int pack_noalloc_body(axr_plan_t* p, void* payload, size_t payload_bytes, void* stream_) {
+  if (!p) return fail(AXR_ERR_INVALID, "null plan");
+  if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
+  if (payload_bytes < p->payload_bytes)
+    return fail(AXR_ERR_LENGTH, "payload buffer is smaller than the plan's payload");
+  if (p->payload_bytes == 0) return AXR_OK;
+  if (!payload) return fail(AXR_ERR_INVALID, "null payload");
+  int rc = build_tables(p);   // host memory only
+  if (rc) return rc;
+  if (!p->host_chunks.empty())
+    return fail(AXR_ERR_UNSUPPORTED,
+                "axr_pack_noalloc: host (kDLCPU) tensors need pinned staging blocks; use axr_pack");
+  if (p->ntiles == 0) return AXR_OK;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  bool capturing = false;
+  if (stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    rc = check_hip(hipStreamIsCapturing(stream, &status), "hipStreamIsCapturing");
+    if (rc) return rc;
+    capturing = status == hipStreamCaptureStatusActive;
+  }
+  KernelArgs a;
+  a.payload = static_cast<uint8_t*>(payload);
+  a.nseg = static_cast<uint32_t>(p->segs.size() - 1);
+  a.ntiles = p->ntiles;
+  a.tiles_per_wave = p->cfg.tiles_per_wave;
+  a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
+  a.seg_shift = p->cfg.seg_shift;
+  auto remember = [&] {
+    if (!capturing &&
+        std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+      p->busy_streams.push_back(stream);
+  };
+  if (tables_fit_kernel_arguments(p)) {
+    if (!p->inline_ready) fill_inline_tables(p);
+    rc = launch_bundle_kernel_inline(true, a, p->cfg, *p->inline_tables,
+                                     static_cast<uint32_t>(p->dims_at),
+                                     static_cast<uint32_t>(p->wave_at), stream);
+    if (rc) return rc;
+    ++p->launches;
+    remember();
+    return AXR_OK;
+  }
+  if (p->table_bytes > kStaticTableBytes)
+    return fail(AXR_ERR_LENGTH, "axr_pack_noalloc: the bundle's tables need " +
+                                    std::to_string(p->table_bytes) + " bytes, the static table area holds " +
+                                    std::to_string(kStaticTableBytes) + "; use axr_pack");
+  if (capturing)
+    return fail(AXR_ERR_UNSUPPORTED,
+                "axr_pack_noalloc: tables beyond the kernel arguments cannot be recorded into a graph");
+  void* area = nullptr;
+  rc = static_table_area(&area);
+  if (rc) return rc;
+  uint8_t* d = static_cast<uint8_t*>(area);
+  // Three copies out of the plan's own (pageable) vectors, ordered on `stream` behind
+  // whatever that stream's previous call still reads from the area.  The vectors live
+  // until the plan is rebound or freed, and both drain the stream first.
+  remember();
+  rc = check_hip(hipMemcpyAsync(d, p->segs.data(), p->segs.size() * sizeof(Seg), hipMemcpyHostToDevice, stream),
+                 "hipMemcpyAsync(segment table -> static area)");
+  if (!rc && !p->dims.empty())
+    rc = check_hip(hipMemcpyAsync(d + p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims),
+                                  hipMemcpyHostToDevice, stream),
+                   "hipMemcpyAsync(dims table -> static area)");
+  if (!rc)
+    rc = check_hip(hipMemcpyAsync(d + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t),
+                                  hipMemcpyHostToDevice, stream),
+                   "hipMemcpyAsync(tile index -> static area)");
+  if (rc) return rc;
+  a.segs = reinterpret_cast<const Seg*>(d);
+  a.dims = reinterpret_cast<const Dims*>(d + p->dims_at);
+  a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
+  rc = launch_bundle_kernel(true, a, p->cfg, stream);
+  if (rc) return rc;
+  ++p->launches;
+  return AXR_OK;
+}
+int axr_pack_noalloc(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream) {
+  return guarded([&] { return pack_noalloc_body(plan, payload, payload_bytes, stream); });
+}
+
 static int plan_launch_info_body(axr_plan_t* plan, axr_launch_info_t* info) {
   if (!plan || !info) return fail(AXR_ERR_INVALID, "axr_plan_launch_info: null argument");
   int rc = build_tables(plan);

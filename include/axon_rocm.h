@@ -300,6 +300,22 @@ AXR_API int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_byt
  * passes through a kernel. */
 AXR_API int axr_plan_prepare(axr_plan_t* plan, void* stream);
 
+/* axr_pack for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference (its payload never passes through a kernel).  Same result as
+ * axr_pack; the call allocates no device or pinned memory and frees none.  A small
+ * bundle carries its tables inside the kernel arguments (as axr_pack's first launch
+ * does); a larger one has them copied on `stream` into a table area that is part of
+ * the library's device code: 1 MiB per GPU, held until the process ends (about
+ * 25,000 contiguous tensors; AXR_ERR_LENGTH beyond that).  Every call on one GPU
+ * shares that GPU's area: calls on ONE stream are ordered and may follow each other
+ * without a wait; calls that overlap on two streams of one GPU race for it and must
+ * be ordered by the caller.  Bundles with kDLCPU tensors (pinned staging) and,
+ * under stream capture, bundles whose tables exceed the kernel arguments are
+ * refused with AXR_ERR_UNSUPPORTED.  The plan must stay alive until the stream has
+ * run the call (axr_plan_free and axr_plan_bind wait for it). */
+AXR_API int axr_pack_noalloc(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream);
+
 /* Launch geometry of a plan's kernel, for profiling reports. */
 typedef struct axr_launch_info {
   uint32_t workgroups;
