@@ -154,9 +154,18 @@ class SegmentInfo(C.Structure):
         ("ndim", C.c_uint32),
         ("granule", C.c_uint32),
         ("tiles", C.c_uint32),
+        ("head", C.c_uint32),
+        ("reserved", C.c_uint32),
         ("shape", C.c_uint32 * 6),
         ("stride_bytes", C.c_int64 * 6),
     ]
+
+
+class Job(C.Structure):
+    """axr_job_t: one gather or scatter of axr_submit."""
+
+    _fields_ = [("plan", C.c_void_p), ("unpack", C.c_int), ("payload", C.c_void_p),
+                ("payload_bytes", C.c_size_t), ("tensor_delta", C.c_int64)]
 
 
 class AmData(C.Structure):
@@ -242,6 +251,7 @@ PROTOTYPES = {
     "axr_unpack": (C.c_int, [_vp, _vp, _sz, _vp]),
     "axr_plan_prepare": (C.c_int, [_vp, _vp]),
     "axr_pack_noalloc": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "axr_submit": (C.c_int, [C.POINTER(Job), _sz, _vp]),
     "axr_plan_launch_info": (C.c_int, [_vp, C.POINTER(LaunchInfo)]),
     "axr_plan_segments": (C.c_int, [_vp, C.POINTER(SegmentInfo), _sz, C.POINTER(_sz)]),
     "axr_tune_set": (C.c_int, [C.c_char_p, C.c_int64]),

@@ -36,6 +36,12 @@ constexpr uint32_t kSegPadMask = 0xfffu;         // meta bits 0..11: zero bytes 
 constexpr uint32_t kSegDimsShift = 12;           // meta bits 12..31: 1 + dims index
 constexpr uint32_t kSegFillOnly = 0xfffffu;      // dims field value: segment only writes zeros
 constexpr uint32_t kMaxAlign = 4096;
+// run_bytes of a contiguous (not strided) segment carries, in its top byte, the number
+// of leading bytes (< 128) that tile 0 moves in addition to its own range: with them
+// peeled off, every tile of the segment starts on a 128-byte line of the written side.
+constexpr uint32_t kSegHeadShift = 56;
+constexpr uint64_t kSegRunMask = (1ull << kSegHeadShift) - 1;
+constexpr uint32_t kLineBytes = 128;
 
 struct Seg {              // 32 bytes
   uint64_t ptr;           // tensor-side address of the first element
@@ -99,6 +105,22 @@ struct KernelArgs {
   uint32_t tiles_per_wave;
   uint32_t xcd_remap;         // 0 or the number of workgroups per die
   uint32_t seg_shift;         // log2 of the tile-block size of wave_seg
+  int64_t tensor_delta = 0;   // added to every tensor-side address of the tables
+};
+
+// One launch serving several bundles: job k owns the workgroups [wg_begin[k], wg_begin[k+1]).
+constexpr uint32_t kMaxJobs = 4;
+struct JobDesc {              // 64 bytes
+  uint64_t segs, dims, wave_seg, payload;   // device addresses
+  int64_t tensor_delta;
+  uint32_t ntiles, tiles_per_wave, seg_shift, wg_begin;
+  uint32_t unpack;            // 0: tensors -> payload, 1: payload -> tensors
+  uint32_t reserved;
+};
+static_assert(sizeof(JobDesc) == 64, "JobDesc layout");
+struct alignas(16) JobTable {
+  uint32_t count, lds_per_wave, nt_bits, reserved;
+  JobDesc job[kMaxJobs];
 };
 
 // Tables of a small bundle handed to the kernel by value.  bytes[0..16) is a head
@@ -152,6 +174,11 @@ struct Tunables {
   std::atomic<int64_t> transpose{1};          // move transposed views as square blocks through LDS
   std::atomic<int64_t> ragged_runs{1};        // short runs of 16+ bytes that are no multiple of 16 move in
                                   // 16-byte granules (the last one overlapping) instead of narrower ones
+  // Contiguous segments longer than a tile start their tiles on a multiple of this many
+  // bytes of the written side (0: tiles start at the segment's first byte).  Measured on the
+  // 4096-tensor bundle: 16 lifts the tight layout by 2 % (every 16-byte store aligned) and
+  // costs the 256-byte aligned layout nothing; 64 and 128 are no better for either.
+  std::atomic<int64_t> head_align{16};
   std::atomic<int64_t> host_threads{4};       // threads (the caller included) for host-side staging copies
   std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
@@ -199,6 +226,9 @@ int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& 
 int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchConfig& cfg,
                                 const InlineTables& tables, uint32_t dims_at, uint32_t wave_at,
                                 void* stream);
+// One launch for up to kMaxJobs bundles that share `cfg` (tile size, workgroup size, cache
+// hints; cfg.workgroups is the whole grid, cfg.lds_per_wave the largest need of any job).
+int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stream);
 int launch_fill(void* dst, int value, size_t bytes, void* stream);
 // Device address, on the current device, of the kStaticTableBytes bytes that hold the
 // tables of axr_pack_noalloc (a __device__ array of the code object: never allocated,

@@ -696,16 +696,17 @@ __device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_
 }
 
 // The whole pack or unpack of a bundle: every wavefront finds the segment of its
-// first tile through the tile-block index and walks forward from there.
+// first tile through the tile-block index and walks forward from there.  `wg` is the
+// workgroup's index within this bundle's share of the grid; `a.tensor_delta` is added to
+// every tensor-side address (one plan serves tensors of the same geometry elsewhere).
 template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
                                             const AXR_CONST uint32_t* wave_seg, gbytes payload,
-                                            const KernelArgs& a, uint32_t lds_per_wave,
+                                            const KernelArgs& a, uint32_t wg, uint32_t lds_per_wave,
                                             uint32_t nt_bits) {
   constexpr uint32_t kTile = ROWS * kRowBytes;
   const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
   const uint32_t lane_off = lane * kVecBytes;
-  uint32_t wg = blockIdx.x;
   if (a.xcd_remap) {
     // consecutive workgroup ids land on consecutive dies; hand die d the d-th
     // contiguous share of the index space so neighbouring tiles share an L2
@@ -716,18 +717,19 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
   if (t >= a.ntiles) return;
   const uint32_t t_end =
       (a.ntiles - t > a.tiles_per_wave) ? t + a.tiles_per_wave : a.ntiles;
+  const uint64_t delta = static_cast<uint64_t>(a.tensor_delta);
   // The index has one entry per block of 2^seg_shift tiles (the planner sizes
   // blocks so that they rarely hold more than one segment); the loop below
   // walks forward from there to the segment of this wave's first tile.
   uint32_t s = wave_seg[t >> a.seg_shift];
-  uint64_t seg_ptr = segs[s].ptr, seg_off = segs[s].off, seg_run = segs[s].run_bytes;
+  uint64_t seg_ptr = segs[s].ptr + delta, seg_off = segs[s].off, seg_run = segs[s].run_bytes;
   uint32_t seg_begin = segs[s].tile_begin, seg_meta = segs[s].meta;
   uint32_t seg_end = segs[s + 1].tile_begin;
 
   while (t < t_end) {
     if (t >= seg_end) {   // wave-uniform: step to the next segment
       ++s;
-      seg_ptr = segs[s].ptr;
+      seg_ptr = segs[s].ptr + delta;
       seg_off = segs[s].off;
       seg_run = segs[s].run_bytes;
       seg_begin = segs[s].tile_begin;
@@ -741,15 +743,21 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
     const bool last = (t + 1 == seg_end);
     gbytes pay = payload + seg_off;
     if (dsel == 0) {
-      // one contiguous run
-      const uint64_t boff = static_cast<uint64_t>(q) * kTile;
-      const uint64_t left = seg_run - boff;
-      gbytes ten = as_global(seg_ptr) + boff;
+      // One contiguous run.  Its first `head` bytes (fewer than 128) are peeled off and
+      // moved by tile 0 on top of its own range, so that every tile starts on a 128-byte
+      // line of the side that is written.
+      const uint32_t head = static_cast<uint32_t>(seg_run >> kSegHeadShift);
+      const uint64_t run = seg_run & kSegRunMask;
+      const uint64_t boff = head + static_cast<uint64_t>(q) * kTile;
+      const uint64_t left = run > boff ? run - boff : 0;
+      gbytes ten = as_global(seg_ptr);
       if constexpr (PACK) {
-        wave_copy<ROWS, NTT, NTP>(ten, pay + boff, left, lane, lane_off);
-        if (last && pad) wave_zero(pay + seg_run, pad, lane);
+        if (head && q == 0) wave_copy_partial<1, NTT, NTP>(ten, pay, head, lane, lane_off);
+        wave_copy<ROWS, NTT, NTP>(ten + boff, pay + boff, left, lane, lane_off);
+        if (last && pad) wave_zero(pay + run, pad, lane);
       } else {
-        wave_copy<ROWS, NTP, NTT>(pay + boff, ten, left, lane, lane_off);
+        if (head && q == 0) wave_copy_partial<1, NTP, NTT>(pay, ten, head, lane, lane_off);
+        wave_copy<ROWS, NTP, NTT>(pay + boff, ten + boff, left, lane, lane_off);
       }
     } else if (dsel == kSegFillOnly) {
       if constexpr (PACK) wave_zero(pay, pad, lane);
@@ -794,7 +802,7 @@ template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
     const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
     uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
-    uint32_t lds_per_wave, uint32_t nt_bits) {
+    uint32_t lds_per_wave, uint32_t nt_bits, int64_t tensor_delta) {
   // Scalar arguments (not one struct) so that the compiler can preload them
   // into SGPRs at dispatch instead of fetching the kernarg segment first.
   KernelArgs a;
@@ -802,11 +810,50 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   a.tiles_per_wave = tiles_per_wave;
   a.xcd_remap = xcd_remap;
   a.seg_shift = seg_shift;
+  a.tensor_delta = tensor_delta;
   bundle_body<PACK, ROWS, NTT, NTP, ELEMENTS>(
       reinterpret_cast<seg_table>(reinterpret_cast<uintptr_t>(segs_arg)),
       reinterpret_cast<dims_table>(reinterpret_cast<uintptr_t>(dims_arg)),
       reinterpret_cast<const AXR_CONST uint32_t*>(reinterpret_cast<uintptr_t>(wave_seg_arg)),
-      reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(payload_arg)), a, lds_per_wave, nt_bits);
+      reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(payload_arg)), a, blockIdx.x, lds_per_wave,
+      nt_bits);
+}
+
+// Several bundles in ONE launch: the grid is cut into consecutive workgroup ranges, one per
+// job, and every workgroup walks the tables of its own job in that job's direction (a
+// sender packing bundle k + 1 while the receiver unpacks bundle k; a batch of small
+// bundles).  Halves the per-launch cost of short kernels.  The job table arrives by value
+// and is read in place in the kernarg segment (scalar loads, no private copy).
+template <uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
+__global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_jobs_kernel(
+    JobTable jobs_arg) {
+  (void)jobs_arg;
+  const AXR_CONST JobTable* jt =
+      (const AXR_CONST JobTable*)__builtin_amdgcn_kernarg_segment_ptr();
+  const uint32_t wg = blockIdx.x;
+  uint32_t j = 0;
+#pragma unroll
+  for (uint32_t k = 1; k < kMaxJobs; ++k)
+    if (k < jt->count && wg >= jt->job[k].wg_begin) j = k;
+  const AXR_CONST JobDesc* d = &jt->job[j];
+  KernelArgs a;
+  a.ntiles = d->ntiles;
+  a.tiles_per_wave = d->tiles_per_wave;
+  a.xcd_remap = 0;
+  a.seg_shift = d->seg_shift;
+  a.tensor_delta = d->tensor_delta;
+  seg_table segs = reinterpret_cast<seg_table>(d->segs);
+  dims_table dims = reinterpret_cast<dims_table>(d->dims);
+  const AXR_CONST uint32_t* wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(d->wave_seg);
+  gbytes payload = reinterpret_cast<gbytes>(d->payload);
+  const uint32_t local = wg - d->wg_begin;
+  if (d->unpack) {   // workgroup-uniform
+    bundle_body<false, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, jt->lds_per_wave,
+                                                 jt->nt_bits);
+  } else {
+    bundle_body<true, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, jt->lds_per_wave,
+                                                jt->nt_bits);
+  }
 }
 
 // Tables of a small bundle travelling in the kernel arguments themselves: no
@@ -837,12 +884,14 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   a.tiles_per_wave = tiles_per_wave;
   a.xcd_remap = xcd_remap;
   a.seg_shift = seg_shift;
+  a.tensor_delta = 0;
   // tensor side streaming, payload side cacheable: what small bundles use
   bundle_body<PACK, 2, true, false, ELEMENTS>(
       reinterpret_cast<seg_table>(base + kInlineTablesHead),
       reinterpret_cast<dims_table>(base + kInlineTablesHead + dims_at),
       reinterpret_cast<const AXR_CONST uint32_t*>(base + kInlineTablesHead + wave_at),
-      reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(payload_arg)), a, lds_per_wave, nt_bits);
+      reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(payload_arg)), a, blockIdx.x, lds_per_wave,
+      nt_bits);
 }
 
 __global__ __launch_bounds__(256) void fill_kernel(uint8_t* dst, uint8_t value, size_t bytes) {
@@ -965,7 +1014,7 @@ template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
   const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * (cfg.threads / kWaveLanes) : 0u;
-#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave, cfg.nontemporal
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave, cfg.nontemporal, args.tensor_delta
 #define AXR_LAUNCH(NTT, NTP, EL) \
   hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, lds_bytes, stream, AXR_ARGS)
   // cfg.elements: strided tensors with short runs or transpositions are present
@@ -1023,6 +1072,54 @@ int launch_bundle_kernel(bool pack, const KernelArgs& args, const LaunchConfig& 
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   return pack ? launch_dir<true>(args, cfg, s) : launch_dir<false>(args, cfg, s);
+}
+
+int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stream) {
+  if (jobs.count == 0 || cfg.workgroups == 0) return AXR_OK;
+  if (jobs.count > kMaxJobs) return fail(AXR_ERR_INVALID, "too many jobs for one launch");
+  if (cfg.threads == 0 || cfg.threads % kWaveLanes ||
+      cfg.threads > (cfg.elements ? kMaxElementThreads : kMaxThreadsPerWorkgroup))
+    return fail(AXR_ERR_INVALID, "workgroup size does not fit the kernel");
+  if (static_cast<uint64_t>(cfg.lds_per_wave) * (cfg.threads / kWaveLanes) > 64u * 1024u)
+    return fail(AXR_ERR_INVALID, "workgroup needs more than 64 KiB of LDS");
+  const uint32_t waves_per_wg = cfg.threads / kWaveLanes;
+  for (uint32_t k = 0; k < jobs.count; ++k) {
+    const JobDesc& d = jobs.job[k];
+    const uint32_t end = k + 1 < jobs.count ? jobs.job[k + 1].wg_begin : cfg.workgroups;
+    if (d.wg_begin > end || (k == 0 && d.wg_begin != 0))
+      return fail(AXR_ERR_INVALID, "job workgroup ranges are not consecutive");
+    const uint64_t covered = static_cast<uint64_t>(end - d.wg_begin) * waves_per_wg * d.tiles_per_wave;
+    if (covered < d.ntiles) return fail(AXR_ERR_INVALID, "launch geometry does not cover a job's tiles");
+  }
+  const dim3 grid(cfg.workgroups), block(cfg.threads);
+  const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * waves_per_wg : 0u;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define AXR_JOBS(ROWS, NTT, NTP, EL) \
+  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, jobs)
+#define AXR_JOBS_NT(ROWS, EL)                                    \
+  switch (cfg.nontemporal & 3u) {                                \
+    case 0: AXR_JOBS(ROWS, false, false, EL); break;             \
+    case 1: AXR_JOBS(ROWS, true, false, EL); break;              \
+    case 2: AXR_JOBS(ROWS, false, true, EL); break;              \
+    default: AXR_JOBS(ROWS, true, true, EL); break;              \
+  }
+  if (cfg.elements) {
+    // bundles with short strided runs or transpositions: the default tile only
+    if (cfg.tile_rows != 2) return fail(AXR_ERR_INVALID, "element-mode jobs need 2 KiB tiles");
+    AXR_JOBS_NT(2, true)
+  } else {
+    switch (cfg.tile_rows) {
+      case 1: AXR_JOBS_NT(1, false) break;
+      case 2: AXR_JOBS_NT(2, false) break;
+      case 4: AXR_JOBS_NT(4, false) break;
+      case 8: AXR_JOBS_NT(8, false) break;
+      case 16: AXR_JOBS_NT(16, false) break;
+      default: return fail(AXR_ERR_INVALID, "tile_rows must be 1, 2, 4, 8 or 16");
+    }
+  }
+#undef AXR_JOBS_NT
+#undef AXR_JOBS
+  return check_hip(hipGetLastError(), "bundle jobs kernel launch");
 }
 
 int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchConfig& cfg,

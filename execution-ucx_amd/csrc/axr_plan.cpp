@@ -113,6 +113,7 @@ struct axr_plan {
   uint64_t payload_bytes = 0, data_bytes = 0;
   std::vector<uint8_t> header;
   bool bound = false;
+  bool receiver = false;             // made by axr_plan_from_header: tiles are anchored on the tensor side
 
   // device tables
   bool tables_built = false;
@@ -315,6 +316,7 @@ struct Builder {
   axr_plan* p;
   uint32_t tile_bytes;    // rows * 1 KiB with rows a power of two
   uint32_t tile_shift;    // log2(tile_bytes)
+  uint64_t head_align;    // 0 or a power of two up to 128
   uint64_t tiles = 0;
 
   int add_seg(uint32_t tensor, uint64_t ptr, uint64_t off, uint64_t run_bytes, uint64_t ntile,
@@ -338,7 +340,15 @@ struct Builder {
   int add_strided(uint32_t tensor, uint64_t ptr, uint64_t off, const uint64_t* ext,
                   const int64_t* str, size_t nd, uint64_t run_bytes) {
     if (nd == 0) {
-      return add_seg(tensor, ptr, off, run_bytes, (run_bytes + tile_bytes - 1) >> tile_shift, 0);
+      // Segments longer than a tile peel off their first bytes up to the next line of the
+      // side that is written (the payload for a sender's plan, the tensor for a receiver's),
+      // so that no two tiles write into one 128-byte line.
+      uint64_t head = 0;
+      if (head_align > 1 && run_bytes > tile_bytes && run_bytes <= kSegRunMask)
+        head = (0 - (p->receiver ? ptr : off)) & (head_align - 1);
+      int rc = add_seg(tensor, ptr, off, run_bytes | (head << kSegHeadShift),
+                       (run_bytes - head + tile_bytes - 1) >> tile_shift, 0);
+      return rc;
     }
     uint64_t inner_runs = 1;
     for (size_t d = 1; d < nd; ++d) inner_runs *= ext[d];
@@ -541,7 +551,8 @@ int build_tables(axr_plan* p) {
                static_cast<uint64_t>(tn.max_tiles))
       rows *= 2;
   }
-  Builder b{p, rows * kRowBytes, static_cast<uint32_t>(__builtin_ctz(rows * kRowBytes))};
+  Builder b{p, rows * kRowBytes, static_cast<uint32_t>(__builtin_ctz(rows * kRowBytes)),
+            static_cast<uint64_t>(tn.head_align)};
   p->segs.reserve(p->tensors.size() + 1);
   p->seg_tensor.reserve(p->tensors.size());
 
@@ -798,7 +809,7 @@ void fill_inline_tables(axr_plan* p) {
   p->inline_ready = true;
 }
 
-int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* stream_) {
+int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* stream_, int64_t delta = 0) {
   if (!p) return fail(AXR_ERR_INVALID, "null plan");
   if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
   if (payload_bytes < p->payload_bytes)
@@ -824,6 +835,8 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
       return fail(AXR_ERR_UNSUPPORTED, "a bundle with host (kDLCPU) tensors cannot be captured in a graph");
   }
   if (!p->host_chunks.empty()) {
+    if (delta != 0)
+      return fail(AXR_ERR_UNSUPPORTED, "a tensor address delta cannot be applied to host (kDLCPU) tensors");
     rc = move_host_tensors(p, pack, static_cast<uint8_t*>(payload), stream);
     if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
       p->busy_streams.push_back(stream);
@@ -837,7 +850,8 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   a.tiles_per_wave = p->cfg.tiles_per_wave;
   a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
   a.seg_shift = p->cfg.seg_shift;
-  if ((capturing ? !p->resident : p->launches == 0 && !p->uploaded) &&
+  a.tensor_delta = delta;
+  if (delta == 0 && (capturing ? !p->resident : p->launches == 0 && !p->uploaded) &&
       tables_fit_kernel_arguments(p)) {
     // Small bundle, first launch: the tables ride in the kernel arguments.  The launch
     // owns its copy, so a capturing stream may record it.  A plan that is launched again
@@ -1107,6 +1121,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   }
   p->header.assign(h, h + length);
   p->bound = false;
+  p->receiver = true;
   *plan = p;
   return AXR_OK;
 }
@@ -1268,6 +1283,120 @@ int axr_pack_noalloc(axr_plan_t* plan, void* payload, size_t payload_bytes, void
   return guarded([&] { return pack_noalloc_body(plan, payload, payload_bytes, stream); });
 }
 
+// Several bundles on one stream, neighbours of one launch geometry sharing a launch.
+static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
+  if (n == 0) return AXR_OK;
+  if (!jobs) return fail(AXR_ERR_INVALID, "axr_submit: null job array");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  bool capturing = false;
+  if (stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    int rc = check_hip(hipStreamIsCapturing(stream, &status), "hipStreamIsCapturing");
+    if (rc) return rc;
+    capturing = status == hipStreamCaptureStatusActive;
+  }
+  // Everything is checked, and every table built, before the first launch: a refused job
+  // leaves nothing half submitted.
+  for (size_t i = 0; i < n; ++i) {
+    const axr_job_t& j = jobs[i];
+    axr_plan* p = j.plan;
+    if (!p) return fail(AXR_ERR_INVALID, "axr_submit: null plan in job " + std::to_string(i));
+    if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
+    if (j.payload_bytes < p->payload_bytes)
+      return fail(AXR_ERR_LENGTH, "payload buffer is smaller than the plan's payload");
+    if (p->payload_bytes && !j.payload) return fail(AXR_ERR_INVALID, "null payload");
+    for (size_t k = 0; k < i; ++k)
+      if (jobs[k].plan == p) return fail(AXR_ERR_INVALID, "axr_submit: one plan appears in two jobs");
+    int rc = build_tables(p);
+    if (rc) return rc;
+    if (j.unpack && p->overlapping_dst)
+      return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
+    if (!p->host_chunks.empty() && (capturing || j.tensor_delta != 0))
+      return fail(AXR_ERR_UNSUPPORTED, "a bundle with host (kDLCPU) tensors can neither be captured nor rebased");
+    if (capturing && p->ntiles && !p->resident)
+      return fail(AXR_ERR_INVALID, "call axr_plan_prepare before capturing this plan in a graph");
+  }
+  auto batchable = [](const axr_plan* p) {
+    return p->ntiles != 0 && p->host_chunks.empty() && !p->cfg.xcd_remap &&
+           (!p->cfg.elements || p->cfg.tile_rows == 2);
+  };
+  auto same_geometry = [](const axr_plan* x, const axr_plan* y) {
+    return x->cfg.tile_rows == y->cfg.tile_rows && x->cfg.threads == y->cfg.threads &&
+           (x->cfg.nontemporal & 3u) == (y->cfg.nontemporal & 3u) &&
+           (!(x->cfg.elements || y->cfg.elements) || (x->cfg.tile_rows == 2 && x->cfg.threads <= kMaxElementThreads));
+  };
+  size_t i = 0;
+  while (i < n) {
+    axr_plan* first = jobs[i].plan;
+    size_t end = i + 1;
+    if (batchable(first)) {
+      while (end < n && end - i < kMaxJobs && batchable(jobs[end].plan) &&
+             same_geometry(first, jobs[end].plan))
+        ++end;
+    }
+    if (end - i == 1) {
+      const axr_job_t& j = jobs[i];
+      int rc = run(j.plan, j.unpack == 0, j.payload, j.payload_bytes, stream_, j.tensor_delta);
+      if (rc) return rc;
+      i = end;
+      continue;
+    }
+    JobTable table;
+    std::memset(&table, 0, sizeof(table));
+    LaunchConfig cfg = first->cfg;
+    uint32_t wg = 0;
+    for (size_t k = i; k < end; ++k) {
+      const axr_job_t& j = jobs[k];
+      axr_plan* p = j.plan;
+      if (!p->resident) {
+        int rc = ensure_uploaded(p, stream);
+        if (rc) return rc;
+      }
+      const uint8_t* d = static_cast<const uint8_t*>(p->block.device);
+      JobDesc& jd = table.job[k - i];
+      jd.segs = reinterpret_cast<uint64_t>(d);
+      jd.dims = reinterpret_cast<uint64_t>(d + p->dims_at);
+      jd.wave_seg = reinterpret_cast<uint64_t>(d + p->wave_at);
+      jd.payload = reinterpret_cast<uint64_t>(j.payload);
+      jd.tensor_delta = j.tensor_delta;
+      jd.ntiles = p->ntiles;
+      jd.tiles_per_wave = p->cfg.tiles_per_wave;
+      jd.seg_shift = p->cfg.seg_shift;
+      jd.wg_begin = wg;
+      jd.unpack = j.unpack ? 1u : 0u;
+      if (static_cast<uint64_t>(wg) + p->cfg.workgroups > 0x7fffffffull)
+        return fail(AXR_ERR_UNSUPPORTED, "axr_submit: the jobs' grids exceed one launch");
+      wg += p->cfg.workgroups;
+      cfg.elements = cfg.elements || p->cfg.elements;
+      cfg.lds_per_wave = std::max(cfg.lds_per_wave, p->cfg.lds_per_wave);
+    }
+    table.count = static_cast<uint32_t>(end - i);
+    table.lds_per_wave = cfg.lds_per_wave;
+    table.nt_bits = cfg.nontemporal;
+    cfg.workgroups = wg;
+    if (cfg.lds_per_wave) {
+      // every plan sized its workgroups for its own LDS need; the launch uses the largest
+      const uint32_t fit = (64u * 1024u / cfg.lds_per_wave) * kWaveLanes;
+      if (cfg.threads > fit)
+        return fail(AXR_ERR_UNSUPPORTED, "axr_submit: jobs with transposed views of different block sizes");
+    }
+    int rc = launch_bundle_jobs(table, cfg, stream);
+    if (rc) return rc;
+    for (size_t k = i; k < end; ++k) {
+      axr_plan* p = jobs[k].plan;
+      ++p->launches;
+      if (!capturing &&
+          std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+        p->busy_streams.push_back(stream);
+    }
+    i = end;
+  }
+  return AXR_OK;
+}
+int axr_submit(const axr_job_t* jobs, size_t n, void* stream) {
+  return guarded([&] { return submit_body(jobs, n, stream); });
+}
+
 static int plan_launch_info_body(axr_plan_t* plan, axr_launch_info_t* info) {
   if (!plan || !info) return fail(AXR_ERR_INVALID, "axr_plan_launch_info: null argument");
   int rc = build_tables(plan);
@@ -1330,7 +1459,9 @@ static int plan_segments_body(axr_plan_t* plan, axr_segment_info_t* out, size_t 
     const uint32_t dsel = s.meta >> kSegDimsShift;
     if (dsel == 0) {
       o.mode = 0;
-      o.nbytes = s.run_bytes;
+      o.run_bytes = s.run_bytes & kSegRunMask;
+      o.head = static_cast<uint32_t>(s.run_bytes >> kSegHeadShift);
+      o.nbytes = o.run_bytes;
     } else if (dsel == kSegFillOnly) {
       o.mode = 3;
     } else {

@@ -409,6 +409,10 @@ static int tune_set_body(const char* key, int64_t value) {
     t.inline_tables = value;
   } else if (k == "transpose") {
     t.transpose = value ? 1 : 0;
+  } else if (k == "head_align") {
+    if (value < 0 || value > 128 || (value & (value - 1)))
+      return fail(AXR_ERR_INVALID, "head_align must be 0 or a power of two up to 128");
+    t.head_align = value;
   } else {
     return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   }
@@ -434,6 +438,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "ragged_runs") *value = t.ragged_runs;
   else if (k == "inline_tables") *value = t.inline_tables;
   else if (k == "host_threads") *value = t.host_threads;
+  else if (k == "head_align") *value = t.head_align;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

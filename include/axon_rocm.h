@@ -300,6 +300,28 @@ AXR_API int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_byt
  * passes through a kernel. */
 AXR_API int axr_plan_prepare(axr_plan_t* plan, void* stream);
 
+/* Several bundles handed over at once.  A worker that has requests to send and
+ * responses to receive at the same moment (ClientSendRequest_ next to
+ * ProcessRndvBuffer_, axon/src/axon_worker.cpp:1424-1490 and :1098-1219, run by
+ * independent coroutines in the reference) submits the gathers and scatters
+ * together: neighbouring jobs of one launch geometry share ONE kernel launch
+ * (up to four per launch; a short kernel's fixed cost is paid once), the rest run
+ * one after the other, all on `stream`.  The jobs of one call must not depend on
+ * each other (no job may read what another one writes) and no plan may appear
+ * twice.  `tensor_delta` is added to every bound tensor address of that job: a
+ * plan bound once serves tensors of the same shapes and strides at another base
+ * (the chunks of a streamed transfer) without rebuilding or re-uploading its
+ * tables; it must be 0 for bundles with kDLCPU tensors.  Results are those of
+ * axr_pack / axr_unpack called job by job. */
+typedef struct axr_job {
+  axr_plan_t* plan;
+  int unpack;            /* 0: gather the tensors into payload; 1: scatter payload */
+  void* payload;
+  size_t payload_bytes;
+  int64_t tensor_delta;
+} axr_job_t;
+AXR_API int axr_submit(const axr_job_t* jobs, size_t n, void* stream);
+
 /* axr_pack for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
  * the reference (its payload never passes through a kernel).  Same result as
@@ -349,6 +371,10 @@ typedef struct axr_segment_info {
   uint32_t ndim;          /* strided outer dimensions (<= 6)                  */
   uint32_t granule;       /* mode 2: bytes per lane access; mode 5: element   */
   uint32_t tiles;
+  uint32_t head;          /* mode 0: leading bytes (< 128) that the first tile
+                             moves on top of its own range, so that the tiles
+                             start on a 128-byte line of the written side      */
+  uint32_t reserved;
   uint32_t shape[6];
   int64_t stride_bytes[6];
 } axr_segment_info_t;
@@ -365,6 +391,10 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "xcd_remap", "transpose" (1: transposed views move as square blocks through
  * LDS; 0: element by element), "ragged_runs" (1: short strided runs whose
  * length is no multiple of 16 bytes still move in 16-byte granules),
+ * "head_align" (contiguous tensors longer than a tile start their tiles on a
+ * multiple of this many bytes of the written side - the payload for a plan made
+ * by axr_plan_create, the tensor for one made by axr_plan_from_header; a power
+ * of two up to 128, default 16, 0: off),
  * "host_threads" (threads, the caller included, that share the host-side copies
  * between pageable memory and the pinned staging blocks once a copy is 2 MiB or
  * more; default 4, 1: the calling thread alone),

@@ -1,0 +1,264 @@
+"""axr_submit (several bundles per launch), tensor address deltas and the head peel of
+contiguous segments, against the CPU oracle and against axr_pack / axr_unpack, through
+the C ABI.  Bit-exact: this is byte movement."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+POISON = 0xCD
+
+
+def chunk_of(t):
+    import torch
+    if isinstance(t, torch.Tensor):
+        c = torch.empty(t.shape, dtype=t.dtype, device=t.device)
+        c.copy_(t)
+        return c.reshape(-1).view(torch.uint8).cpu().numpy()
+    return np.ascontiguousarray(t).view(np.uint8).reshape(-1)
+
+
+def random_tensors(rng, gpu, count, lo=16, hi=48 * 1024, strided_every=0, transposed_every=0):
+    import torch
+    dtypes = [torch.uint8, torch.float16, torch.float32, torch.int64]
+    out = []
+    for i in range(count):
+        dt = dtypes[i % 4]
+        item = torch.empty((), dtype=dt).element_size()
+        if transposed_every and i % transposed_every == 1:
+            r, c = int(rng.integers(40, 200)), int(rng.integers(40, 200))
+            raw = torch.from_numpy(rng.integers(0, 256, size=r * c * item, dtype=np.uint8)).to(gpu)
+            out.append(raw.view(dt).reshape(r, c).t())
+        elif strided_every and i % strided_every == 0:
+            rows, cols, pitch = int(rng.integers(2, 20)), int(rng.integers(1, 900)), 1024
+            raw = torch.from_numpy(rng.integers(0, 256, size=rows * pitch * item, dtype=np.uint8)).to(gpu)
+            out.append(raw.view(dt).reshape(rows, pitch)[:, :cols])
+        else:
+            n = max(1, int(np.exp(rng.uniform(np.log(lo), np.log(hi)))) // item)
+            raw = torch.from_numpy(rng.integers(0, 256, size=n * item, dtype=np.uint8)).to(gpu)
+            out.append(raw.view(dt))
+    return out
+
+
+def zeros_like_views(tensors):
+    """Destinations with the same shapes and strides as the sources (views stay views)."""
+    import torch
+    outs = []
+    for t in tensors:
+        if t.is_contiguous():
+            outs.append(torch.zeros_like(t))
+        else:
+            base = torch.zeros(t.untyped_storage().nbytes(), dtype=torch.uint8, device=t.device)
+            outs.append(torch.as_strided(base.view(t.dtype), t.shape, t.stride(), t.storage_offset()))
+    return outs
+
+
+def job_array(capi, jobs):
+    arr = (capi.Job * len(jobs))()
+    for i, (plan, unpack, ptr, nbytes, delta) in enumerate(jobs):
+        arr[i] = capi.Job(plan._h, unpack, ptr, nbytes, delta)
+    return arr
+
+
+@pytest.mark.parametrize("align", [1, 256])
+def test_submit_matches_the_oracle_and_separate_calls(pkg, orc, gpu, align):
+    """Six jobs in one call: packs and unpacks of bundles with plain tensors, strided
+    views, transposed views (element kernels), a bundle small enough for inline tables,
+    one with a host tensor (runs on its own) and one with another tile size."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    rng = np.random.default_rng(31 + align)
+    stream = C.c_void_p()
+    capi.check(lib.axr_stream_create(C.byref(stream)))
+    bundles = [
+        random_tensors(rng, gpu, 400),                                  # plain, pack
+        random_tensors(rng, gpu, 300, strided_every=5),                 # run tiles + elements, pack
+        random_tensors(rng, gpu, 5),                                    # tiny
+        random_tensors(rng, gpu, 200, strided_every=4, transposed_every=6),
+        random_tensors(rng, gpu, 64, lo=100000, hi=400000),            # larger tensors
+    ]
+    host = rng.integers(0, 256, size=70001, dtype=np.uint8)
+    bundles.append([bundles[0][3], host, bundles[0][4]])                # host tensor inside
+    torch.cuda.synchronize()
+    plans, bufs, wants = [], [], []
+    for tensors in bundles:
+        plan = pkg.BundlePlan.create(tensors, align=align)
+        plans.append(plan)
+        bufs.append(torch.full((plan.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu))
+        wants.append(orc.pack([chunk_of(t) for t in tensors], align))
+    torch.cuda.synchronize()
+    try:
+        # all packs in one call
+        arr = job_array(capi, [(p, 0, b.data_ptr(), p.payload_bytes, 0) for p, b in zip(plans, bufs)])
+        capi.check(lib.axr_submit(arr, len(plans), stream))
+        capi.check(lib.axr_stream_synchronize(stream))
+        for p, b, w in zip(plans, bufs, wants):
+            got = b.cpu().numpy()
+            assert np.array_equal(got[:p.payload_bytes], w)
+            assert (got[p.payload_bytes:] == POISON).all()
+        # unpacks of bundles 0..4 together with a fresh pack of bundle 0's twin: mixed directions
+        outs = [zeros_like_views(t) for t in bundles[:5]]
+        rplans = [pkg.BundlePlan.from_header(p.header).bind(o) for p, o in zip(plans[:5], outs)]
+        twin = pkg.BundlePlan.create(bundles[0], align=align)
+        twin_buf = torch.full((twin.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu)
+        torch.cuda.synchronize()
+        jobs = [(rp, 1, b.data_ptr(), p.payload_bytes, 0) for rp, p, b in zip(rplans, plans, bufs)]
+        jobs.insert(1, (twin, 0, twin_buf.data_ptr(), twin.payload_bytes, 0))
+        arr = job_array(capi, jobs)
+        capi.check(lib.axr_submit(arr, len(jobs), stream))
+        capi.check(lib.axr_stream_synchronize(stream))
+        for tensors, o in zip(bundles[:5], outs):
+            for a, b in zip(tensors, o):
+                assert np.array_equal(chunk_of(a), chunk_of(b))
+        assert np.array_equal(twin_buf.cpu().numpy()[:twin.payload_bytes], wants[0])
+        # the same through axr_pack: identical bytes
+        ref = torch.full((plans[1].payload_bytes,), POISON, dtype=torch.uint8, device=gpu)
+        solo = pkg.BundlePlan.create(bundles[1], align=align)
+        solo.pack(ref.data_ptr(), solo.payload_bytes, stream.value)
+        capi.check(lib.axr_stream_synchronize(stream))
+        assert torch.equal(ref, bufs[1][:solo.payload_bytes])
+        for p in rplans + [twin, solo]:
+            p.close()
+    finally:
+        for p in plans:
+            p.close()
+        capi.check(lib.axr_stream_destroy(stream))
+
+
+def test_submit_refusals(pkg, gpu):
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    x = torch.arange(4096, dtype=torch.uint8, device=gpu)
+    plan = pkg.BundlePlan.create([x], align=1)
+    buf = torch.zeros(4096, dtype=torch.uint8, device=gpu)
+    torch.cuda.synchronize()
+    assert lib.axr_submit(None, 0, None) == 0
+    assert lib.axr_submit(None, 1, None) == capi.AXR_ERR_INVALID
+    arr = job_array(capi, [(plan, 0, buf.data_ptr(), 4095, 0)])
+    assert lib.axr_submit(arr, 1, None) == capi.AXR_ERR_LENGTH
+    arr = job_array(capi, [(plan, 0, buf.data_ptr(), 4096, 0), (plan, 0, buf.data_ptr(), 4096, 0)])
+    assert lib.axr_submit(arr, 2, None) == capi.AXR_ERR_INVALID          # one plan twice
+    host = np.arange(64, dtype=np.uint8)
+    hplan = pkg.BundlePlan.create([host], align=1)
+    arr = job_array(capi, [(hplan, 0, buf.data_ptr(), 64, 128)])
+    assert lib.axr_submit(arr, 1, None) == capi.AXR_ERR_UNSUPPORTED      # host tensors cannot be rebased
+    unbound = pkg.BundlePlan.from_header(plan.header)
+    arr = job_array(capi, [(unbound, 1, buf.data_ptr(), 4096, 0)])
+    assert lib.axr_submit(arr, 1, None) == capi.AXR_ERR_INVALID
+    torch.cuda.synchronize()
+    assert bool((buf == 0).all())                                        # nothing ran
+    for p in (plan, hplan, unbound):
+        p.close()
+
+
+def test_tensor_delta_serves_chunks_of_one_geometry(pkg, orc, gpu):
+    """One plan bound to chunk 0 of a pitched parent gathers chunks 1..3 through the
+    delta, and one receiver plan scatters them into another parent."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    rng = np.random.default_rng(9)
+    chunks, views, rows, cols, pitch = 4, 6, 40, 1000, 1536
+    src = torch.from_numpy(rng.integers(-2 ** 15, 2 ** 15, size=(chunks, views, rows, pitch),
+                                        dtype=np.int16)).to(gpu)
+    dst = torch.zeros_like(src)
+    chunk_bytes = views * rows * pitch * 2
+
+    def tensors_of(parent, k):
+        return [parent[k, v, :, :cols] for v in range(views)]
+
+    plan = pkg.BundlePlan.create(tensors_of(src, 0), align=256)
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(tensors_of(dst, 0))
+    n = plan.payload_bytes
+    bufs = [torch.full((n,), POISON, dtype=torch.uint8, device=gpu) for _ in range(chunks)]
+    torch.cuda.synchronize()
+    # every tensor of the bundle moves by the same number of bytes from chunk to chunk
+    for k in range(chunks):
+        arr = job_array(capi, [(plan, 0, bufs[k].data_ptr(), n, k * chunk_bytes)])
+        capi.check(lib.axr_submit(arr, 1, None))
+    torch.cuda.synchronize()
+    view_bytes = rows * cols * 2
+    for k in range(chunks):
+        got = bufs[k].cpu().numpy()
+        want = orc.pack([chunk_of(src[k, v, :, :cols]) for v in range(views)], 256)
+        assert np.array_equal(got, want), k
+    for k in range(chunks):
+        arr = job_array(capi, [(rplan, 1, bufs[k].data_ptr(), n, k * chunk_bytes)])
+        capi.check(lib.axr_submit(arr, 1, None))
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:, :, :, :cols], src[:, :, :, :cols])
+    assert bool((dst[:, :, :, cols:] == 0).all())
+    assert view_bytes * views <= n
+    # the delta also reaches the segments of a plan whose tables ride in the kernel arguments
+    # on its first launch: a rebased first launch must not take that path with delta 0
+    fresh = pkg.BundlePlan.create(tensors_of(src, 0), align=256)
+    one = torch.full((n,), POISON, dtype=torch.uint8, device=gpu)
+    arr = job_array(capi, [(fresh, 0, one.data_ptr(), n, 2 * chunk_bytes)])
+    capi.check(lib.axr_submit(arr, 1, None))
+    torch.cuda.synchronize()
+    assert torch.equal(one, bufs[2])
+    fresh.close()
+    plan.close()
+    rplan.close()
+
+
+@pytest.mark.parametrize("head_align", [128, 16, 0])
+def test_head_peel_every_misalignment(pkg, orc, gpu, head_align):
+    """Contiguous tensors longer than a tile whose tensor address and payload offset take
+    every residue modulo 128, in both directions and with plans used against their
+    orientation (a sender's plan unpacking, a receiver's plan packing)."""
+    import torch
+    before = C.c_int64()
+    pkg._capi.check(pkg._capi.load().axr_tune_get(b"head_align", C.byref(before)))
+    pkg.tune(head_align=head_align)
+    try:
+        rng = np.random.default_rng(77)
+        arena = torch.from_numpy(rng.integers(0, 256, size=4 << 20, dtype=np.uint8)).to(gpu)
+        views, at = [], 0
+        for k in range(140):
+            n = int(rng.integers(2049, 9000)) if k % 3 else int(rng.integers(1, 2200))
+            at += int(rng.integers(0, 3)) * 64 + (k % 128)              # every residue on the tensor side
+            views.append(arena[at:at + n])
+            at += n
+        chunks = [chunk_of(v) for v in views]
+        for align in (1, 4, 256):
+            for shift in (0, 1, 77):                                      # payload base not aligned either
+                plan = pkg.BundlePlan.create(views, align=align)
+                n = plan.payload_bytes
+                heads = [s["head"] for s in plan.segments()]
+                assert max(heads) < max(head_align, 1)
+                if head_align and align == 1:
+                    assert max(heads) > 0                                 # the peel is in use
+                buf = torch.full((n + shift + 64,), POISON, dtype=torch.uint8, device=gpu)
+                plan.pack(buf.data_ptr() + shift, n)
+                torch.cuda.synchronize()
+                got = buf.cpu().numpy()
+                assert np.array_equal(got[shift:shift + n], orc.pack(chunks, align)), (align, shift)
+                assert (got[:shift] == POISON).all() and (got[shift + n:] == POISON).all()
+                # receiver's plan (anchored on the tensor side) scatters
+                out_arena = torch.full_like(arena, POISON)
+                outs = [out_arena[v.data_ptr() - arena.data_ptr():][:v.numel()] for v in views]
+                rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+                rplan.unpack(buf.data_ptr() + shift, n)
+                torch.cuda.synchronize()
+                mask = torch.zeros_like(arena, dtype=torch.bool)
+                for v in views:
+                    o = v.data_ptr() - arena.data_ptr()
+                    mask[o:o + v.numel()] = True
+                assert torch.equal(out_arena[mask], arena[mask])
+                assert bool((out_arena[~mask] == POISON).all())           # nothing beside the tensors
+                # against orientation: the receiver's plan packs, the sender's plan unpacks
+                buf2 = torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu)
+                rplan.pack(buf2.data_ptr(), n)
+                out2 = torch.full_like(arena, POISON)
+                outs2 = [out2[v.data_ptr() - arena.data_ptr():][:v.numel()] for v in views]
+                plan2 = pkg.BundlePlan.create(outs2, align=align)
+                plan2.unpack(buf.data_ptr() + shift, n)
+                torch.cuda.synchronize()
+                assert np.array_equal(buf2.cpu().numpy()[:n], orc.pack(chunks, align))
+                assert torch.equal(out2[mask], arena[mask]) and bool((out2[~mask] == POISON).all())
+                for p in (plan, rplan, plan2):
+                    p.close()
+    finally:
+        pkg.tune(head_align=before.value)
