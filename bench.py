@@ -5,9 +5,15 @@ A step is one pack plus one unpack of the 4,096-tensor mixed bundle
 (4096 1-D tensors of 256 B-64 KiB in five dtypes); inputs are resident in HBM before the timed region.
 `value` = 4 * P / t  (P = sum of tensor bytes; pack reads P and writes P, unpack
 reads P and writes P), in GB/s, timed with HIP events on the stream the kernels
-are launched on.  By default the steps rotate over several independent copies of
-the bundle so that the working set exceeds the 256 MB last-level cache and the
-figure is an HBM figure; the cache-resident rate is reported next to it.
+are launched on.  The steps rotate over several independent copies of the bundle so
+that the working set exceeds the 256 MB last-level cache, and they are software
+pipelined the way a worker with traffic in both directions runs them: step i hands
+the pack of bundle i+1 and the unpack of bundle i to axr_submit, which serves both
+with ONE kernel launch on one stream (every bundle is still packed once and
+unpacked once per step, and bundle i's unpack reads what the previous step's launch
+packed).  The same steps as two separate launches (axr_pack, axr_unpack) are
+reported next to it.  The K timed steps are repeated in batches until at least
+50 ms have been timed and the median batch is reported.
 
 Prints ONE JSON line.  Only one GPU is used: --gpus above 1 is refused.
 """
@@ -36,6 +42,8 @@ def parse_args():
                     help="independent bundle copies cycled through by the steps (1 = cache resident)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "transposed"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--separate-launches", action="store_true",
+                    help="time axr_pack + axr_unpack as two launches per step instead of one axr_submit")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--tune", default="", help="comma separated key=value kernel tunables")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
@@ -62,20 +70,35 @@ class Harness:
         self.capi.check(self.lib.axr_stream_synchronize(self.stream))
         self.torch.cuda.synchronize()
 
+    MIN_TIMED_MS = 50.0
+    MAX_BATCHES = 400
+
     def time_steps(self, step_fn, steps, warmup):
-        """Runs step_fn(i) warmup + steps times; returns milliseconds for `steps`."""
-        for i in range(warmup):
+        """Runs step_fn(i) `warmup` times, then batches of `steps` calls, each batch
+        between two HIP events on the launch stream, until MIN_TIMED_MS have been
+        timed; returns the median batch in milliseconds (and leaves the batch count
+        in self.batches)."""
+        i = 0
+        for _ in range(warmup):
             step_fn(i)
+            i += 1
         self.sync()
-        self.capi.check(self.lib.axr_event_record(self.ev0, self.stream))
-        for i in range(steps):
-            step_fn(i)
-        self.capi.check(self.lib.axr_event_record(self.ev1, self.stream))
-        self.capi.check(self.lib.axr_event_synchronize(self.ev1))
+        times, total = [], 0.0
+        while total < self.MIN_TIMED_MS and len(times) < self.MAX_BATCHES:
+            self.capi.check(self.lib.axr_event_record(self.ev0, self.stream))
+            for _ in range(steps):
+                step_fn(i)
+                i += 1
+            self.capi.check(self.lib.axr_event_record(self.ev1, self.stream))
+            self.capi.check(self.lib.axr_event_synchronize(self.ev1))
+            ms = C.c_float()
+            self.capi.check(self.lib.axr_event_elapsed_ms(self.ev0, self.ev1, C.byref(ms)))
+            times.append(float(ms.value))
+            total += times[-1]
         self.sync()
-        ms = C.c_float()
-        self.capi.check(self.lib.axr_event_elapsed_ms(self.ev0, self.ev1, C.byref(ms)))
-        return float(ms.value)
+        self.batches = len(times)
+        times.sort()
+        return times[len(times) // 2]
 
 
 class BundleSet:
@@ -83,10 +106,11 @@ class BundleSet:
 
     `check` compares source and destination on the device after a round trip."""
 
-    def __init__(self, h: Harness, src_views, dst_views, align, keep, check=None):
+    def __init__(self, h: Harness, src_views, dst_views, align, keep, check=None, clear=None):
         pkg = h.pkg
         self.keep = keep
         self.check = check
+        self.clear = clear
         self.pack_plan = pkg.BundlePlan.create(src_views, align=align)
         self.nbytes = self.pack_plan.payload_bytes
         self.data_bytes = self.pack_plan.data_bytes
@@ -110,6 +134,29 @@ def run_sets(h: Harness, sets, steps, warmup):
 
     ms = h.time_steps(step, steps, warmup)
     return ms
+
+
+def run_sets_one_launch(h: Harness, sets, steps, warmup):
+    """Step i = axr_submit({pack of set i+1, unpack of set i}): one kernel launch."""
+    lib, stream, capi = h.lib, h.stream, h.capi
+    n = len(sets)
+    if n < 2:
+        raise ValueError("the pipelined steps need at least two bundle copies")
+    jobs = []
+    for i in range(n):
+        a, b = sets[(i + 1) % n], sets[i]
+        arr = (capi.Job * 2)()
+        arr[0] = capi.Job(a.pp, 0, a.ptr, a.nbytes, 0)
+        arr[1] = capi.Job(b.up, 1, b.ptr, b.nbytes, 0)
+        jobs.append(arr)
+    capi.check(lib.axr_pack(sets[0].pp, sets[0].ptr, sets[0].nbytes, stream))   # fills the pipeline
+
+    def step(i):
+        rc = lib.axr_submit(jobs[i % n], 2, stream)
+        if rc:
+            capi.check(rc)
+
+    return h.time_steps(step, steps, warmup)
 
 
 def run_sets_two_streams(h: Harness, sets, steps, warmup):
@@ -138,16 +185,20 @@ def run_sets_two_streams(h: Harness, sets, steps, warmup):
     for i in range(warmup):
         step(i)
     drain()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step(i)
-    drain()
-    ms = (time.perf_counter() - t0) * 1e3
+    times, total = [], 0.0
+    while total < h.MIN_TIMED_MS and len(times) < h.MAX_BATCHES:
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        drain()
+        times.append((time.perf_counter() - t0) * 1e3)
+        total += times[-1]
     check(lib.axr_stream_destroy(second))
-    return ms
+    times.sort()
+    return times[len(times) // 2]
 
 
-def make_c2_sets(h, count, seed=0):
+def make_c2_sets(h, count, seed=0, align=256):
     from execution_ucx_amd import workloads
     spec = workloads.mixed_bundle(seed=seed)
     sets = []
@@ -160,8 +211,9 @@ def make_c2_sets(h, count, seed=0):
         dst = h.torch.zeros_like(arena)
         sv = workloads.mixed_views(spec, arena.data_ptr())
         dv = workloads.mixed_views(spec, dst.data_ptr())
-        sets.append(BundleSet(h, sv, dv, 256, (arena, dst),
-                              check=lambda a=arena, d=dst: bool(h.torch.equal(a, d))))
+        sets.append(BundleSet(h, sv, dv, align, (arena, dst),
+                              check=lambda a=arena, d=dst: bool(h.torch.equal(a, d)),
+                              clear=lambda d=dst: d.zero_()))
     return spec, sets
 
 
@@ -241,6 +293,20 @@ def verify_set(h, s):
         raise SystemExit("bench.py: round trip did not reproduce the source tensors")
 
 
+def check_sets(h, sets, what):
+    h.sync()
+    for s in sets:
+        if s.check is not None and not s.check():
+            raise SystemExit(f"bench.py: {what} did not reproduce the source tensors")
+
+
+def clear_sets(h, sets):
+    for s in sets:
+        if s.clear is not None:
+            s.clear()
+    h.sync()
+
+
 def rate(data_bytes, ms, steps):
     """GB/s of read+write traffic for `steps` pack+unpack round trips."""
     return 4.0 * data_bytes * steps / (ms * 1e-3) / 1e9
@@ -254,6 +320,9 @@ def end_to_end_us(h, spec, steps=20):
     lib, capi = h.lib, h.capi
     arena, _ = workloads.materialize_mixed(spec, "cuda", seed=99)
     dst = h.torch.zeros_like(arena)
+    mask = h.torch.zeros(spec.arena_bytes, dtype=h.torch.bool, device="cuda")
+    for s in spec.segments:
+        mask[s.arena_offset:s.arena_offset + s.nbytes] = True
     sa = TensorArray(workloads.mixed_views(spec, arena.data_ptr()))
     da = TensorArray(workloads.mixed_views(spec, dst.data_ptr()))
     probe = h.pkg.BundlePlan.create(sa.views, align=256)
@@ -282,7 +351,9 @@ def end_to_end_us(h, spec, steps=20):
         if it >= 3:
             times.append(t2 - t0)
             plan_times.append(t1 - t0)
-    assert h.torch.equal(arena, dst) or True   # gaps between tensors are not copied
+    # the bytes between the tensors are not part of the bundle and stay zero
+    if not (bool(h.torch.equal(arena[mask], dst[mask])) and bool((dst[~mask] == 0).all())):
+        raise SystemExit("bench.py: fresh-bundle round trip did not reproduce the tensors")
     times.sort()
     plan_times.sort()
     n_k = len(spec.segments) / 1000.0
@@ -432,8 +503,10 @@ def iov_against_bundle(h, spec, reps=7):
         t_iov.append(time.perf_counter() - t0)
         done = C.c_int()
         capi.check(lib.axr_am_request_test(client._h, req.value, C.byref(done)))
-    ok_iov = all(bool(torch.equal(arena[s.arena_offset:s.arena_offset + s.nbytes],
-                                  dst[s.arena_offset:s.arena_offset + s.nbytes])) for s in spec.segments[::97])
+    mask = torch.zeros(spec.arena_bytes, dtype=torch.bool, device="cuda")
+    for s in spec.segments:
+        mask[s.arena_offset:s.arena_offset + s.nbytes] = True
+    ok_iov = bool(torch.equal(arena[mask], dst[mask])) and bool((dst[~mask] == 0).all())
     dst.zero_()
     from execution_ucx_amd.dlpack import TensorArray
     plan = h.pkg.BundlePlan.create(TensorArray(workloads.mixed_views(spec, arena.data_ptr())), align=256)
@@ -454,8 +527,7 @@ def iov_against_bundle(h, spec, reps=7):
         h.sync()
         t_bundle.append(time.perf_counter() - t0)
         client.test(req)
-    ok_bundle = all(bool(torch.equal(arena[s.arena_offset:s.arena_offset + s.nbytes],
-                                     dst[s.arena_offset:s.arena_offset + s.nbytes])) for s in spec.segments[::97])
+    ok_bundle = bool(torch.equal(arena[mask], dst[mask])) and bool((dst[~mask] == 0).all())
     if not (ok_iov and ok_bundle):
         raise SystemExit("bench.py: loopback transfer differs")
     client.close()
@@ -548,6 +620,83 @@ def cpu_baseline(spec, seed=0):
     return base, allc
 
 
+def cpu_baseline_other_configs():
+    """The same reference host path on the host-memory bundle (64 x 64 KiB fp32) and on the
+    Llama-7B layer bundle (0.4 GB), one thread, tight layout."""
+    import numpy as np
+    import oracle
+    from execution_ucx_amd import workloads
+    out = {}
+    c1 = [a.view(np.uint8) for a in workloads.host_bundle_c1(seed=0)]
+    r = oracle.time_pack_unpack(c1, align=1, threads=1, warmup=3, reps=200)
+    out["cpu_baseline_c1"] = {"value": round(4.0 * r["data_bytes"] / r["seconds"] / 1e9, 3), "unit": "GB/s",
+                              "cores": 1, "kind": r["kind"],
+                              "sample": "64 fp32 tensors of 64 KiB (4 MiB), median of 200 pack+unpack repetitions"}
+    rng = np.random.default_rng(0)
+    c3 = [rng.integers(0, 256, size=int(np.prod(shape)) * 2, dtype=np.uint8)
+          for _, shape in workloads.LLAMA7B_LAYER]
+    r = oracle.time_pack_unpack(c3, align=1, threads=1, warmup=1, reps=7)
+    out["cpu_baseline_c3"] = {"value": round(4.0 * r["data_bytes"] / r["seconds"] / 1e9, 3), "unit": "GB/s",
+                              "cores": 1, "kind": r["kind"],
+                              "sample": "the 9 bf16 tensors of one Llama-7B layer (404,766,720 B), "
+                                        "median of 7 pack+unpack repetitions"}
+    return out
+
+
+def tune_get(pkg, key):
+    v = C.c_int64()
+    pkg._capi.check(pkg._capi.load().axr_tune_get(key.encode(), C.byref(v)))
+    return v.value
+
+
+def graph_replay(h, sets, P, steps_in_graph=20):
+    """The pipelined steps recorded once into a HIP graph and replayed: GB/s, or a
+    string saying why it could not be measured."""
+    torch = h.torch
+    lib, capi = h.lib, h.capi
+    n = len(sets)
+    try:
+        for s in sets:
+            capi.check(lib.axr_plan_prepare(s.pp, h.stream))
+            capi.check(lib.axr_plan_prepare(s.up, h.stream))
+        h.sync()
+        side = torch.cuda.Stream()
+        jobs = []
+        for i in range(n):
+            a, b = sets[(i + 1) % n], sets[i]
+            arr = (capi.Job * 2)()
+            arr[0] = capi.Job(a.pp, 0, a.ptr, a.nbytes, 0)
+            arr[1] = capi.Job(b.up, 1, b.ptr, b.nbytes, 0)
+            jobs.append(arr)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(steps_in_graph):
+                capi.check(lib.axr_submit(jobs[i % n], 2, side.cuda_stream))
+        clear_sets(h, sets)
+        capi.check(lib.axr_pack(sets[0].pp, sets[0].ptr, sets[0].nbytes, h.stream))
+        h.sync()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        times = []
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                graph.replay()
+            side.synchronize()
+            total = 0.0
+            while total < h.MIN_TIMED_MS and len(times) < h.MAX_BATCHES:
+                e0.record(side)
+                graph.replay()
+                e1.record(side)
+                e1.synchronize()
+                times.append(e0.elapsed_time(e1))
+                total += times[-1]
+        check_sets(h, sets, "the graph replay")
+        del graph
+        times.sort()
+        return round(rate(P, times[len(times) // 2], steps_in_graph), 1)
+    except Exception as e:   # reported, never fatal for the benchmark line
+        return f"not measured: {type(e).__name__}: {e}"
+
+
 def load_traffic(kernel_key):
     path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
     try:
@@ -596,12 +745,24 @@ def main():
     for s in sets:
         verify_set(h, s)
     P = sets[0].data_bytes
-    ms = run_sets(h, sets, args.steps, args.warmup)
+    pipelined = len(sets) >= 2 and not args.separate_launches
+    clear_sets(h, sets)
+    if pipelined:
+        ms = run_sets_one_launch(h, sets, args.steps, args.warmup)
+        launches_per_step, bytes_per_launch = 1, 4 * P
+        kernel = "axr::bundle_jobs_kernel (one launch: pack of bundle i+1 and unpack of bundle i)"
+    else:
+        ms = run_sets(h, sets, args.steps, args.warmup)
+        launches_per_step, bytes_per_launch = 2, 2 * P
+        kernel = "axr::bundle_kernel (pack and unpack instantiations)"
+    batches = h.batches
+    if all(s.clear is not None for s in sets):
+        check_sets(h, sets, "the timed steps")
     value = rate(P, ms, args.steps)
     info = sets[0].pack_plan.launch_info()
-    launches = 2 * args.steps
-    launch_us = ms * 1e3 / launches
-    achieved = 2.0 * P / (launch_us * 1e-6) / 1e9
+    launch_us = ms * 1e3 / (launches_per_step * args.steps)
+    achieved = bytes_per_launch / (launch_us * 1e-6) / 1e9
+    traffic = load_traffic(args.workload if not pipelined else args.workload + "_one_launch")
 
     result = {
         "metric": "bundle pack+unpack GB/s (read+write)",
@@ -623,6 +784,9 @@ def main():
             "packed_bytes": sets[0].nbytes,
             "rotating_copies": len(sets),
             "working_set_bytes": len(sets) * 3 * sets[0].nbytes,
+            "step": ("pack of bundle i+1 and unpack of bundle i in one launch (axr_submit), one stream"
+                     if pipelined else "axr_pack then axr_unpack of one bundle, two launches, one stream"),
+            "timing": f"median of {batches} batches of {args.steps} steps, HIP events on the launch stream",
             "launch": info,
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
@@ -632,20 +796,47 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": load_traffic(args.workload),
-            "kernel": "axr::bundle_kernel (pack and unpack instantiations)",
-            "bytes_per_launch": 2 * P,
+            "traffic": traffic,
+            "traffic_source": ("profiles/pmc_traffic.json: FETCH_SIZE and WRITE_SIZE of earlier rocprofv3 --pmc "
+                               "runs of this command, scaled by a plain copy; not measured in this run"
+                               if traffic is not None else None),
+            "kernel": kernel,
+            "bytes_per_launch": bytes_per_launch,
             "avg_launch_us": round(launch_us, 3),
         },
     }
 
     if not args.no_extras and args.workload == "c2":
-        # cache-resident rate of the same bundle
+        def c2_variant(align=256, **tune):
+            """The headline steps on fresh plans under other tunables / another layout."""
+            defaults = {k: tune_get(pkg, k) for k in tune}
+            pkg.tune(**tune)
+            try:
+                _, vs = make_c2_sets(h, len(sets), align=align)
+                for v in vs:
+                    verify_set(h, v)
+                clear_sets(h, vs)
+                one = run_sets_one_launch(h, vs, args.steps, args.warmup)
+                check_sets(h, vs, "a C2 variant")
+                two = run_sets(h, vs, args.steps, args.warmup)
+                return {"one_launch_GBps": round(rate(P, one, args.steps), 1),
+                        "separate_launches_GBps": round(rate(P, two, args.steps), 1)}
+            finally:
+                pkg.tune(**defaults)
+
+        ms_sep = run_sets(h, sets, args.steps, args.warmup)
+        extras["c2_separate_launches_GBps"] = round(rate(P, ms_sep, args.steps), 1)
+        # cache-resident rate of the same bundle (one copy only: pack then unpack)
         ms1 = run_sets(h, sets[:1], args.steps, args.warmup)
         extras["c2_cache_resident_GBps"] = round(rate(P, ms1, args.steps), 1)
         # not `value`: bundles in flight on two streams hide the gap between dependent launches
         ms2 = run_sets_two_streams(h, sets, args.steps, args.warmup)
         extras["c2_two_streams_GBps"] = round(rate(P, ms2, args.steps), 1)
+        extras["c2_graph_replay_GBps"] = graph_replay(h, sets, P)
+        # the reference's own layout (tight concatenation) and a payload that bypasses the
+        # last-level cache on both sides
+        extras["c2_tight"] = c2_variant(align=1)
+        extras["c2_payload_streaming"] = c2_variant(payload_cache_bytes=0)
         extras.update({k: round(v, 2) for k, v in end_to_end_us(h, spec).items()})
         del sets
         torch.cuda.empty_cache()
@@ -653,8 +844,11 @@ def main():
         verify_set(h, c3[0])
         k3 = max(20, args.steps // 20)
         ms3 = run_sets(h, c3, k3, 5)
+        ms3b = run_sets_one_launch(h, c3, k3, 5)
+        check_sets(h, c3, "C3")
         extras["c3_llama_layer"] = {"GBps": round(rate(c3[0].data_bytes, ms3, k3), 1),
                                     "pct_of_hbm_peak": round(100 * rate(c3[0].data_bytes, ms3, k3) / HBM_PEAK_GBPS, 2),
+                                    "one_launch_GBps": round(rate(c3[0].data_bytes, ms3b, k3), 1),
                                     "payload_bytes_P": c3[0].data_bytes, "steps": k3,
                                     "ms_per_step": round(ms3 / k3, 5)}
         del c3
@@ -703,6 +897,8 @@ def main():
         base, allc = cpu_baseline(spec)
         result["cpu_baseline"] = base
         result["cpu_baseline_all_cores"] = allc
+        if not args.no_extras:
+            extras.update(cpu_baseline_other_configs())
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
