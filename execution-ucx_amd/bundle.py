@@ -220,6 +220,26 @@ class PackedBundle:
     def mem_h(self):
         return self.payload.mem_h
 
+    def close(self) -> None:
+        """Release the plan first (it waits for the pack kernel on its stream), then
+        return the payload block to the pool: a pool block is reusable the moment it
+        is freed, so it must not be freed while the kernel may still write it."""
+        if self.plan is not None:
+            self.plan.close()
+        if self.payload is not None:
+            self.payload.release()
+
+    def __del__(self):
+        # Dropping the object must not free the payload before the plan has drained the
+        # pack stream (the fields would otherwise go in declaration order, payload first).
+        # The payload itself is left to its own reference count: zero-copy views made
+        # from it may still be alive.
+        try:
+            if self.plan is not None:
+                self.plan.close()
+        except Exception:  # noqa: BLE001
+            pass
+
 
 def pack_bundle(tensors: Sequence[Any], align: int = 256, pool: Optional[DevicePool] = None,
                 stream=None) -> PackedBundle:

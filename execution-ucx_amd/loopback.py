@@ -154,6 +154,7 @@ class LoopbackAmContext:
         if self._h:
             _capi.check(self._lib.axr_am_context_destroy(self._h))
             self._h = None
+        self._keep.clear()      # sends that were never test()ed: nothing reads their bundles any more
 
     def __del__(self):
         try:

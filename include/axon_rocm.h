@@ -200,6 +200,12 @@ AXR_API int axr_pool_set_registrar(axr_pool_t* pool, axr_register_fn reg,
  * ucx_am_data_t::mem_h (ucx_context/ucx_context_def.h:80-93). */
 AXR_API int axr_pool_alloc(axr_pool_t* pool, size_t bytes, size_t alignment,
                            void** ptr, void** mem_h);
+/* The block is reusable the moment it is freed: nothing orders the free behind work
+ * that is still enqueued on a stream (the reference's cudaFree synchronises
+ * implicitly, cuda/ucx_cuda_memory_manager.hpp:108-131; a pool must not).  Free a
+ * payload only after the launches that touch it have finished: axr_plan_free and
+ * axr_plan_bind wait for a plan's launches, so "free the plan, then the payload"
+ * is always safe. */
 AXR_API int axr_pool_free(axr_pool_t* pool, void* ptr);
 /* Return fully free slabs to the driver. */
 AXR_API int axr_pool_trim(axr_pool_t* pool);

@@ -38,6 +38,21 @@ def test_host_layer_on_device(gpu):
     assert "host_selftest ok" in out.stdout
 
 
+@pytest.mark.gpu
+def test_receive_adapters_against_the_reference_classes(gpu):
+    """oracle/_ref/adapters_selftest (tests/cpp/adapters_selftest.cpp, built by oracle/Makefile
+    where the execution-ucx tree is mounted, with its real ucx_context_data.hpp and
+    ucx_memory_resource.cpp): PackTensors -> ToUcxBuffer -> ReceiveBufferFor -> memcpy ->
+    ToUcxBufferVec and RocmBundleReceivePolicy on the device, views against the reference's own
+    to_buffer_vec, payload against the oracle's pack, every pool block released once."""
+    exe = os.path.join(ROOT, "oracle", "_ref", "adapters_selftest")
+    assert os.path.exists(exe), "oracle/_ref/adapters_selftest is missing: run __graft_entry__.build() " \
+                                "where the reference tree is mounted"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "adapters_selftest ok" in out.stdout
+
+
 def test_planner_and_header_codec_under_sanitizers(tmp_path):
     """tests/cpp/plan_fuzz.cpp against a planner compiled with AddressSanitizer and
     UBSan (host code only; the kernels' object file is linked as built): random tensor
