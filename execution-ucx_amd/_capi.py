@@ -165,7 +165,12 @@ class Job(C.Structure):
     """axr_job_t: one gather or scatter of axr_submit."""
 
     _fields_ = [("plan", C.c_void_p), ("unpack", C.c_int), ("payload", C.c_void_p),
-                ("payload_bytes", C.c_size_t), ("tensor_delta", C.c_int64)]
+                ("payload_bytes", C.c_size_t), ("tensor_delta", C.c_int64), ("flags", C.c_uint32),
+                ("reserved", C.c_uint32)]
+
+
+JOB_PAYLOAD_STREAMING = 1
+JOB_PAYLOAD_CACHED = 2
 
 
 class AmData(C.Structure):
@@ -268,6 +273,10 @@ PROTOTYPES = {
     "axr_am_recv_buffer_iov": (C.c_int, [_vp, C.c_uint64, C.c_int, C.POINTER(Buffer), _sz, _vp]),
     "axr_am_message_release": (C.c_int, [_vp, C.c_uint64]),
     "axr_am_pending": (C.c_int, [_vp, C.POINTER(_sz)]),
+    "axr_transfer_create": (C.c_int, [_vp, _sz, C.c_int, C.c_int, _vpp]),
+    "axr_transfer_submit": (C.c_int, [_vp, _vp, C.c_int64, _vp, C.c_int64]),
+    "axr_transfer_finish": (C.c_int, [_vp]),
+    "axr_transfer_destroy": (C.c_int, [_vp]),
     "axr_divide_by_two": (C.c_int, [_vp, _sz, _vp]),
     "axr_compare": (C.c_int, [_vp, _vp, _sz, _u64p]),
     "axr_checksum": (C.c_int, [_vp, _sz, C.c_uint64, _u64p]),

@@ -179,6 +179,9 @@ struct Tunables {
   // 4096-tensor bundle: 16 lifts the tight layout by 2 % (every 16-byte store aligned) and
   // costs the 256-byte aligned layout nothing; 64 and 128 are no better for either.
   std::atomic<int64_t> head_align{16};
+  // The loopback transport moves a device payload to device memory of the same GPU with the
+  // library's copy kernel (1) or with hipMemcpyAsync (0).
+  std::atomic<int64_t> loopback_copy_kernel{1};
   std::atomic<int64_t> host_threads{4};       // threads (the caller included) for host-side staging copies
   std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
@@ -230,6 +233,8 @@ int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchC
 // hints; cfg.workgroups is the whole grid, cfg.lds_per_wave the largest need of any job).
 int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stream);
 int launch_fill(void* dst, int value, size_t bytes, void* stream);
+// dst[0, bytes) = src[0, bytes), both in device memory of the current device, no alignment needed.
+int launch_stream_copy(void* dst, const void* src, size_t bytes, bool nontemporal, void* stream);
 // Device address, on the current device, of the kStaticTableBytes bytes that hold the
 // tables of axr_pack_noalloc (a __device__ array of the code object: never allocated,
 // shared by every call on that device).

@@ -1010,6 +1010,22 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
   for (size_t i = tid; i < nvec; i += nthreads) dst[i] = src[i];
 }
 
+// One contiguous range, 2 KiB per wavefront with the same tile copy as the bundle
+// kernels (two 16-byte loads per lane in flight, an overlapped final vector instead of a
+// byte tail).  The loopback transport moves same-device payloads with it.
+template <bool NT>
+__global__ __launch_bounds__(256) void stream_copy_kernel(const uint8_t* src_arg, uint8_t* dst_arg,
+                                                          uint64_t bytes) {
+  constexpr uint32_t kTile = 2 * kRowBytes;
+  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
+  const uint64_t wave = uniform(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+  const uint64_t off = wave * kTile;
+  if (off >= bytes) return;
+  gcbytes src = reinterpret_cast<gcbytes>(reinterpret_cast<uintptr_t>(src_arg)) + off;
+  gbytes dst = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(dst_arg)) + off;
+  wave_copy<2, NT, NT>(src, dst, bytes - off, lane, lane * kVecBytes);
+}
+
 template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
@@ -1188,6 +1204,23 @@ int static_table_area(void** ptr) {
   }
   *ptr = address;
   return AXR_OK;
+}
+
+int launch_stream_copy(void* dst, const void* src, size_t bytes, bool nontemporal, void* stream) {
+  if (bytes == 0) return AXR_OK;
+  const uint64_t waves = (static_cast<uint64_t>(bytes) + 2 * kRowBytes - 1) / (2 * kRowBytes);
+  const uint64_t groups = (waves + 3) / 4;
+  if (groups > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "range too long for one copy launch");
+  const dim3 grid(static_cast<uint32_t>(groups)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (nontemporal) {
+    hipLaunchKernelGGL(stream_copy_kernel<true>, grid, block, 0, s, static_cast<const uint8_t*>(src),
+                       static_cast<uint8_t*>(dst), static_cast<uint64_t>(bytes));
+  } else {
+    hipLaunchKernelGGL(stream_copy_kernel<false>, grid, block, 0, s, static_cast<const uint8_t*>(src),
+                       static_cast<uint8_t*>(dst), static_cast<uint64_t>(bytes));
+  }
+  return check_hip(hipGetLastError(), "stream copy launch");
 }
 
 int launch_fill(void* dst, int value, size_t bytes, void* stream) {

@@ -85,6 +85,13 @@ int copy_piece(int dst_type, void* dst, int src_type, const void* src, size_t n,
     std::memcpy(dst, src, n);
     return AXR_OK;
   }
+  if (dst_type == AXR_MEM_ROCM && src_type == AXR_MEM_ROCM && tunables().loopback_copy_kernel != 0) {
+    // same GPU on both sides: the copy kernel (cacheable while the payload fits the last-level
+    // cache, as the bundle kernels treat a payload)
+    // (source and destination both take room there)
+    const bool nt = 2 * static_cast<uint64_t>(n) > static_cast<uint64_t>(tunables().payload_cache_bytes);
+    return launch_stream_copy(dst, src, n, nt, s);
+  }
   return check_hip(hipMemcpyAsync(dst, src, n, hipMemcpyDefault, s), "hipMemcpyAsync(loopback)");
 }
 

@@ -809,7 +809,16 @@ void fill_inline_tables(axr_plan* p) {
   p->inline_ready = true;
 }
 
-int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* stream_, int64_t delta = 0) {
+// The cache hint bits a job runs with: the plan's own, or with the payload side forced.
+uint32_t effective_nontemporal(const axr_plan* p, uint32_t job_flags) {
+  uint32_t nt = p->cfg.nontemporal & 3u;
+  if (job_flags & AXR_JOB_PAYLOAD_STREAMING) nt |= 2u;
+  else if (job_flags & AXR_JOB_PAYLOAD_CACHED) nt &= ~2u;
+  return nt;
+}
+
+int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* stream_, int64_t delta = 0,
+        uint32_t job_flags = 0) {
   if (!p) return fail(AXR_ERR_INVALID, "null plan");
   if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
   if (payload_bytes < p->payload_bytes)
@@ -851,8 +860,10 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
   a.seg_shift = p->cfg.seg_shift;
   a.tensor_delta = delta;
-  if (delta == 0 && (capturing ? !p->resident : p->launches == 0 && !p->uploaded) &&
-      tables_fit_kernel_arguments(p)) {
+  LaunchConfig cfg = p->cfg;
+  cfg.nontemporal = effective_nontemporal(p, job_flags);
+  if (delta == 0 && cfg.nontemporal == (p->cfg.nontemporal & 3u) &&
+      (capturing ? !p->resident : p->launches == 0 && !p->uploaded) && tables_fit_kernel_arguments(p)) {
     // Small bundle, first launch: the tables ride in the kernel arguments.  The launch
     // owns its copy, so a capturing stream may record it.  A plan that is launched again
     // is being reused: from the second launch on it pays one upload and then the shorter
@@ -882,7 +893,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   a.segs = reinterpret_cast<const Seg*>(d);
   a.dims = reinterpret_cast<const Dims*>(d + p->dims_at);
   a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
-  rc = launch_bundle_kernel(pack, a, p->cfg, stream);
+  rc = launch_bundle_kernel(pack, a, cfg, stream);
   if (rc) return rc;
   ++p->launches;
   // a capturing stream cannot be drained later; the caller keeps the plan alive
@@ -1301,6 +1312,10 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     const axr_job_t& j = jobs[i];
     axr_plan* p = j.plan;
     if (!p) return fail(AXR_ERR_INVALID, "axr_submit: null plan in job " + std::to_string(i));
+    if ((j.flags & ~(AXR_JOB_PAYLOAD_STREAMING | AXR_JOB_PAYLOAD_CACHED)) ||
+        (j.flags & (AXR_JOB_PAYLOAD_STREAMING | AXR_JOB_PAYLOAD_CACHED)) ==
+            (AXR_JOB_PAYLOAD_STREAMING | AXR_JOB_PAYLOAD_CACHED))
+      return fail(AXR_ERR_INVALID, "axr_submit: bad flags in job " + std::to_string(i));
     if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
     if (j.payload_bytes < p->payload_bytes)
       return fail(AXR_ERR_LENGTH, "payload buffer is smaller than the plan's payload");
@@ -1320,9 +1335,10 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     return p->ntiles != 0 && p->host_chunks.empty() && !p->cfg.xcd_remap &&
            (!p->cfg.elements || p->cfg.tile_rows == 2);
   };
-  auto same_geometry = [](const axr_plan* x, const axr_plan* y) {
+  auto same_geometry = [](const axr_job_t& jx, const axr_job_t& jy) {
+    const axr_plan *x = jx.plan, *y = jy.plan;
     return x->cfg.tile_rows == y->cfg.tile_rows && x->cfg.threads == y->cfg.threads &&
-           (x->cfg.nontemporal & 3u) == (y->cfg.nontemporal & 3u) &&
+           effective_nontemporal(x, jx.flags) == effective_nontemporal(y, jy.flags) &&
            (!(x->cfg.elements || y->cfg.elements) || (x->cfg.tile_rows == 2 && x->cfg.threads <= kMaxElementThreads));
   };
   size_t i = 0;
@@ -1331,12 +1347,12 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     size_t end = i + 1;
     if (batchable(first)) {
       while (end < n && end - i < kMaxJobs && batchable(jobs[end].plan) &&
-             same_geometry(first, jobs[end].plan))
+             same_geometry(jobs[i], jobs[end]))
         ++end;
     }
     if (end - i == 1) {
       const axr_job_t& j = jobs[i];
-      int rc = run(j.plan, j.unpack == 0, j.payload, j.payload_bytes, stream_, j.tensor_delta);
+      int rc = run(j.plan, j.unpack == 0, j.payload, j.payload_bytes, stream_, j.tensor_delta, j.flags);
       if (rc) return rc;
       i = end;
       continue;
@@ -1344,6 +1360,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     JobTable table;
     std::memset(&table, 0, sizeof(table));
     LaunchConfig cfg = first->cfg;
+    cfg.nontemporal = effective_nontemporal(first, jobs[i].flags);
     uint32_t wg = 0;
     for (size_t k = i; k < end; ++k) {
       const axr_job_t& j = jobs[k];

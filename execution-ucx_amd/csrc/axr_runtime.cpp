@@ -409,6 +409,8 @@ static int tune_set_body(const char* key, int64_t value) {
     t.inline_tables = value;
   } else if (k == "transpose") {
     t.transpose = value ? 1 : 0;
+  } else if (k == "loopback_copy_kernel") {
+    t.loopback_copy_kernel = value ? 1 : 0;
   } else if (k == "head_align") {
     if (value < 0 || value > 128 || (value & (value - 1)))
       return fail(AXR_ERR_INVALID, "head_align must be 0 or a power of two up to 128");
@@ -439,6 +441,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "inline_tables") *value = t.inline_tables;
   else if (k == "host_threads") *value = t.host_threads;
   else if (k == "head_align") *value = t.head_align;
+  else if (k == "loopback_copy_kernel") *value = t.loopback_copy_kernel;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

@@ -325,7 +325,16 @@ typedef struct axr_job {
   void* payload;
   size_t payload_bytes;
   int64_t tensor_delta;
+  uint32_t flags;        /* 0, or one AXR_JOB_PAYLOAD_* value                      */
+  uint32_t reserved;     /* 0                                                      */
 } axr_job_t;
+/* Cache treatment of the payload side for this job, overriding the plan's choice
+ * (cacheable up to "payload_cache_bytes", so that a consumer that follows at once
+ * finds the payload in the last-level cache): STREAMING when more payloads are in
+ * flight than that cache holds (the slots of a streamed transfer), CACHED to keep
+ * a larger payload cacheable. */
+#define AXR_JOB_PAYLOAD_STREAMING 1u
+#define AXR_JOB_PAYLOAD_CACHED 2u
 AXR_API int axr_submit(const axr_job_t* jobs, size_t n, void* stream);
 
 /* axr_pack for callers that cannot allocate device memory: code under HIP graph
@@ -404,6 +413,8 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "host_threads" (threads, the caller included, that share the host-side copies
  * between pageable memory and the pinned staging blocks once a copy is 2 MiB or
  * more; default 4, 1: the calling thread alone),
+ * "loopback_copy_kernel" (1, default: the loopback context moves a device payload
+ * to device memory with the library's copy kernel; 0: with hipMemcpyAsync),
  * "inline_tables" (the first launch of a bundle of at most this many tiles
  * whose tables fit into 3.5 KiB carries the tables inside the kernel arguments:
  * no table block and no upload; a plan that is launched again uploads its
@@ -498,6 +509,39 @@ AXR_API int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_
 AXR_API int axr_am_message_release(axr_am_context_t* ctx, uint64_t key);
 /* Messages queued and not yet taken by axr_am_recv_header. */
 AXR_API int axr_am_pending(axr_am_context_t* ctx, size_t* count);
+
+/* ------------------------------------------------------- streamed transfers */
+
+/* A large payload moved in chunks: pack -> connection_send -> connection_recv_buffer
+ * -> unpack per chunk (ucx_am_context.hpp:2234-2642 for the send, :1511-1844 for the
+ * receive), double-buffered: `lanes` lanes (2 is the classic double buffer), each a
+ * send slot and a receive slot of slot_bytes from `pool` (NULL: the default pool),
+ * over `streams` streams (1 <= streams <= lanes).  Chunk k uses lane k % lanes on
+ * stream (k % lanes) % streams.  streams == lanes: while chunk k is on the wire and
+ * being scattered, chunk k + 1 is gathered on the other stream.  streams == 1: the
+ * chunks run back to back on one stream and the second lane only lets the host queue
+ * one chunk ahead; on one GPU, where gather, wire copy and scatter all compete for
+ * the same HBM, this is the faster arrangement.  The transport is a loopback context
+ * pair inside the object: every chunk with a payload is a rendezvous whose fetch is
+ * a stream-ordered device copy from the send slot to the receive slot.
+ *
+ * The caller keeps ONE sender plan and ONE receiver plan (axr_plan_from_header of
+ * the sender's header, bound to the destination tensors) for all chunks of one
+ * geometry; send_delta / recv_delta say how far this chunk's tensors lie from the
+ * ones the plans are bound to (see axr_job_t.tensor_delta).  axr_transfer_submit
+ * never plans, uploads or allocates (after each plan's first use); it waits on the
+ * host only for the chunk that used the lane last.  AXR_ERR_MISMATCH when the
+ * receiver's plan does not describe the sender's header, AXR_ERR_LENGTH when a
+ * chunk exceeds a slot.  One thread at a time per transfer. */
+typedef struct axr_transfer axr_transfer_t;
+AXR_API int axr_transfer_create(axr_pool_t* pool, size_t slot_bytes, int lanes, int streams,
+                                axr_transfer_t** transfer);
+AXR_API int axr_transfer_submit(axr_transfer_t* transfer, axr_plan_t* send_plan, int64_t send_delta,
+                                axr_plan_t* recv_plan, int64_t recv_delta);
+/* Returns when every submitted chunk has arrived in its destination tensors. */
+AXR_API int axr_transfer_finish(axr_transfer_t* transfer);
+/* Finishes, then releases the slots, streams and contexts. */
+AXR_API int axr_transfer_destroy(axr_transfer_t* transfer);
 
 /* -------------------------------------------------- verification utilities */
 

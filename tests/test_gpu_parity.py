@@ -704,28 +704,90 @@ def test_c5_pitched_chunk(pkg, orc, gpu):
 
 def test_c5_streamed_pipeline(pkg, gpu):
     """Double-buffered pack -> loopback send -> unpack over two streams: small
-    chunks (eager and rendezvous sizes) and four full 256 MiB chunks."""
+    chunks (eager and rendezvous sizes by the reference's threshold) and the full
+    stream of 32 chunks of 256 MiB (8 GiB), all chunks of a stream served by one
+    sender plan and one receiver plan."""
     import torch
     from execution_ucx_amd import workloads
     for spec, chunks in ((workloads.pitched_chunk(views=3, rows=4, cols=64), 7),
                          (workloads.pitched_chunk(views=5, rows=64, cols=256), 9),
-                         (workloads.pitched_chunk(), 4)):
+                         (workloads.pitched_chunk(), 32)):
         src = torch.empty(chunks, spec.views, spec.rows, spec.pitch, dtype=torch.bfloat16, device=gpu)
         src.view(torch.int16).random_(-32768, 32767)
         dst = torch.zeros_like(src)
         torch.cuda.synchronize()
         slot = (spec.view_bytes + 255) // 256 * 256 * spec.views
-        st = pkg.StreamedTransfer(slot_bytes=slot)
+        st = pkg.StreamedTransfer(slot_bytes=slot, streams=2)
         per_chunk = spec.views * spec.parent_elems * 2
         for k in range(chunks):
             st.submit(workloads.pitched_views(src.data_ptr() + k * per_chunk, spec),
                       workloads.pitched_views(dst.data_ptr() + k * per_chunk, spec))
+        assert st._plans is not None and len(st._keep) == chunks     # one pair of plans for the stream
         st.finish()
         s16, d16 = src.view(torch.int16), dst.view(torch.int16)
         assert torch.equal(d16[..., :spec.cols], s16[..., :spec.cols])
         assert int(d16[..., spec.cols:].ne(0).sum()) == 0
         st.close()
         assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+        del src, dst, s16, d16
+        torch.cuda.empty_cache()
+
+
+def test_streamed_transfer_through_the_c_abi(pkg, orc, gpu):
+    """axr_transfer_* with plans the caller keeps: chunks of one geometry at growing
+    deltas, one, two and three lanes, a change of geometry, and the refusals."""
+    import ctypes as C
+    import torch
+    from execution_ucx_amd import workloads
+    lib, capi = pkg._capi.load(), pkg._capi
+    spec = workloads.pitched_chunk(views=4, rows=33, cols=200)
+    chunks = 11
+    per_chunk = spec.views * spec.parent_elems * 2
+    rng = np.random.default_rng(3)
+    src = torch.from_numpy(rng.integers(-2 ** 15, 2 ** 15, size=(chunks, spec.views, spec.rows, spec.pitch),
+                                        dtype=np.int16)).to(gpu).view(torch.bfloat16)
+    send = pkg.BundlePlan.create(workloads.pitched_views(src.data_ptr(), spec), align=256)
+    slot = send.payload_bytes
+    for lanes, streams in ((1, 1), (2, 2), (2, 1), (3, 2)):
+        dst = torch.zeros_like(src)
+        recv = pkg.BundlePlan.from_header(send.header).bind(workloads.pitched_views(dst.data_ptr(), spec))
+        torch.cuda.synchronize()
+        t = C.c_void_p()
+        assert lib.axr_transfer_create(None, slot, lanes, lanes + 1, C.byref(t)) == capi.AXR_ERR_INVALID
+        capi.check(lib.axr_transfer_create(None, slot, lanes, streams, C.byref(t)))
+        # chunks in a scrambled order: deltas need not grow
+        order = [int(k) for k in rng.permutation(chunks)]
+        for k in order:
+            capi.check(lib.axr_transfer_submit(t, send._h, k * per_chunk, recv._h, k * per_chunk))
+        capi.check(lib.axr_transfer_finish(t))
+        s16, d16 = src.view(torch.int16), dst.view(torch.int16)
+        assert torch.equal(d16[..., :spec.cols], s16[..., :spec.cols])
+        assert int(d16[..., spec.cols:].ne(0).sum()) == 0
+        # refusals: a receiver plan of another header; a chunk beyond the slot
+        other = pkg.BundlePlan.create([torch.zeros(64, dtype=torch.uint8, device=gpu)], align=256)
+        assert lib.axr_transfer_submit(t, send._h, 0, other._h, 0) == capi.AXR_ERR_MISMATCH
+        big = torch.zeros(slot + 256, dtype=torch.uint8, device=gpu)
+        bigplan = pkg.BundlePlan.create([big], align=256)
+        bigrecv = pkg.BundlePlan.from_header(bigplan.header).bind([torch.zeros_like(big)])
+        assert lib.axr_transfer_submit(t, bigplan._h, 0, bigrecv._h, 0) == capi.AXR_ERR_LENGTH
+        # another geometry through the same transfer (smaller than a slot)
+        a = torch.from_numpy(rng.integers(0, 256, size=5000, dtype=np.uint8)).to(gpu)
+        b = torch.zeros_like(a)
+        p1 = pkg.BundlePlan.create([a[:3000], a[3000:]], align=1)
+        p2 = pkg.BundlePlan.from_header(p1.header).bind([b[:3000], b[3000:]])
+        torch.cuda.synchronize()
+        capi.check(lib.axr_transfer_submit(t, p1._h, 0, p2._h, 0))
+        capi.check(lib.axr_transfer_finish(t))
+        assert torch.equal(a, b)
+        # an empty bundle is a chunk without a message
+        e1 = pkg.BundlePlan.create([a[:0]], align=1)
+        e2 = pkg.BundlePlan.from_header(e1.header).bind([b[:0]])
+        capi.check(lib.axr_transfer_submit(t, e1._h, 0, e2._h, 0))
+        capi.check(lib.axr_transfer_destroy(t))
+        for p in (recv, other, bigplan, bigrecv, p1, p2, e1, e2):
+            p.close()
+        assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+    send.close()
 
 
 # ------------------------------------------------------------------ checksums, compare

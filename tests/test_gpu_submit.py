@@ -127,6 +127,38 @@ def test_submit_matches_the_oracle_and_separate_calls(pkg, orc, gpu, align):
         capi.check(lib.axr_stream_destroy(stream))
 
 
+def test_payload_cache_hints_move_the_same_bytes(pkg, orc, gpu):
+    """AXR_JOB_PAYLOAD_STREAMING / _CACHED only choose the cache treatment of the payload side."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    rng = np.random.default_rng(12)
+    tensors = random_tensors(rng, gpu, 300, strided_every=6)
+    want = orc.pack([chunk_of(t) for t in tensors], 256)
+    torch.cuda.synchronize()
+    for flags in (0, capi.JOB_PAYLOAD_STREAMING, capi.JOB_PAYLOAD_CACHED):
+        plan = pkg.BundlePlan.create(tensors, align=256)
+        buf = torch.full((plan.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu)
+        outs = zeros_like_views(tensors)
+        rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+        torch.cuda.synchronize()
+        for _ in range(2):          # first launch (tables may ride in the arguments) and a later one
+            arr = (capi.Job * 1)(capi.Job(plan._h, 0, buf.data_ptr(), plan.payload_bytes, 0, flags, 0))
+            capi.check(lib.axr_submit(arr, 1, None))
+            arr = (capi.Job * 1)(capi.Job(rplan._h, 1, buf.data_ptr(), plan.payload_bytes, 0, flags, 0))
+            capi.check(lib.axr_submit(arr, 1, None))
+            torch.cuda.synchronize()
+            got = buf.cpu().numpy()
+            assert np.array_equal(got[:want.size], want) and (got[want.size:] == POISON).all()
+            for a, b in zip(tensors, outs):
+                assert np.array_equal(chunk_of(a), chunk_of(b))
+        arr = (capi.Job * 1)(capi.Job(plan._h, 0, buf.data_ptr(), plan.payload_bytes, 0, 3, 0))
+        assert lib.axr_submit(arr, 1, None) == capi.AXR_ERR_INVALID      # both hints at once
+        arr = (capi.Job * 1)(capi.Job(plan._h, 0, buf.data_ptr(), plan.payload_bytes, 0, 8, 0))
+        assert lib.axr_submit(arr, 1, None) == capi.AXR_ERR_INVALID      # unknown bit
+        plan.close()
+        rplan.close()
+
+
 def test_submit_refusals(pkg, gpu):
     import torch
     lib, capi = pkg._capi.load(), pkg._capi
