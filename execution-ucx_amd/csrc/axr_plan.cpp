@@ -21,6 +21,7 @@
 #include <algorithm>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <new>
 
 #include "axr_internal.h"
@@ -117,6 +118,7 @@ struct axr_plan {
 
   // device tables
   bool tables_built = false;
+  bool device_built = false;         // the device built its tables itself from compact records
   std::vector<Seg> segs;
   std::vector<Dims> dims;
   std::vector<uint32_t> wave_seg;
@@ -148,6 +150,76 @@ struct axr_plan {
 };
 
 namespace {
+
+// Plans of thousands of tensors hold about a megabyte in vectors; fresh ones of that size
+// come from mmap and are paged in on first touch, which costs more than filling them.  A few
+// released plans are therefore kept, emptied, and handed out again with their capacity.
+struct PlanShells {
+  std::mutex mu;
+  std::vector<axr_plan*> idle;
+  ~PlanShells() {
+    for (axr_plan* p : idle) delete p;
+  }
+};
+PlanShells& plan_shells() {
+  static PlanShells shells;
+  return shells;
+}
+constexpr size_t kMaxIdlePlans = 8;
+constexpr size_t kMaxIdlePlanBytes = 16u << 20;
+
+axr_plan* plan_new() {
+  {
+    PlanShells& shells = plan_shells();
+    std::lock_guard<std::mutex> lock(shells.mu);
+    if (!shells.idle.empty()) {
+      axr_plan* p = shells.idle.back();
+      shells.idle.pop_back();
+      return p;
+    }
+  }
+  return new (std::nothrow) axr_plan();
+}
+
+// The plan owns no device resource any more; keeps the vectors' capacity, resets the rest.
+void plan_delete(axr_plan* p) {
+  auto keep = [](auto& v) {
+    v.clear();
+    return v.capacity() * sizeof(v[0]);
+  };
+  std::vector<TensorRec> tensors;
+  std::vector<int64_t> dims64;
+  std::vector<uint8_t> header;
+  std::vector<Seg> segs;
+  std::vector<Dims> dims;
+  std::vector<uint32_t> wave_seg;
+  tensors.swap(p->tensors);
+  dims64.swap(p->dims64);
+  header.swap(p->header);
+  segs.swap(p->segs);
+  dims.swap(p->dims);
+  wave_seg.swap(p->wave_seg);
+  const size_t bytes = keep(tensors) + keep(dims64) + keep(header) + keep(segs) + keep(dims) + keep(wave_seg);
+  if (bytes > kMaxIdlePlanBytes) {
+    delete p;
+    return;
+  }
+  p->~axr_plan();
+  new (p) axr_plan();
+  tensors.swap(p->tensors);
+  dims64.swap(p->dims64);
+  header.swap(p->header);
+  segs.swap(p->segs);
+  dims.swap(p->dims);
+  wave_seg.swap(p->wave_seg);
+  PlanShells& shells = plan_shells();
+  std::lock_guard<std::mutex> lock(shells.mu);
+  if (shells.idle.size() < kMaxIdlePlans) {
+    shells.idle.push_back(p);
+    return;
+  }
+  delete p;   // (under the lock: rare, and the plan is empty)
+}
 
 // False when an offset or the payload size does not fit 64 bits (a crafted header,
 // or a tensor list whose sizes add up past 2^64): nothing is laid out then.
@@ -208,6 +280,7 @@ int check_align(uint32_t align) {
 
 void invalidate_tables(axr_plan* p) {
   p->tables_built = false;
+  p->device_built = false;
   p->uploaded = false;
   p->resident = false;
   p->inline_ready = false;
@@ -520,9 +593,165 @@ struct Builder {
   }
 };
 
+int build_tables(axr_plan* p);
+
+// Launch geometry of a bundle of p->ntiles tiles in nseg segments: one tile per wave until
+// the grid would exceed max_waves, workgroup size, cache hints, and the size of the blocks of
+// the tile-block index (about one segment each, a power of two up to 256 tiles: a bundle of
+// few large tensors gets a tiny index, a bundle of many small ones an entry per few tiles).
+void finish_geometry(axr_plan* p, uint32_t rows, size_t nseg) {
+  const Tunables& tn = tunables();
+  uint64_t tpw = (p->ntiles + static_cast<uint64_t>(tn.max_waves) - 1) /
+                 static_cast<uint64_t>(tn.max_waves);
+  if (tpw == 0) tpw = 1;
+  p->cfg.threads = tn.threads ? static_cast<uint32_t>(tn.threads) : (p->ntiles < 65536 ? 256u : 128u);
+  p->cfg.elements = false;
+  for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode != kModeRunTiles;
+  if (p->cfg.elements) p->cfg.threads = std::min(p->cfg.threads, kMaxElementThreads);
+  if (p->cfg.lds_per_wave) {
+    // transposed blocks: every wave of a workgroup owns a slice of at most 64 KiB of LDS
+    const uint32_t fit = (64u * 1024u / p->cfg.lds_per_wave) * kWaveLanes;
+    p->cfg.threads = std::min(p->cfg.threads, fit);
+  }
+  const uint32_t waves_per_wg = p->cfg.threads / kWaveLanes;
+  const uint64_t per_wg = tpw * waves_per_wg;
+  p->cfg.tiles_per_wave = static_cast<uint32_t>(tpw);
+  p->cfg.workgroups = static_cast<uint32_t>((p->ntiles + per_wg - 1) / per_wg);
+  p->cfg.xcd_remap = tn.xcd_remap != 0 && p->cfg.workgroups >= 4 * kXcds;
+  if (p->cfg.xcd_remap) p->cfg.workgroups = (p->cfg.workgroups + kXcds - 1) / kXcds * kXcds;
+  p->cfg.tile_rows = rows;
+  if (tn.nontemporal < 0) {
+    p->cfg.nontemporal = p->payload_bytes > static_cast<uint64_t>(tn.payload_cache_bytes) ? 3u : 1u;
+  } else {
+    p->cfg.nontemporal = static_cast<uint32_t>(tn.nontemporal) & 3u;
+  }
+  uint32_t shift = 0;
+  while (shift < 8 && (static_cast<uint64_t>(nseg) << (shift + 1)) <= p->ntiles) ++shift;
+  p->cfg.seg_shift = shift;
+}
+
+// Tile rows of a bundle whose tensors are all compact: 2 KiB tiles, doubled while the bundle
+// would exceed max_tiles.
+uint32_t rows_for_compact_bundle(const axr_plan* p) {
+  const Tunables& tn = tunables();
+  uint32_t rows = static_cast<uint32_t>(tn.tile_rows);
+  if (rows) return rows;
+  rows = 2;
+  while (rows < kMaxTileRows &&
+         p->payload_bytes / (static_cast<uint64_t>(rows) * kRowBytes) > static_cast<uint64_t>(tn.max_tiles))
+    rows *= 2;
+  return rows;
+}
+
+bool compact_strides(const int64_t* shape, const int64_t* strides, int32_t ndim) {
+  int64_t expect = 1;
+  for (int32_t d = ndim - 1; d >= 0; --d) {
+    if (shape[d] == 1) continue;
+    if (strides[d] != expect) return false;
+    expect *= shape[d];
+  }
+  return true;
+}
+
+// Bundles of many contiguous device tensors: the host writes one 24-byte record per tensor
+// into pinned memory and a one-workgroup kernel expands them on the device into the segment
+// table and the tile-block index, in front of the bundle kernel on the same stream.  Returns
+// AXR_OK with *done set when the tables are on their way, AXR_OK with *done clear when the
+// bundle does not qualify (the caller builds the tables on the host), or an error.
+int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
+  *done = false;
+  const Tunables& tn = tunables();
+  const size_t n = p->tensors.size();
+  const int64_t least = tn.device_tables;
+  if (least <= 0 || n < static_cast<uint64_t>(least) || n > (1u << 20) || !p->bound) return AXR_OK;
+  const uint32_t rows = rows_for_compact_bundle(p);
+  const uint32_t tile_bytes = rows * kRowBytes;
+  const uint32_t tile_shift = static_cast<uint32_t>(__builtin_ctz(tile_bytes));
+  const uint64_t head_align = static_cast<uint64_t>(tn.head_align);
+  const uint64_t head_mask = head_align > 1 ? head_align - 1 : 0;
+  // room for the index: with blocks of 2^shift tiles, shift < 8 means fewer than 2 n blocks
+  const uint64_t tiles_bound = (p->payload_bytes >> tile_shift) + n;
+  if (tiles_bound > 0xffffffffull) return AXR_OK;
+  const size_t blocks_bound = std::max<size_t>(2 * n + 2, static_cast<size_t>(tiles_bound >> 8) + 2);
+  const size_t wave_at = align_up((n + 1) * sizeof(Seg), 16);
+  const size_t bytes = std::max(wave_at + blocks_bound * sizeof(uint32_t), n * sizeof(CompactRec));
+  if (p->block.host && p->block.bytes < bytes) {
+    quiesce(p);
+    table_block_release(&p->block);
+  }
+  if (!p->block.host) {
+    int rc = table_block_acquire(bytes, &p->block);
+    if (rc) return rc;
+  } else {
+    quiesce(p);   // earlier launches may still read the block
+  }
+  CompactRec* recs = static_cast<CompactRec*>(p->block.host);
+  uint64_t tiles = 0;
+  const bool receiver = p->receiver;
+  for (size_t i = 0; i < n; ++i) {
+    const TensorRec& t = p->tensors[i];
+    if ((t.device_type != kDLROCM && t.device_type != kDLROCMHost) || t.nbytes > kSegRunMask) return AXR_OK;
+    if (t.has_strides && t.nbytes && !compact_strides(p->shape_of(t), p->strides_of(t), t.ndim)) return AXR_OK;
+    recs[i].ptr = t.address;
+    recs[i].off = t.offset;
+    recs[i].nbytes = t.nbytes;
+    if (t.nbytes) {
+      const uint64_t head = (head_mask && t.nbytes > tile_bytes) ? (0 - (receiver ? t.address : t.offset)) & head_mask : 0;
+      tiles += (t.nbytes - head + tile_bytes - 1) >> tile_shift;
+    }
+  }
+  if (tiles == 0 || tiles > 0xffffffffull) return AXR_OK;
+  p->segs.clear();
+  p->dims.clear();
+  p->wave_seg.clear();
+  p->ntiles = static_cast<uint32_t>(tiles);
+  p->cfg.lds_per_wave = 0;
+  finish_geometry(p, rows, n);
+  p->dims_at = wave_at;
+  p->wave_at = wave_at;
+  p->table_bytes = wave_at + ((static_cast<size_t>(p->ntiles) >> p->cfg.seg_shift) + 1) * sizeof(uint32_t);
+  ExpandParams prm;
+  prm.align_mask = static_cast<uint64_t>(p->align) - 1;
+  prm.payload_bytes = p->payload_bytes;
+  prm.tile_shift = tile_shift;
+  prm.seg_shift = p->cfg.seg_shift;
+  prm.head_mask = static_cast<uint32_t>(head_mask);
+  prm.anchor_tensor = receiver ? 1u : 0u;
+  uint8_t* d = static_cast<uint8_t*>(p->block.device);
+  int rc = launch_expand_tables(recs, static_cast<uint32_t>(n), reinterpret_cast<Seg*>(d),
+                                reinterpret_cast<uint32_t*>(d + wave_at), prm, stream);
+  if (rc) return rc;
+  if (!p->upload_event) {
+    rc = check_hip(hipEventCreateWithFlags(&p->upload_event, hipEventDisableTiming), "hipEventCreate");
+    if (rc) return rc;
+  }
+  rc = check_hip(hipEventRecord(p->upload_event, stream), "hipEventRecord");
+  if (rc) return rc;
+  if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
+    p->busy_streams.push_back(stream);
+  p->upload_stream = stream;
+  p->uploaded = true;
+  p->device_built = true;
+  *done = true;
+  return AXR_OK;
+}
+
+// Tables for a launch on `stream`: what is there already, else built by the device when the
+// bundle qualifies and the stream is not capturing, else built on the host.
+int ensure_tables(axr_plan* p, hipStream_t stream, bool capturing) {
+  if (p->tables_built || p->device_built) return AXR_OK;
+  if (!capturing) {
+    bool done = false;
+    int rc = device_build_tables(p, stream, &done);
+    if (rc || done) return rc;
+  }
+  return build_tables(p);
+}
+
 int build_tables(axr_plan* p) {
   if (p->tables_built) return AXR_OK;
   if (!p->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
+  if (p->device_built) quiesce(p);   // the host tables replace the device-built ones at the next launch
   invalidate_tables(p);
   const Tunables& tn = tunables();
   uint32_t rows = static_cast<uint32_t>(tn.tile_rows);
@@ -534,6 +763,10 @@ int build_tables(axr_plan* p) {
     bool uniform_runs = !p->tensors.empty();
     for (const TensorRec& t : p->tensors) {
       if (t.nbytes == 0) continue;
+      if (!t.has_strides) {   // a compact tensor: not a bundle of strided views
+        uniform_runs = false;
+        break;
+      }
       const uint64_t item = (static_cast<uint64_t>(t.bits) + 7) / 8;
       Collapsed c;
       collapse(t, p->shape_of(t), p->strides_of(t), item, &c);
@@ -569,7 +802,12 @@ int build_tables(axr_plan* p) {
         if (strides[d] == 0 && shape[d] > 1) p->overlapping_dst = true;
     }
     Collapsed c;
-    collapse(t, shape, strides, item, &c);
+    if (!strides) {   // compact by definition: one run, nothing to collapse
+      c.nd = 0;
+      c.run_bytes = t.nbytes;
+    } else {
+      collapse(t, shape, strides, item, &c);
+    }
     int rc;
     if (t.device_type == kDLROCM || t.device_type == kDLROCMHost) {
       rc = b.add_strided(static_cast<uint32_t>(i), t.address, t.offset, c.extent, c.stride, c.nd,
@@ -614,40 +852,14 @@ int build_tables(axr_plan* p) {
   sentinel.tile_begin = p->ntiles;
   p->segs.push_back(sentinel);
 
-  // launch geometry: one tile per wave until the grid would exceed max_waves
-  uint64_t tpw = (p->ntiles + static_cast<uint64_t>(tn.max_waves) - 1) /
-                 static_cast<uint64_t>(tn.max_waves);
-  if (tpw == 0) tpw = 1;
-  p->cfg.threads = tn.threads ? static_cast<uint32_t>(tn.threads) : (p->ntiles < 65536 ? 256u : 128u);
-  p->cfg.elements = false;
-  for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode != kModeRunTiles;
-  if (p->cfg.elements) p->cfg.threads = std::min(p->cfg.threads, kMaxElementThreads);
-  if (p->cfg.lds_per_wave) {
-    // transposed blocks: every wave of a workgroup owns a slice of at most 64 KiB of LDS
-    const uint32_t fit = (64u * 1024u / p->cfg.lds_per_wave) * kWaveLanes;
-    p->cfg.threads = std::min(p->cfg.threads, fit);
-  }
-  const uint32_t waves_per_wg = p->cfg.threads / kWaveLanes;
-  const uint64_t per_wg = tpw * waves_per_wg;
-  p->cfg.tiles_per_wave = static_cast<uint32_t>(tpw);
-  p->cfg.workgroups = static_cast<uint32_t>((p->ntiles + per_wg - 1) / per_wg);
-  p->cfg.xcd_remap = tn.xcd_remap != 0 && p->cfg.workgroups >= 4 * kXcds;
-  if (p->cfg.xcd_remap) p->cfg.workgroups = (p->cfg.workgroups + kXcds - 1) / kXcds * kXcds;
-  p->cfg.tile_rows = rows;
-  if (tn.nontemporal < 0) {
-    p->cfg.nontemporal = p->payload_bytes > static_cast<uint64_t>(tn.payload_cache_bytes) ? 3u : 1u;
-  } else {
-    p->cfg.nontemporal = static_cast<uint32_t>(tn.nontemporal) & 3u;
-  }
+  const size_t nseg = p->segs.size() - 1;
+  finish_geometry(p, rows, nseg);
 
   // Tile-block index: entry k = segment that holds tile k << seg_shift.  Blocks
   // are sized to about one segment each (a power of two, at most 256 tiles), so
   // a bundle of few large tensors gets a tiny index and a bundle of many small
   // ones one entry per few tiles; a wave walks at most a segment or two forward.
-  const size_t nseg = p->segs.size() - 1;
-  uint32_t shift = 0;
-  while (shift < 8 && (static_cast<uint64_t>(nseg) << (shift + 1)) <= p->ntiles) ++shift;
-  p->cfg.seg_shift = shift;
+  const uint32_t shift = p->cfg.seg_shift;
   const size_t nblocks = (static_cast<size_t>(p->ntiles) >> shift) + 1;
   p->wave_seg.assign(nblocks, 0);
   size_t s = 0;
@@ -792,7 +1004,7 @@ int move_host_tensors(axr_plan* p, bool pack, uint8_t* payload, hipStream_t stre
 // kernel arguments (3.5 KiB at most) instead of a device block.
 bool tables_fit_kernel_arguments(const axr_plan* p) {
   const int64_t limit = tunables().inline_tables;
-  return limit > 0 && p->ntiles <= static_cast<uint64_t>(limit) &&
+  return limit > 0 && p->tables_built && p->ntiles <= static_cast<uint64_t>(limit) &&
          p->table_bytes + kInlineTablesHead <= kInlineTableBytes && p->cfg.tile_rows == 2 &&
          (p->cfg.nontemporal & 3u) == 1u && !p->cfg.xcd_remap;
 }
@@ -825,20 +1037,21 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
     return fail(AXR_ERR_LENGTH, "payload buffer is smaller than the plan's payload");
   if (p->payload_bytes == 0) return AXR_OK;
   if (!payload) return fail(AXR_ERR_INVALID, "null payload");
-  int rc = build_tables(p);
-  if (rc) return rc;
-  if (!pack && p->overlapping_dst)
-    return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   // Under stream capture only the kernel launch may be recorded: the tables must be
   // resident already (axr_plan_prepare) and nothing may wait on the host.
   bool capturing = false;
+  int rc = AXR_OK;
   if (stream) {
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
     rc = check_hip(hipStreamIsCapturing(stream, &status), "hipStreamIsCapturing");
     if (rc) return rc;
     capturing = status == hipStreamCaptureStatusActive;
   }
+  rc = ensure_tables(p, stream, capturing);
+  if (rc) return rc;
+  if (!pack && p->overlapping_dst)
+    return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
   if (capturing) {
     if (!p->host_chunks.empty())
       return fail(AXR_ERR_UNSUPPORTED, "a bundle with host (kDLCPU) tensors cannot be captured in a graph");
@@ -854,7 +1067,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   if (p->ntiles == 0) return AXR_OK;
   KernelArgs a;
   a.payload = static_cast<uint8_t*>(payload);
-  a.nseg = static_cast<uint32_t>(p->segs.size() - 1);
+  a.nseg = p->segs.empty() ? 0u : static_cast<uint32_t>(p->segs.size() - 1);
   a.ntiles = p->ntiles;
   a.tiles_per_wave = p->cfg.tiles_per_wave;
   a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
@@ -947,7 +1160,7 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   if (flags != 0) return fail(AXR_ERR_INVALID, "axr_plan_create: flags are reserved and must be 0");
   int rc = check_align(align);
   if (rc) return rc;
-  axr_plan* p = new (std::nothrow) axr_plan();
+  axr_plan* p = plan_new();
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_create: out of host memory");
   p->align = align;
   p->tensors.resize(n);
@@ -958,12 +1171,12 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   for (size_t i = 0; i < n; ++i) {
     rc = store_tensor(p, tensors[i], &p->tensors[i]);
     if (rc) {
-      delete p;
+      plan_delete(p);
       return rc;
     }
   }
   if (!compute_layout(p)) {
-    delete p;
+    plan_delete(p);
     return fail(AXR_ERR_INVALID, "axr_plan_create: bundle size overflows 64 bits");
   }
   encode_header(p);
@@ -989,7 +1202,7 @@ static int plan_free_body(axr_plan_t* plan) {
     table_block_release(&st.block);
     if (st.ready) (void)hipEventDestroy(st.ready);
   }
-  delete plan;
+  plan_delete(plan);
   return AXR_OK;
 }
 int axr_plan_free(axr_plan_t* plan) {
@@ -1080,7 +1293,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   if (check_align(align) != AXR_OK) return fail(AXR_ERR_HEADER, "bundle header has a bad alignment");
   if (static_cast<uint64_t>(n) * kTensorHeader > length - kFixedHeader)
     return fail(AXR_ERR_HEADER, "bundle header truncated");
-  axr_plan* p = new (std::nothrow) axr_plan();
+  axr_plan* p = plan_new();
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_from_header: out of host memory");
   p->align = align;
   p->tensors.resize(n);
@@ -1088,7 +1301,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   size_t at = kFixedHeader;
   for (uint32_t i = 0; i < n; ++i) {
     if (length - at < kTensorHeader) {
-      delete p;
+      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header truncated");
     }
     TensorRec& t = p->tensors[i];
@@ -1104,7 +1317,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
     at += kTensorHeader;
     if (t.ndim < 0 || t.ndim > kMaxNdim ||
         static_cast<size_t>(t.ndim) * 8 > length - at || byte_offset != 0) {
-      delete p;
+      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header has a bad tensor record");
     }
     t.shape_at = p->dims64.size();
@@ -1112,14 +1325,14 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
     at += static_cast<size_t>(t.ndim) * 8;
     uint64_t rule = 0;
     if (nbytes_rule(t.ndim, p->dims64.data() + t.shape_at, t.bits, &rule) != AXR_OK || rule != nb) {
-      delete p;
+      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header tensor size does not follow from its shape");
     }
     t.nbytes = nb;
     t.offset = off;   // checked against the layout rule below
   }
   if (at != length) {
-    delete p;
+    plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header has trailing bytes");
   }
   std::vector<uint64_t> sent(n);
@@ -1127,7 +1340,7 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   bool ok = compute_layout(p) && p->payload_bytes == payload;
   for (uint32_t i = 0; i < n && ok; ++i) ok = sent[i] == p->tensors[i].offset;
   if (!ok) {
-    delete p;
+    plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header offsets do not follow the layout rule");
   }
   p->header.assign(h, h + length);
@@ -1322,7 +1535,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     if (p->payload_bytes && !j.payload) return fail(AXR_ERR_INVALID, "null payload");
     for (size_t k = 0; k < i; ++k)
       if (jobs[k].plan == p) return fail(AXR_ERR_INVALID, "axr_submit: one plan appears in two jobs");
-    int rc = build_tables(p);
+    int rc = ensure_tables(p, stream, capturing);
     if (rc) return rc;
     if (j.unpack && p->overlapping_dst)
       return fail(AXR_ERR_INVALID, "unpack destination has overlapping elements (zero stride)");
@@ -1436,10 +1649,10 @@ static int plan_launch_info_body(axr_plan_t* plan, axr_launch_info_t* info) {
 static int plan_prepare_body(axr_plan_t* plan, void* stream_) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_prepare: null plan");
   if (!plan->bound) return fail(AXR_ERR_INVALID, "plan has no tensor addresses bound");
-  int rc = build_tables(plan);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  int rc = ensure_tables(plan, stream, false);
   if (rc) return rc;
   if (plan->ntiles == 0 || plan->resident) return AXR_OK;
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
   rc = ensure_uploaded(plan, stream);
   if (rc) return rc;
   rc = check_hip(hipEventSynchronize(plan->upload_event), "hipEventSynchronize(plan tables)");

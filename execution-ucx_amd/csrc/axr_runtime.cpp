@@ -409,6 +409,9 @@ static int tune_set_body(const char* key, int64_t value) {
     t.inline_tables = value;
   } else if (k == "transpose") {
     t.transpose = value ? 1 : 0;
+  } else if (k == "device_tables") {
+    if (value < 0) return fail(AXR_ERR_INVALID, "device_tables must not be negative");
+    t.device_tables = value;
   } else if (k == "loopback_copy_kernel") {
     t.loopback_copy_kernel = value ? 1 : 0;
   } else if (k == "head_align") {
@@ -442,6 +445,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "host_threads") *value = t.host_threads;
   else if (k == "head_align") *value = t.head_align;
   else if (k == "loopback_copy_kernel") *value = t.loopback_copy_kernel;
+  else if (k == "device_tables") *value = t.device_tables;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

@@ -413,6 +413,10 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "host_threads" (threads, the caller included, that share the host-side copies
  * between pageable memory and the pinned staging blocks once a copy is 2 MiB or
  * more; default 4, 1: the calling thread alone),
+ * "device_tables" (a bundle of at least this many tensors, all contiguous device
+ * tensors, gets its device tables from a small kernel that expands one 24-byte
+ * record per tensor, instead of tables built on the host and uploaded; default 512,
+ * 0: never),
  * "loopback_copy_kernel" (1, default: the loopback context moves a device payload
  * to device memory with the library's copy kernel; 0: with hipMemcpyAsync),
  * "inline_tables" (the first launch of a bundle of at most this many tiles

@@ -294,3 +294,75 @@ def test_head_peel_every_misalignment(pkg, orc, gpu, head_align):
                     p.close()
     finally:
         pkg.tune(head_align=before.value)
+
+
+@pytest.mark.parametrize("align", [1, 256])
+def test_tables_built_on_the_device_match_the_oracle(pkg, orc, gpu, align):
+    """Bundles of contiguous device tensors whose tables a kernel expands from one record per
+    tensor ("device_tables"): every count from one tensor to several per thread of the
+    expanding workgroup, empty tensors in between, tensors of many thousand tiles, odd
+    addresses; packed bytes against the oracle, unpack round trip, and the same plans with
+    host-built tables."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    before = C.c_int64()
+    capi.check(lib.axr_tune_get(b"device_tables", C.byref(before)))
+    rng = np.random.default_rng(99 + align)
+    arena = torch.from_numpy(rng.integers(0, 256, size=96 << 20, dtype=np.uint8)).to(gpu)
+    cases = []
+    for count, lo, hi in ((1, 5000, 5001), (3, 1, 40), (70, 1, 9000), (1023, 1, 3000), (1025, 1, 3000),
+                          (2500, 1, 12000), (5, 3 << 20, 9 << 20), (40, 1, 1 << 20)):
+        views, at = [], int(rng.integers(0, 64))
+        for k in range(count):
+            n = 0 if (count > 3 and k % 17 == 5) else int(rng.integers(lo, hi))
+            at += int(rng.integers(0, 130))
+            views.append(arena[at:at + n])
+            at += n
+        assert at <= arena.numel()
+        cases.append(views)
+    try:
+        for views in cases:
+            want = orc.pack([chunk_of(v) for v in views], align)
+            for device_tables in (1, 0):
+                pkg.tune(device_tables=device_tables)
+                plan = pkg.BundlePlan.create(views, align=align)
+                n = plan.payload_bytes
+                buf = torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu)
+                for _ in range(2):      # the second launch reuses the tables
+                    plan.pack(buf.data_ptr(), n)
+                torch.cuda.synchronize()
+                got = buf.cpu().numpy()
+                assert np.array_equal(got[:n], want), (len(views), device_tables)
+                assert (got[n:] == POISON).all()
+                out_arena = torch.full_like(arena, POISON)
+                outs = [out_arena[v.data_ptr() - arena.data_ptr():][:v.numel()] for v in views]
+                rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+                rplan.unpack(buf.data_ptr(), n)
+                torch.cuda.synchronize()
+                mask = torch.zeros_like(arena, dtype=torch.bool)
+                for v in views:
+                    o = v.data_ptr() - arena.data_ptr()
+                    mask[o:o + v.numel()] = True
+                assert torch.equal(out_arena[mask], arena[mask])
+                assert bool((out_arena[~mask] == POISON).all())
+                # asking for the tables on the host afterwards gives the same launch geometry
+                # and the next launch still moves the same bytes
+                info = plan.launch_info()
+                assert info["tiles"] > 0 or n == 0
+                buf.fill_(POISON)
+                plan.pack(buf.data_ptr(), n)
+                torch.cuda.synchronize()
+                assert np.array_equal(buf.cpu().numpy()[:n], want)
+                plan.close()
+                rplan.close()
+        # a strided view among them: the host builds the tables, same result
+        pkg.tune(device_tables=1)
+        mixed = cases[2][:20] + [arena[:4096].view(torch.int16).reshape(32, 64)[:, :20]] + cases[2][20:40]
+        plan = pkg.BundlePlan.create(mixed, align=align)
+        buf = torch.full((plan.payload_bytes,), POISON, dtype=torch.uint8, device=gpu)
+        plan.pack(buf.data_ptr(), plan.payload_bytes)
+        torch.cuda.synchronize()
+        assert np.array_equal(buf.cpu().numpy(), orc.pack([chunk_of(v) for v in mixed], align))
+        plan.close()
+    finally:
+        pkg.tune(device_tables=before.value)
