@@ -133,21 +133,6 @@ struct alignas(16) InlineTables {
   uint8_t bytes[kInlineTableBytes];
 };
 
-// What the host writes per tensor when the device builds the tables itself (bundles of
-// contiguous device tensors): expand_tables_kernel turns n of these into Seg[n + 1] and the
-// tile-block index.
-struct CompactRec {
-  uint64_t ptr, off, nbytes;
-};
-struct ExpandParams {
-  uint64_t align_mask;      // bundle alignment - 1
-  uint64_t payload_bytes;
-  uint32_t tile_shift;      // log2 of the tile size in bytes
-  uint32_t seg_shift;
-  uint32_t head_mask;       // head_align - 1, 0 when no head is peeled
-  uint32_t anchor_tensor;   // heads line up the tensor side (a receiver's plan), else the payload side
-};
-
 struct LaunchConfig {
   uint32_t workgroups = 0;
   uint32_t tiles_per_wave = 0;
@@ -197,8 +182,9 @@ struct Tunables {
   // The loopback transport moves a device payload to device memory of the same GPU with the
   // library's copy kernel (1) or with hipMemcpyAsync (0).
   std::atomic<int64_t> loopback_copy_kernel{1};
-  // Bundles of at least this many tensors, all of them contiguous device tensors, have their
-  // tables built by a kernel from 24-byte records (0: the host always builds them).
+  // Bundles of at least this many tensors, all of them contiguous device tensors, get their
+  // tables in one pass over the tensors into pinned memory plus a kernel that brings them to
+  // the device and writes the tile-block index (0: the general host path always).
   std::atomic<int64_t> device_tables{512};
   std::atomic<int64_t> host_threads{4};       // threads (the caller included) for host-side staging copies
   std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
@@ -251,9 +237,10 @@ int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchC
 // hints; cfg.workgroups is the whole grid, cfg.lds_per_wave the largest need of any job).
 int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stream);
 int launch_fill(void* dst, int value, size_t bytes, void* stream);
-// recs is device-accessible (pinned host memory will do); segs and wave_seg are device memory.
-int launch_expand_tables(const CompactRec* recs, uint32_t n, Seg* segs, uint32_t* wave_seg,
-                         const ExpandParams& prm, void* stream);
+// staged: n + 1 segment records in device-accessible memory (pinned host memory will do);
+// segs and wave_seg are device memory.  Copies the records and writes the tile-block index.
+int launch_expand_tables(const Seg* staged, uint32_t n, Seg* segs, uint32_t* wave_seg, uint32_t seg_shift,
+                         void* stream);
 // dst[0, bytes) = src[0, bytes), both in device memory of the current device, no alignment needed.
 int launch_stream_copy(void* dst, const void* src, size_t bytes, bool nontemporal, void* stream);
 // Device address, on the current device, of the kStaticTableBytes bytes that hold the

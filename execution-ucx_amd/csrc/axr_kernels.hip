@@ -1010,71 +1010,23 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
   for (size_t i = tid; i < nvec; i += nthreads) dst[i] = src[i];
 }
 
-// Device-side construction of the tables of a bundle of contiguous device tensors, so that
-// the host only writes one 24-byte record per tensor.  One workgroup: every thread takes a
-// run of consecutive tensors, counts their tiles, the workgroup scans the counts, and each
-// thread writes its tensors' Seg entries and the tile-block index entries that fall into
-// them.  Tensors without bytes become segments without tiles, which the bundle kernel's
-// walk steps over.
-__global__ __launch_bounds__(1024) void expand_tables_kernel(const CompactRec* recs, uint32_t n, Seg* segs,
-                                                             uint32_t* wave_seg, ExpandParams prm) {
-  __shared__ uint32_t wave_total[16];
-  const uint32_t tid = threadIdx.x;
-  const uint32_t per = (n + blockDim.x - 1) / blockDim.x;
-  const uint32_t begin = tid * per < n ? tid * per : n;
-  const uint32_t end = begin + per < n ? begin + per : n;
-  const uint64_t tile = 1ull << prm.tile_shift;
-  auto head_of = [&](const CompactRec& r) -> uint64_t {
-    if (prm.head_mask == 0 || r.nbytes <= tile) return 0;
-    return (0 - (prm.anchor_tensor ? r.ptr : r.off)) & prm.head_mask;
-  };
-  uint32_t mine = 0;
-  for (uint32_t i = begin; i < end; ++i) {
-    const CompactRec r = recs[i];
-    if (r.nbytes) mine += static_cast<uint32_t>((r.nbytes - head_of(r) + tile - 1) >> prm.tile_shift);
-  }
-  // exclusive scan of `mine` over the workgroup: within the wavefront, then over wavefronts
-  uint32_t incl = mine;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint32_t up = __shfl_up(incl, d, 64);
-    if ((tid & 63u) >= static_cast<uint32_t>(d)) incl += up;
-  }
-  if ((tid & 63u) == 63u) wave_total[tid >> 6] = incl;
-  __syncthreads();
-  uint32_t base = 0;
-  for (uint32_t w = 0; w < (tid >> 6); ++w) base += wave_total[w];
-  uint32_t t = base + incl - mine;
-  for (uint32_t i = begin; i < end; ++i) {
-    const CompactRec r = recs[i];
-    const uint64_t head = head_of(r);
-    const uint32_t tiles = r.nbytes ? static_cast<uint32_t>((r.nbytes - head + tile - 1) >> prm.tile_shift) : 0u;
-    const uint64_t stop = r.off + r.nbytes;
-    uint64_t padded = (stop + prm.align_mask) & ~prm.align_mask;
-    if (padded > prm.payload_bytes) padded = prm.payload_bytes;
-    Seg sg;
-    sg.ptr = r.ptr;
-    sg.off = r.off;
-    sg.run_bytes = r.nbytes | (head << kSegHeadShift);
-    sg.tile_begin = t;
-    sg.meta = r.nbytes ? static_cast<uint32_t>(padded - stop) : 0u;
-    segs[i] = sg;
-    // index entries k with t <= (k << seg_shift) < t + tiles
-    const uint32_t step = 1u << prm.seg_shift;
-    for (uint64_t k = (static_cast<uint64_t>(t) + step - 1) >> prm.seg_shift;
-         (k << prm.seg_shift) < static_cast<uint64_t>(t) + tiles; ++k)
-      wave_seg[k] = i;
-    t += tiles;
-  }
-  if (tid == blockDim.x - 1) {   // holds the grand total
-    Seg sentinel;
-    sentinel.ptr = 0;
-    sentinel.off = 0;
-    sentinel.run_bytes = 0;
-    sentinel.tile_begin = t;
-    sentinel.meta = 0;
-    segs[n] = sentinel;
-  }
+// Tables of a bundle of contiguous device tensors.  The host writes the n + 1 segment
+// records (one pass over the tensors, straight into pinned memory); this kernel, one thread
+// per segment, brings them into device memory and writes the entries of the tile-block index
+// that fall into each segment, so that the host neither builds the index nor waits for a copy
+// engine.  Tensors without bytes are segments without tiles, which the bundle kernel's walk
+// steps over.
+__global__ __launch_bounds__(256) void expand_tables_kernel(const Seg* staged, uint32_t n, Seg* segs,
+                                                            uint32_t* wave_seg, uint32_t seg_shift) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i > n) return;
+  const Seg sg = staged[i];
+  segs[i] = sg;
+  if (i == n) return;   // the sentinel
+  const uint64_t first = sg.tile_begin, last = staged[i + 1].tile_begin;
+  // index entries k with first <= (k << seg_shift) < last
+  const uint64_t step = 1ull << seg_shift;
+  for (uint64_t k = (first + step - 1) >> seg_shift; (k << seg_shift) < last; ++k) wave_seg[k] = i;
 }
 
 // One contiguous range, 2 KiB per wavefront with the same tile copy as the bundle
@@ -1273,11 +1225,10 @@ int static_table_area(void** ptr) {
   return AXR_OK;
 }
 
-int launch_expand_tables(const CompactRec* recs, uint32_t n, Seg* segs, uint32_t* wave_seg,
-                         const ExpandParams& prm, void* stream) {
-  if (n == 0) return AXR_OK;
-  hipLaunchKernelGGL(expand_tables_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), recs, n,
-                     segs, wave_seg, prm);
+int launch_expand_tables(const Seg* staged, uint32_t n, Seg* segs, uint32_t* wave_seg, uint32_t seg_shift,
+                         void* stream) {
+  hipLaunchKernelGGL(expand_tables_kernel, dim3((n + 1 + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), staged, n, segs, wave_seg, seg_shift);
   return check_hip(hipGetLastError(), "table expansion launch");
 }
 

@@ -37,15 +37,15 @@ constexpr size_t kTensorHeader = 40;
 constexpr int32_t kDLCPU = 1, kDLROCM = 10, kDLROCMHost = 11;
 constexpr int kMaxNdim = 64;
 
-struct TensorRec {
+struct TensorRec {          // 56 bytes
+  uint64_t address = 0;     // data + byte_offset, 0 when unbound
+  uint64_t offset = 0, nbytes = 0;
+  uint32_t shape_at = 0;    // index into plan->dims64
+  uint32_t strides_at = 0;
   int32_t device_type = 0, device_id = 0, ndim = 0;
   uint8_t code = 0, bits = 0;
   uint16_t lanes = 0;
-  size_t shape_at = 0;      // index into plan->dims64
   bool has_strides = false;
-  size_t strides_at = 0;
-  uint64_t address = 0;     // data + byte_offset, 0 when unbound
-  uint64_t offset = 0, nbytes = 0;
 };
 
 struct HostCopy {
@@ -81,13 +81,17 @@ bool mul_overflow(uint64_t a, uint64_t b, uint64_t* out) {
   return __builtin_mul_overflow(a, b, out);
 }
 
-int nbytes_rule(int32_t ndim, const int64_t* shape, uint8_t bits, uint64_t* out) {
+inline int nbytes_rule(int32_t ndim, const int64_t* shape, uint8_t bits, uint64_t* out) {
   if (ndim == 0) {   // the reference sizes a 0-d tensor as 0 bytes
     *out = 0;
     return AXR_OK;
   }
   if (ndim < 0 || ndim > kMaxNdim) return fail(AXR_ERR_INVALID, "tensor ndim out of range");
   if (!shape) return fail(AXR_ERR_INVALID, "tensor shape is null for ndim > 0");
+  if (ndim == 1 && shape[0] >= 0 && shape[0] < (int64_t(1) << 56)) {   // the common case, no overflow possible
+    *out = static_cast<uint64_t>(shape[0]) * ((static_cast<uint64_t>(bits) + 7) / 8);
+    return AXR_OK;
+  }
   uint64_t elems = 1;
   for (int32_t i = 0; i < ndim; ++i) {
     if (shape[i] < 0) return fail(AXR_ERR_INVALID, "negative tensor extent");
@@ -111,6 +115,8 @@ struct axr_plan {
   uint32_t align = 1;
   std::vector<TensorRec> tensors;
   std::vector<int64_t> dims64;       // shapes and strides of all tensors
+  std::vector<TensorRec> staged_tensors;   // axr_plan_bind fills these and swaps on success
+  std::vector<int64_t> staged_dims64;
   uint64_t payload_bytes = 0, data_bytes = 0;
   std::vector<uint8_t> header;
   bool bound = false;
@@ -187,19 +193,22 @@ void plan_delete(axr_plan* p) {
     v.clear();
     return v.capacity() * sizeof(v[0]);
   };
-  std::vector<TensorRec> tensors;
-  std::vector<int64_t> dims64;
+  std::vector<TensorRec> tensors, tensors2;
+  std::vector<int64_t> dims64, dims64_2;
   std::vector<uint8_t> header;
   std::vector<Seg> segs;
   std::vector<Dims> dims;
   std::vector<uint32_t> wave_seg;
   tensors.swap(p->tensors);
   dims64.swap(p->dims64);
+  tensors2.swap(p->staged_tensors);
+  dims64_2.swap(p->staged_dims64);
   header.swap(p->header);
   segs.swap(p->segs);
   dims.swap(p->dims);
   wave_seg.swap(p->wave_seg);
-  const size_t bytes = keep(tensors) + keep(dims64) + keep(header) + keep(segs) + keep(dims) + keep(wave_seg);
+  const size_t bytes = keep(tensors) + keep(dims64) + keep(header) + keep(segs) + keep(dims) + keep(wave_seg) +
+                       keep(tensors2) + keep(dims64_2);
   if (bytes > kMaxIdlePlanBytes) {
     delete p;
     return;
@@ -208,6 +217,8 @@ void plan_delete(axr_plan* p) {
   new (p) axr_plan();
   tensors.swap(p->tensors);
   dims64.swap(p->dims64);
+  tensors2.swap(p->staged_tensors);
+  dims64_2.swap(p->staged_dims64);
   header.swap(p->header);
   segs.swap(p->segs);
   dims.swap(p->dims);
@@ -221,55 +232,29 @@ void plan_delete(axr_plan* p) {
   delete p;   // (under the lock: rare, and the plan is empty)
 }
 
-// False when an offset or the payload size does not fit 64 bits (a crafted header,
-// or a tensor list whose sizes add up past 2^64): nothing is laid out then.
-bool compute_layout(axr_plan* p) {
-  uint64_t off = 0, data = 0, end = 0;
-  const uint64_t mask = static_cast<uint64_t>(p->align) - 1;
-  for (auto& t : p->tensors) {
-    if (__builtin_add_overflow(off, mask, &off)) return false;
-    off &= ~mask;
-    t.offset = off;
-    if (__builtin_add_overflow(off, t.nbytes, &off)) return false;
-    end = off;
-    data += t.nbytes;   // at most `off`, which did not overflow
-  }
-  p->payload_bytes = end;
-  p->data_bytes = data;
-  return true;
-}
+// One tensor's record of the header, as it lies on the wire (little-endian targets only).
+#pragma pack(push, 1)
+struct WireTensor {
+  uint64_t offset, nbytes;
+  int32_t device_type, device_id, ndim;
+  uint8_t code, bits;
+  uint16_t lanes;
+  uint64_t byte_offset;
+};
+#pragma pack(pop)
+static_assert(sizeof(WireTensor) == kTensorHeader, "header record layout");
 
-void encode_header(axr_plan* p) {
-  size_t total = kFixedHeader;
-  for (const auto& t : p->tensors) total += kTensorHeader + 8 * static_cast<size_t>(t.ndim);
-  std::vector<uint8_t>& h = p->header;
-  h.resize(total);
-  uint8_t* w = h.data();
-  auto emit = [&w](const void* src, size_t n) {   // targets are little-endian (x86-64, gfx950)
-    std::memcpy(w, src, n);
-    w += n;
-  };
+// The fixed part of the header; the per-tensor records are written while the tensors are read.
+void encode_preamble(axr_plan* p) {
+  uint8_t* w = p->header.data();
   const uint32_t magic = kMagic, n = static_cast<uint32_t>(p->tensors.size()), align = p->align;
   const uint16_t version = kVersion, flags = 0;
-  emit(&magic, 4);
-  emit(&version, 2);
-  emit(&flags, 2);
-  emit(&n, 4);
-  emit(&align, 4);
-  emit(&p->payload_bytes, 8);
-  const uint64_t zero = 0;   // byte_offset: the packed copy starts at its offset
-  for (const auto& t : p->tensors) {
-    emit(&t.offset, 8);
-    emit(&t.nbytes, 8);
-    emit(&t.device_type, 4);
-    emit(&t.device_id, 4);
-    emit(&t.ndim, 4);
-    emit(&t.code, 1);
-    emit(&t.bits, 1);
-    emit(&t.lanes, 2);
-    emit(&zero, 8);
-    if (t.ndim) emit(p->shape_of(t), 8 * static_cast<size_t>(t.ndim));
-  }
+  std::memcpy(w, &magic, 4);
+  std::memcpy(w + 4, &version, 2);
+  std::memcpy(w + 6, &flags, 2);
+  std::memcpy(w + 8, &n, 4);
+  std::memcpy(w + 12, &align, 4);
+  std::memcpy(w + 16, &p->payload_bytes, 8);
 }
 
 int check_align(uint32_t align) {
@@ -653,11 +638,12 @@ bool compact_strides(const int64_t* shape, const int64_t* strides, int32_t ndim)
   return true;
 }
 
-// Bundles of many contiguous device tensors: the host writes one 24-byte record per tensor
-// into pinned memory and a one-workgroup kernel expands them on the device into the segment
-// table and the tile-block index, in front of the bundle kernel on the same stream.  Returns
-// AXR_OK with *done set when the tables are on their way, AXR_OK with *done clear when the
-// bundle does not qualify (the caller builds the tables on the host), or an error.
+// Bundles of many contiguous device tensors: one pass over the tensors writes the segment
+// records straight into pinned memory, and a kernel (one thread per segment) brings them to
+// the device and writes the tile-block index, in front of the bundle kernel on the same
+// stream: no strides to collapse, no index built on the host, no copy engine to wait for.
+// Returns AXR_OK with *done set when the tables are on their way, AXR_OK with *done clear when
+// the bundle does not qualify (the caller takes the general path), or an error.
 int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   *done = false;
   const Tunables& tn = tunables();
@@ -674,7 +660,7 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   if (tiles_bound > 0xffffffffull) return AXR_OK;
   const size_t blocks_bound = std::max<size_t>(2 * n + 2, static_cast<size_t>(tiles_bound >> 8) + 2);
   const size_t wave_at = align_up((n + 1) * sizeof(Seg), 16);
-  const size_t bytes = std::max(wave_at + blocks_bound * sizeof(uint32_t), n * sizeof(CompactRec));
+  const size_t bytes = wave_at + blocks_bound * sizeof(uint32_t);
   if (p->block.host && p->block.bytes < bytes) {
     quiesce(p);
     table_block_release(&p->block);
@@ -685,22 +671,33 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   } else {
     quiesce(p);   // earlier launches may still read the block
   }
-  CompactRec* recs = static_cast<CompactRec*>(p->block.host);
+  Seg* staged = static_cast<Seg*>(p->block.host);
   uint64_t tiles = 0;
   const bool receiver = p->receiver;
+  const uint64_t align_mask = static_cast<uint64_t>(p->align) - 1;
   for (size_t i = 0; i < n; ++i) {
     const TensorRec& t = p->tensors[i];
     if ((t.device_type != kDLROCM && t.device_type != kDLROCMHost) || t.nbytes > kSegRunMask) return AXR_OK;
     if (t.has_strides && t.nbytes && !compact_strides(p->shape_of(t), p->strides_of(t), t.ndim)) return AXR_OK;
-    recs[i].ptr = t.address;
-    recs[i].off = t.offset;
-    recs[i].nbytes = t.nbytes;
+    Seg& sg = staged[i];
+    sg.ptr = t.address;
+    sg.off = t.offset;
+    sg.tile_begin = static_cast<uint32_t>(tiles);
     if (t.nbytes) {
-      const uint64_t head = (head_mask && t.nbytes > tile_bytes) ? (0 - (receiver ? t.address : t.offset)) & head_mask : 0;
+      const uint64_t head =
+          (head_mask && t.nbytes > tile_bytes) ? (0 - (receiver ? t.address : t.offset)) & head_mask : 0;
+      const uint64_t stop = t.offset + t.nbytes;
+      sg.run_bytes = t.nbytes | (head << kSegHeadShift);
+      sg.meta = static_cast<uint32_t>(std::min((stop + align_mask) & ~align_mask, p->payload_bytes) - stop);
       tiles += (t.nbytes - head + tile_bytes - 1) >> tile_shift;
+    } else {
+      sg.run_bytes = 0;
+      sg.meta = 0;
     }
   }
   if (tiles == 0 || tiles > 0xffffffffull) return AXR_OK;
+  std::memset(&staged[n], 0, sizeof(Seg));
+  staged[n].tile_begin = static_cast<uint32_t>(tiles);
   p->segs.clear();
   p->dims.clear();
   p->wave_seg.clear();
@@ -710,16 +707,9 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   p->dims_at = wave_at;
   p->wave_at = wave_at;
   p->table_bytes = wave_at + ((static_cast<size_t>(p->ntiles) >> p->cfg.seg_shift) + 1) * sizeof(uint32_t);
-  ExpandParams prm;
-  prm.align_mask = static_cast<uint64_t>(p->align) - 1;
-  prm.payload_bytes = p->payload_bytes;
-  prm.tile_shift = tile_shift;
-  prm.seg_shift = p->cfg.seg_shift;
-  prm.head_mask = static_cast<uint32_t>(head_mask);
-  prm.anchor_tensor = receiver ? 1u : 0u;
   uint8_t* d = static_cast<uint8_t*>(p->block.device);
-  int rc = launch_expand_tables(recs, static_cast<uint32_t>(n), reinterpret_cast<Seg*>(d),
-                                reinterpret_cast<uint32_t*>(d + wave_at), prm, stream);
+  int rc = launch_expand_tables(staged, static_cast<uint32_t>(n), reinterpret_cast<Seg*>(d),
+                                reinterpret_cast<uint32_t*>(d + wave_at), p->cfg.seg_shift, stream);
   if (rc) return rc;
   if (!p->upload_event) {
     rc = check_hip(hipEventCreateWithFlags(&p->upload_event, hipEventDisableTiming), "hipEventCreate");
@@ -1117,7 +1107,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   return AXR_OK;
 }
 
-int store_tensor(axr_plan* p, const axr_tensor_t& in, TensorRec* rec) {
+int store_tensor(std::vector<int64_t>& dims64, const axr_tensor_t& in, TensorRec* rec) {
   rec->device_type = in.device_type;
   rec->device_id = in.device_id;
   rec->ndim = in.ndim;
@@ -1126,12 +1116,20 @@ int store_tensor(axr_plan* p, const axr_tensor_t& in, TensorRec* rec) {
   rec->lanes = in.dtype_lanes;
   int rc = nbytes_rule(in.ndim, in.shape, in.dtype_bits, &rec->nbytes);
   if (rc) return rc;
-  rec->shape_at = p->dims64.size();
-  for (int32_t d = 0; d < in.ndim; ++d) p->dims64.push_back(in.shape[d]);
+  rec->shape_at = static_cast<uint32_t>(dims64.size());
   rec->has_strides = in.strides != nullptr && in.ndim > 0;
-  if (rec->has_strides) {
-    rec->strides_at = p->dims64.size();
-    for (int32_t d = 0; d < in.ndim; ++d) p->dims64.push_back(in.strides[d]);
+  if (in.ndim == 1) {
+    dims64.push_back(in.shape[0]);
+    if (rec->has_strides) {
+      rec->strides_at = rec->shape_at + 1;
+      dims64.push_back(in.strides[0]);
+    }
+  } else {
+    dims64.insert(dims64.end(), in.shape, in.shape + in.ndim);
+    if (rec->has_strides) {
+      rec->strides_at = static_cast<uint32_t>(dims64.size());
+      dims64.insert(dims64.end(), in.strides, in.strides + in.ndim);
+    }
   }
   if (rec->nbytes != 0 && in.data == nullptr)
     return fail(AXR_ERR_INVALID, "tensor data pointer is null");
@@ -1164,22 +1162,55 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_create: out of host memory");
   p->align = align;
   p->tensors.resize(n);
-  size_t ndims = 0;
-  for (size_t i = 0; i < n; ++i)
-    if (tensors[i].ndim > 0 && tensors[i].ndim <= kMaxNdim) ndims += 2 * static_cast<size_t>(tensors[i].ndim);
-  p->dims64.reserve(ndims);
+  size_t ndims = 0, shape_words = 0;
   for (size_t i = 0; i < n; ++i) {
-    rc = store_tensor(p, tensors[i], &p->tensors[i]);
+    if (tensors[i].ndim > 0 && tensors[i].ndim <= kMaxNdim) {
+      shape_words += static_cast<size_t>(tensors[i].ndim);
+      ndims += (tensors[i].strides ? 2 : 1) * static_cast<size_t>(tensors[i].ndim);
+    }
+  }
+  p->dims64.clear();
+  p->dims64.reserve(ndims);
+  // one pass: tensor record, layout and header record
+  std::vector<uint8_t>& h = p->header;
+  h.resize(kFixedHeader + n * kTensorHeader + 8 * shape_words);
+  uint8_t* w = h.data() + kFixedHeader;
+  uint64_t off = 0, data = 0, end = 0;
+  const uint64_t mask = static_cast<uint64_t>(align) - 1;
+  for (size_t i = 0; i < n; ++i) {
+    TensorRec& t = p->tensors[i];
+    rc = store_tensor(p->dims64, tensors[i], &t);
     if (rc) {
       plan_delete(p);
       return rc;
     }
+    if (__builtin_add_overflow(off, mask, &off) || (off &= ~mask, __builtin_add_overflow(off, t.nbytes, &end))) {
+      plan_delete(p);
+      return fail(AXR_ERR_INVALID, "axr_plan_create: bundle size overflows 64 bits");
+    }
+    t.offset = off;
+    off = end;
+    data += t.nbytes;
+    WireTensor rec;
+    rec.offset = t.offset;
+    rec.nbytes = t.nbytes;
+    rec.device_type = t.device_type;
+    rec.device_id = t.device_id;
+    rec.ndim = t.ndim;
+    rec.code = t.code;
+    rec.bits = t.bits;
+    rec.lanes = t.lanes;
+    rec.byte_offset = 0;   // the packed copy starts at its offset
+    std::memcpy(w, &rec, kTensorHeader);
+    w += kTensorHeader;
+    if (t.ndim) {
+      std::memcpy(w, tensors[i].shape, 8 * static_cast<size_t>(t.ndim));
+      w += 8 * static_cast<size_t>(t.ndim);
+    }
   }
-  if (!compute_layout(p)) {
-    plan_delete(p);
-    return fail(AXR_ERR_INVALID, "axr_plan_create: bundle size overflows 64 bits");
-  }
-  encode_header(p);
+  p->payload_bytes = end;
+  p->data_bytes = data;
+  encode_preamble(p);
   p->bound = true;
   *plan = p;
   return AXR_OK;
@@ -1299,50 +1330,68 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   p->tensors.resize(n);
   p->dims64.reserve((length - kFixedHeader - static_cast<size_t>(n) * kTensorHeader) / 8);   // all shapes
   size_t at = kFixedHeader;
+  uint64_t expect = 0, end = 0, data = 0;
+  const uint64_t mask = static_cast<uint64_t>(align) - 1;
+  if ((length - kFixedHeader - static_cast<size_t>(n) * kTensorHeader) / 8 > 0xffffffffull) {
+    plan_delete(p);
+    return fail(AXR_ERR_HEADER, "bundle header too long");
+  }
   for (uint32_t i = 0; i < n; ++i) {
     if (length - at < kTensorHeader) {
       plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header truncated");
     }
     TensorRec& t = p->tensors[i];
-    const uint64_t off = get<uint64_t>(h + at);
-    const uint64_t nb = get<uint64_t>(h + at + 8);
-    t.device_type = get<int32_t>(h + at + 16);
-    t.device_id = get<int32_t>(h + at + 20);
-    t.ndim = get<int32_t>(h + at + 24);
-    t.code = get<uint8_t>(h + at + 28);
-    t.bits = get<uint8_t>(h + at + 29);
-    t.lanes = get<uint16_t>(h + at + 30);
-    const uint64_t byte_offset = get<uint64_t>(h + at + 32);
+    WireTensor rec;
+    std::memcpy(&rec, h + at, kTensorHeader);
+    const uint64_t off = rec.offset, nb = rec.nbytes, byte_offset = rec.byte_offset;
+    t.device_type = rec.device_type;
+    t.device_id = rec.device_id;
+    t.ndim = rec.ndim;
+    t.code = rec.code;
+    t.bits = rec.bits;
+    t.lanes = rec.lanes;
     at += kTensorHeader;
     if (t.ndim < 0 || t.ndim > kMaxNdim ||
         static_cast<size_t>(t.ndim) * 8 > length - at || byte_offset != 0) {
       plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header has a bad tensor record");
     }
-    t.shape_at = p->dims64.size();
-    for (int32_t d = 0; d < t.ndim; ++d) p->dims64.push_back(get<int64_t>(h + at + 8 * d));
+    t.shape_at = static_cast<uint32_t>(p->dims64.size());
+    if (t.ndim == 1) {
+      p->dims64.push_back(get<int64_t>(h + at));
+    } else if (t.ndim) {
+      p->dims64.resize(t.shape_at + static_cast<size_t>(t.ndim));
+      std::memcpy(p->dims64.data() + t.shape_at, h + at, 8 * static_cast<size_t>(t.ndim));
+    }
     at += static_cast<size_t>(t.ndim) * 8;
     uint64_t rule = 0;
     if (nbytes_rule(t.ndim, p->dims64.data() + t.shape_at, t.bits, &rule) != AXR_OK || rule != nb) {
       plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header tensor size does not follow from its shape");
     }
+    // the offset must be the one the layout rule gives (no wrapping of 64 bits on the way)
+    uint64_t stop = 0;
+    if (__builtin_add_overflow(expect, mask, &expect) || (expect &= ~mask, expect != off) ||
+        __builtin_add_overflow(off, nb, &stop)) {
+      plan_delete(p);
+      return fail(AXR_ERR_HEADER, "bundle header offsets do not follow the layout rule");
+    }
+    expect = end = stop;
+    data += nb;
     t.nbytes = nb;
-    t.offset = off;   // checked against the layout rule below
+    t.offset = off;
   }
   if (at != length) {
     plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header has trailing bytes");
   }
-  std::vector<uint64_t> sent(n);
-  for (uint32_t i = 0; i < n; ++i) sent[i] = p->tensors[i].offset;
-  bool ok = compute_layout(p) && p->payload_bytes == payload;
-  for (uint32_t i = 0; i < n && ok; ++i) ok = sent[i] == p->tensors[i].offset;
-  if (!ok) {
+  if (end != payload) {
     plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header offsets do not follow the layout rule");
   }
+  p->payload_bytes = end;
+  p->data_bytes = data;
   p->header.assign(h, h + length);
   p->bound = false;
   p->receiver = true;
@@ -1358,24 +1407,22 @@ static int plan_bind_body(axr_plan_t* plan, const axr_tensor_t* tensors, size_t 
   if (n != plan->tensors.size())
     return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor count differs from the plan");
   if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_bind: null tensor array");
-  // Everything is validated and staged in temporaries first: a failure leaves the
-  // plan as it was.
-  std::vector<int64_t> dims64;
-  std::vector<TensorRec> recs(n);
-  {
-    axr_plan tmp;   // reuse store_tensor's bookkeeping
-    tmp.dims64.reserve(plan->dims64.size() * 2);
-    for (size_t i = 0; i < n; ++i) {
-      const TensorRec& t = plan->tensors[i];
-      int rc = store_tensor(&tmp, tensors[i], &recs[i]);   // size rule, null checks
-      if (rc) return rc;
-      if (recs[i].nbytes != t.nbytes ||
-          (t.nbytes != 0 && (recs[i].bits + 7) / 8 != (t.bits + 7) / 8))
-        return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor " + std::to_string(i) +
-                                          " does not match the plan's size or element width");
-      recs[i].offset = t.offset;
-    }
-    dims64.swap(tmp.dims64);
+  // Everything is validated and staged first (in vectors the plan keeps for this): a
+  // failure leaves the plan as it was.
+  std::vector<TensorRec>& recs = plan->staged_tensors;
+  std::vector<int64_t>& dims64 = plan->staged_dims64;
+  recs.resize(n);
+  dims64.clear();
+  dims64.reserve(plan->dims64.size() * 2);
+  for (size_t i = 0; i < n; ++i) {
+    const TensorRec& t = plan->tensors[i];
+    int rc = store_tensor(dims64, tensors[i], &recs[i]);   // size rule, null checks
+    if (rc) return rc;
+    if (recs[i].nbytes != t.nbytes ||
+        (t.nbytes != 0 && (recs[i].bits + 7) / 8 != (t.bits + 7) / 8))
+      return fail(AXR_ERR_MISMATCH, "axr_plan_bind: tensor " + std::to_string(i) +
+                                        " does not match the plan's size or element width");
+    recs[i].offset = t.offset;
   }
   quiesce(plan);
   invalidate_tables(plan);

@@ -414,8 +414,9 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * between pageable memory and the pinned staging blocks once a copy is 2 MiB or
  * more; default 4, 1: the calling thread alone),
  * "device_tables" (a bundle of at least this many tensors, all contiguous device
- * tensors, gets its device tables from a small kernel that expands one 24-byte
- * record per tensor, instead of tables built on the host and uploaded; default 512,
+ * tensors, takes a short path to its device tables: one pass over the tensors into
+ * pinned memory and a kernel that brings the records to the device and writes the
+ * tile-block index, instead of the general host build plus an upload; default 512,
  * 0: never),
  * "loopback_copy_kernel" (1, default: the loopback context moves a device payload
  * to device memory with the library's copy kernel; 0: with hipMemcpyAsync),
