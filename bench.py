@@ -313,8 +313,9 @@ def rate(data_bytes, ms, steps):
 
 
 def end_to_end_us(h, spec, steps=20):
-    """Wall time of plan -> pack -> sync -> plan-from-header -> bind -> unpack -> sync for a
-    fresh 4,096-tensor bundle, C ABI only (tensor descriptors prebuilt)."""
+    """Wall time of plan -> pack -> sync -> plan from header and destination tensors
+    (axr_plan_from_header_bind) -> unpack -> sync for a fresh 4,096-tensor bundle, C ABI only
+    (tensor descriptors prebuilt)."""
     from execution_ucx_amd import workloads
     from execution_ucx_amd.dlpack import TensorArray
     lib, capi = h.lib, h.capi
@@ -341,8 +342,7 @@ def end_to_end_us(h, spec, steps=20):
         capi.check(lib.axr_pack(p, payload.data_ptr(), nbytes, h.stream))
         capi.check(lib.axr_stream_synchronize(h.stream))
         r = C.c_void_p()
-        capi.check(lib.axr_plan_from_header(hp, hn.value, C.byref(r)))
-        capi.check(lib.axr_plan_bind(r, da.pointer(), da.count))
+        capi.check(lib.axr_plan_from_header_bind(hp, hn.value, da.pointer(), da.count, C.byref(r)))
         capi.check(lib.axr_unpack(r, payload.data_ptr(), nbytes, h.stream))
         capi.check(lib.axr_stream_synchronize(h.stream))
         t2 = time.perf_counter()

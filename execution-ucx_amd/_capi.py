@@ -251,6 +251,7 @@ PROTOTYPES = {
     "axr_plan_header": (C.c_int, [_vp, _vpp, C.POINTER(_sz)]),
     "axr_plan_from_header": (C.c_int, [_vp, _sz, _vpp]),
     "axr_plan_bind": (C.c_int, [_vp, _TensorP, _sz]),
+    "axr_plan_from_header_bind": (C.c_int, [_vp, _sz, _TensorP, _sz, _vpp]),
     "axr_plan_split": (C.c_int, [_vp, _vp, _sz, C.POINTER(Buffer)]),
     "axr_pack": (C.c_int, [_vp, _vp, _sz, _vp]),
     "axr_unpack": (C.c_int, [_vp, _vp, _sz, _vp]),

@@ -96,6 +96,16 @@ class BundlePlan:
         _capi.check(lib.axr_plan_from_header(buf, len(buf), C.byref(h)))
         return cls(h.value)
 
+    @classmethod
+    def from_header_bound(cls, header: bytes, tensors: Sequence[Any]) -> "BundlePlan":
+        """``from_header(header).bind(tensors)`` in one pass over the header."""
+        lib = _capi.load()
+        buf = bytes(header)
+        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
+        h = C.c_void_p()
+        _capi.check(lib.axr_plan_from_header_bind(buf, len(buf), arr.pointer(), arr.count, C.byref(h)))
+        return cls(h.value, keepalive=arr)
+
     def bind(self, tensors: Sequence[Any]) -> "BundlePlan":
         arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
         _capi.check(self._lib.axr_plan_bind(self._h, arr.pointer(), arr.count))

@@ -1309,7 +1309,10 @@ int axr_plan_header(const axr_plan_t* plan, const void** header, size_t* length)
   return guarded([&] { return plan_header_body(plan, header, length); });
 }
 
-static int plan_from_header_body(const void* header, size_t length, axr_plan_t** plan) {
+// `bound` (may be null): the receiver's tensors, attached in the same pass (axr_plan_from_header
+// followed by axr_plan_bind, without a second walk over the records).
+static int plan_from_header_body(const void* header, size_t length, const axr_tensor_t* bound,
+                                 size_t nbound, bool binding, axr_plan_t** plan) {
   if (!plan) return fail(AXR_ERR_INVALID, "axr_plan_from_header: null result");
   *plan = nullptr;
   if (!header) return fail(AXR_ERR_INVALID, "axr_plan_from_header: null header");
@@ -1324,11 +1327,15 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   if (check_align(align) != AXR_OK) return fail(AXR_ERR_HEADER, "bundle header has a bad alignment");
   if (static_cast<uint64_t>(n) * kTensorHeader > length - kFixedHeader)
     return fail(AXR_ERR_HEADER, "bundle header truncated");
+  if (binding) {
+    if (nbound != n) return fail(AXR_ERR_MISMATCH, "axr_plan_from_header_bind: tensor count differs from the header");
+    if (n && !bound) return fail(AXR_ERR_INVALID, "axr_plan_from_header_bind: null tensor array");
+  }
   axr_plan* p = plan_new();
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_from_header: out of host memory");
   p->align = align;
   p->tensors.resize(n);
-  p->dims64.reserve((length - kFixedHeader - static_cast<size_t>(n) * kTensorHeader) / 8);   // all shapes
+  p->dims64.reserve((length - kFixedHeader - static_cast<size_t>(n) * kTensorHeader) / 8 * (binding ? 2 : 1));
   size_t at = kFixedHeader;
   uint64_t expect = 0, end = 0, data = 0;
   const uint64_t mask = static_cast<uint64_t>(align) - 1;
@@ -1357,18 +1364,39 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
       plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header has a bad tensor record");
     }
-    t.shape_at = static_cast<uint32_t>(p->dims64.size());
-    if (t.ndim == 1) {
-      p->dims64.push_back(get<int64_t>(h + at));
-    } else if (t.ndim) {
-      p->dims64.resize(t.shape_at + static_cast<size_t>(t.ndim));
-      std::memcpy(p->dims64.data() + t.shape_at, h + at, 8 * static_cast<size_t>(t.ndim));
+    uint64_t rule = 0;
+    int sized;
+    if (!binding) {
+      t.shape_at = static_cast<uint32_t>(p->dims64.size());
+      if (t.ndim == 1) {
+        p->dims64.push_back(get<int64_t>(h + at));
+      } else if (t.ndim) {
+        p->dims64.resize(t.shape_at + static_cast<size_t>(t.ndim));
+        std::memcpy(p->dims64.data() + t.shape_at, h + at, 8 * static_cast<size_t>(t.ndim));
+      }
+      sized = nbytes_rule(t.ndim, p->dims64.data() + t.shape_at, t.bits, &rule);
+    } else {
+      int64_t sent_shape[kMaxNdim];   // the record's shape is only checked; the bound tensor's is kept
+      std::memcpy(sent_shape, h + at, 8 * static_cast<size_t>(t.ndim));
+      sized = nbytes_rule(t.ndim, sent_shape, t.bits, &rule);
     }
     at += static_cast<size_t>(t.ndim) * 8;
-    uint64_t rule = 0;
-    if (nbytes_rule(t.ndim, p->dims64.data() + t.shape_at, t.bits, &rule) != AXR_OK || rule != nb) {
+    if (sized != AXR_OK || rule != nb) {
       plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header tensor size does not follow from its shape");
+    }
+    if (binding) {
+      const uint32_t sent_item = (static_cast<uint32_t>(t.bits) + 7) / 8;
+      int rc = store_tensor(p->dims64, bound[i], &t);   // size rule, null checks; replaces the record
+      if (rc) {
+        plan_delete(p);
+        return rc;
+      }
+      if (t.nbytes != nb || (nb != 0 && (static_cast<uint32_t>(t.bits) + 7) / 8 != sent_item)) {
+        plan_delete(p);
+        return fail(AXR_ERR_MISMATCH, "axr_plan_from_header_bind: tensor " + std::to_string(i) +
+                                          " does not match the header's size or element width");
+      }
     }
     // the offset must be the one the layout rule gives (no wrapping of 64 bits on the way)
     uint64_t stop = 0;
@@ -1393,13 +1421,17 @@ static int plan_from_header_body(const void* header, size_t length, axr_plan_t**
   p->payload_bytes = end;
   p->data_bytes = data;
   p->header.assign(h, h + length);
-  p->bound = false;
+  p->bound = binding;
   p->receiver = true;
   *plan = p;
   return AXR_OK;
 }
 int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan) {
-  return guarded([&] { return plan_from_header_body(header, length, plan); });
+  return guarded([&] { return plan_from_header_body(header, length, nullptr, 0, false, plan); });
+}
+int axr_plan_from_header_bind(const void* header, size_t length, const axr_tensor_t* tensors, size_t n,
+                              axr_plan_t** plan) {
+  return guarded([&] { return plan_from_header_body(header, length, tensors, n, true, plan); });
 }
 
 static int plan_bind_body(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n) {

@@ -276,6 +276,13 @@ AXR_API int axr_plan_from_header(const void* header, size_t length, axr_plan_t**
  * (unpack into views).  Overlapping destinations (a stride of 0 on an extent
  * above 1) are refused for unpack. */
 AXR_API int axr_plan_bind(axr_plan_t* plan, const axr_tensor_t* tensors, size_t n);
+/* axr_plan_from_header followed by axr_plan_bind in one pass over the header's
+ * records, for a receiver that has its destination tensors at hand when the
+ * header arrives (a memory policy that answers from a cache of buffers,
+ * axon/src/axon_worker.cpp:1150-1172).  Same checks and errors as the two calls;
+ * *plan is NULL on failure. */
+AXR_API int axr_plan_from_header_bind(const void* header, size_t length, const axr_tensor_t* tensors,
+                                      size_t n, axr_plan_t** plan);
 
 /* Zero-copy receive mode: views[i] = {payload + offset[i], nbytes[i]}, the
  * result of UcxBuffer::to_buffer_vec(sizes) (ucx_context_data.hpp:641-665).

@@ -141,6 +141,21 @@ int main(int argc, char** argv) {
     rc = axr_plan_bind(back, n ? c.tensors.data() : nullptr, n);
     if (rc != AXR_OK && rc != AXR_ERR_MISMATCH) die("bind", rc);
     if (rc == AXR_OK) inspect(back, n);
+    {   // the same in one pass: same verdict, same tables
+      axr_plan_t* fused = nullptr;
+      const int rc1 = axr_plan_from_header_bind(bytes.data(), bytes.size(), n ? c.tensors.data() : nullptr, n, &fused);
+      if (rc1 != rc) die("from_header_bind verdict differs from from_header + bind", rc1);
+      if (rc1 == AXR_OK) {
+        inspect(fused, n);
+        size_t c1 = 0, c2 = 0;
+        axr_plan_segments(fused, nullptr, 0, &c1);
+        axr_plan_segments(back, nullptr, 0, &c2);
+        if (c1 != c2) die("from_header_bind segment count", -1);
+        axr_plan_free(fused);
+      } else if (fused) {
+        die("plan set on failed from_header_bind", rc1);
+      }
+    }
     axr_plan_free(back);
 
     for (int m = 0; m < 8; ++m) {   // mutated headers
@@ -160,6 +175,12 @@ int main(int argc, char** argv) {
       // exact-size heap copy so that a read past the end is an ASan error
       uint8_t* heap = static_cast<uint8_t*>(std::malloc(mutated.size() ? mutated.size() : 1));
       std::memcpy(heap, mutated.data(), mutated.size());
+      {   // mutated headers through the one-pass call too (its result is only freed)
+        axr_plan_t* q = nullptr;
+        const int rq = axr_plan_from_header_bind(heap, mutated.size(), n ? c.tensors.data() : nullptr, n, &q);
+        if (rq == AXR_OK) axr_plan_free(q);
+        else if (q) die("plan set on failed from_header_bind", rq);
+      }
       rc = axr_plan_from_header(heap, mutated.size(), &p);
       ++decodes;
       if (rc == AXR_OK) {

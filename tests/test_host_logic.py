@@ -424,6 +424,39 @@ def test_bind_validation(pkg, orc):
     assert [s["mode"] for s in plan.segments()] == [0, 2]
 
 
+def test_header_and_tensors_in_one_pass(pkg, orc):
+    """axr_plan_from_header_bind gives the plan that axr_plan_from_header + axr_plan_bind give,
+    with the same refusals."""
+    metas = [{"device": (10, 0), "dtype": (2, 32, 1), "shape": (100,)},
+             {"device": (10, 0), "dtype": (4, 16, 1), "shape": (8, 8)},
+             {"device": (10, 0), "dtype": (1, 8, 1), "shape": (0,)},
+             {"device": (10, 0), "dtype": (1, 8, 1), "shape": (5000,)}]
+    for align in (1, 256):
+        hdr = orc.encode_header(metas, align)
+        views = [tv(pkg, 0x1000, [100], dtype=(0, 32, 1)),
+                 tv(pkg, 0x2000, [8, 8], strides=[16, 1], dtype=(2, 16, 1)),
+                 tv(pkg, 0, [0]), tv(pkg, 0x5003, [5000])]
+        two = pkg.BundlePlan.from_header(hdr).bind(views)
+        one = pkg.BundlePlan.from_header_bound(hdr, views)
+        assert one.segments() == two.segments()
+        assert one.layout() == two.layout() and one.header == two.header == hdr
+        assert one.launch_info() == two.launch_info()
+        assert one.payload_bytes == two.payload_bytes and one.data_bytes == two.data_bytes
+        assert [m.shape for m in one.metas()] == [m.shape for m in two.metas()]
+        with pytest.raises(pkg.MismatchError):
+            pkg.BundlePlan.from_header_bound(hdr, views[:3])
+        with pytest.raises(pkg.MismatchError):
+            pkg.BundlePlan.from_header_bound(hdr, views[:3] + [tv(pkg, 0x5003, [5001])])
+        with pytest.raises(pkg.MismatchError):      # same bytes, other element width
+            pkg.BundlePlan.from_header_bound(hdr, [tv(pkg, 0x1000, [200], dtype=(0, 16, 1))] + views[1:])
+        with pytest.raises(pkg.AxonRocmError):      # null data for a tensor with bytes
+            pkg.BundlePlan.from_header_bound(hdr, views[:3] + [tv(pkg, 0, [5000])])
+        with pytest.raises(pkg.HeaderError):
+            pkg.BundlePlan.from_header_bound(hdr[:-1], views)
+        with pytest.raises(pkg.HeaderError):
+            pkg.BundlePlan.from_header_bound(hdr[:20] + b"\x01" + hdr[21:], views)
+
+
 # ------------------------------------------------------------------ DLPack and devices
 
 def test_dlpack_extract_numpy(pkg):
