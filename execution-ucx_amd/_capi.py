@@ -27,6 +27,8 @@ AXR_ERR_HEADER = -8
 AXR_ERR_MISMATCH = -9
 AXR_ERR_NO_DEVICE = -10
 AXR_ERR_BUSY = -11
+AXR_ERR_CANCELED = -12
+AXR_ERR_CANCELED = -12
 
 # ucx_memory_type_t numbering (ucx_context/ucx_context_def.h:27-39)
 MEM_HOST = 0
@@ -268,6 +270,8 @@ PROTOTYPES = {
     "axr_am_send": (C.c_int, [_vp, C.c_uint64, C.POINTER(AmData), _vp, _u64p]),
     "axr_am_send_iov": (C.c_int, [_vp, C.c_uint64, C.POINTER(AmIovec), _vp, _u64p]),
     "axr_am_request_test": (C.c_int, [_vp, C.c_uint64, _intp]),
+    "axr_am_request_cancel": (C.c_int, [_vp, C.c_uint64]),
+    "axr_am_progress": (C.c_int, [_vp, C.POINTER(_sz), C.POINTER(_sz)]),
     "axr_am_recv_header": (C.c_int, [_vp, C.POINTER(AmMessage)]),
     "axr_am_recv_buffer": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
     "axr_am_recv_buffer_async": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),

@@ -3,6 +3,7 @@
 // are given with the declarations in axon_rocm.h.
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -27,6 +28,7 @@ struct Piece {
 struct Request {
   std::atomic<int> done{0};        // 1 complete, -1 cancelled or failed
   hipEvent_t event = nullptr;      // set by an asynchronous fetch: done once it has fired
+  bool claimed = false;            // a receiver has begun to fetch the payload: too late to cancel
   std::mutex mu;
   ~Request() {
     if (event) (void)hipEventDestroy(event);
@@ -45,8 +47,25 @@ struct Message {
   std::shared_ptr<Request> request;
 };
 
+// 0 pending, 1 complete, -1 cancelled or failed; an asynchronous fetch completes with its event.
+int poll_request(Request* r) {
+  int st = r->done.load();
+  if (st == 0) {
+    std::lock_guard<std::mutex> rl(r->mu);
+    if (r->event) {
+      const hipError_t q = hipEventQuery(r->event);
+      if (q == hipSuccess) st = 1;
+      else if (q != hipErrorNotReady) st = -1;
+      if (st != 0) r->done.store(st);
+    }
+  }
+  return st;
+}
+
 bool host_type(int t) { return t == AXR_MEM_HOST || t == AXR_MEM_ROCM_MANAGED; }
 bool known_type(int t) { return host_type(t) || t == AXR_MEM_ROCM; }
+
+constexpr size_t kMaxInFlight = 256;
 
 std::atomic<uint64_t> g_next_id{1};
 
@@ -66,6 +85,16 @@ struct axr_am_context {
   std::map<uint64_t, std::unique_ptr<Message>> parked;   // handed out, awaiting fetch/release
   std::map<uint64_t, axr_am_context*> endpoints;         // conn id -> peer
   std::map<uint64_t, std::shared_ptr<Request>> requests;
+  // Sends that have started and not completed (rendezvous sends whose payload has not been
+  // fetched): at most kMaxInFlight, as the reference's context admits 256 operations
+  // (kCompletionQueueEntryCount, ucx_am_context.hpp:94,836-839).  Further sends wait here, in
+  // order, and start as completions make room (pendingIoQueue_, ucx_am_context.cpp:271-274).
+  std::vector<std::shared_ptr<Request>> in_flight;
+  struct Waiting {
+    uint64_t conn_id;
+    std::unique_ptr<Message> message;
+  };
+  std::deque<Waiting> waiting;
 };
 
 namespace {
@@ -95,19 +124,8 @@ int copy_piece(int dst_type, void* dst, int src_type, const void* src, size_t n,
   return check_hip(hipMemcpyAsync(dst, src, n, hipMemcpyDefault, s), "hipMemcpyAsync(loopback)");
 }
 
-int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, uint64_t* request) {
-  axr_am_context* peer = nullptr;
-  {
-    std::lock_guard<std::mutex> lock(ctx->mu);
-    auto it = ctx->endpoints.find(conn_id);
-    if (it == ctx->endpoints.end()) return fail(AXR_ERR_INVALID, "unknown connection id");
-    peer = it->second;
-    const uint64_t rid = g_next_id++;
-    ctx->requests[rid] = m->request;
-    if (request) *request = rid;
-  }
-  m->key = g_next_id++;
-  m->conn_id = conn_id;
+// Puts the message into the peer's arrival queue.  ctx->mu is NOT held.
+int hand_over(axr_am_context* peer, std::unique_ptr<Message> m) {
   std::lock_guard<std::mutex> alive(g_contexts_mu);
   if (!g_contexts.count(peer)) {
     m->request->done.store(-1);
@@ -116,6 +134,67 @@ int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, u
   std::lock_guard<std::mutex> lock(peer->mu);
   peer->arrived.push_back(std::move(m));
   return AXR_OK;
+}
+
+// Forgets completed sends and starts waiting ones while there is room, in order.
+void progress(axr_am_context* ctx) {
+  for (;;) {
+    axr_am_context* peer = nullptr;
+    std::unique_ptr<Message> m;
+    {
+      std::lock_guard<std::mutex> lock(ctx->mu);
+      auto& fl = ctx->in_flight;
+      fl.erase(std::remove_if(fl.begin(), fl.end(),
+                              [](const std::shared_ptr<Request>& r) { return poll_request(r.get()) != 0; }),
+               fl.end());
+      // cancelled while waiting: dropped without ever reaching the peer
+      ctx->waiting.erase(std::remove_if(ctx->waiting.begin(), ctx->waiting.end(),
+                                        [](const axr_am_context::Waiting& w) {
+                                          return w.message->request->done.load() == -1;
+                                        }),
+                         ctx->waiting.end());
+      if (ctx->waiting.empty()) return;
+      Message* front = ctx->waiting.front().message.get();
+      const bool counts = front->rndv;
+      if (counts && fl.size() >= kMaxInFlight) return;
+      auto it = ctx->endpoints.find(ctx->waiting.front().conn_id);
+      peer = it == ctx->endpoints.end() ? nullptr : it->second;
+      m = std::move(ctx->waiting.front().message);
+      ctx->waiting.pop_front();
+      if (counts) fl.push_back(m->request);
+    }
+    if (!peer) {
+      m->request->done.store(-1);
+      continue;
+    }
+    (void)hand_over(peer, std::move(m));   // a destroyed peer fails the request; the rest goes on
+  }
+}
+
+int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, uint64_t* request) {
+  progress(ctx);
+  axr_am_context* peer = nullptr;
+  bool wait = false;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto it = ctx->endpoints.find(conn_id);
+    if (it == ctx->endpoints.end()) return fail(AXR_ERR_INVALID, "unknown connection id");
+    peer = it->second;
+    const uint64_t rid = g_next_id++;
+    ctx->requests[rid] = m->request;
+    if (request) *request = rid;
+    m->key = g_next_id++;
+    m->conn_id = conn_id;
+    // behind sends that wait (order is kept), or when the context is full
+    wait = !ctx->waiting.empty() || (m->rndv && ctx->in_flight.size() >= kMaxInFlight);
+    if (wait) {
+      ctx->waiting.push_back({conn_id, std::move(m)});
+    } else if (m->rndv) {
+      ctx->in_flight.push_back(m->request);
+    }
+  }
+  if (wait) return AXR_OK;
+  return hand_over(peer, std::move(m));
 }
 
 }  // namespace
@@ -149,6 +228,7 @@ static int am_context_destroy_body(axr_am_context_t* ctx) {
     std::lock_guard<std::mutex> lock(ctx->mu);
     for (auto& m : ctx->arrived) m->request->done.store(-1);
     for (auto& kv : ctx->parked) kv.second->request->done.store(-1);
+    for (auto& w : ctx->waiting) w.message->request->done.store(-1);
   }
   delete ctx;
   return AXR_OK;
@@ -242,19 +322,11 @@ int axr_am_send_iov(axr_am_context_t* ctx,
 
 static int am_request_test_body(axr_am_context_t* ctx, uint64_t request, int* done) {
   if (!ctx || !done) return fail(AXR_ERR_INVALID, "axr_am_request_test: null argument");
+  progress(ctx);
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->requests.find(request);
   if (it == ctx->requests.end()) return fail(AXR_ERR_INVALID, "axr_am_request_test: unknown request");
-  int st = it->second->done.load();
-  if (st == 0) {
-    std::lock_guard<std::mutex> rl(it->second->mu);
-    if (it->second->event) {
-      const hipError_t q = hipEventQuery(it->second->event);
-      if (q == hipSuccess) st = 1;
-      else if (q != hipErrorNotReady) st = -1;
-      if (st != 0) it->second->done.store(st);
-    }
-  }
+  const int st = poll_request(it->second.get());
   *done = st;
   if (st != 0) ctx->requests.erase(it);
   return AXR_OK;
@@ -266,6 +338,9 @@ int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done) {
 static int am_recv_header_body(axr_am_context_t* ctx, axr_am_message_t* out) {
   if (!ctx || !out) return fail(AXR_ERR_INVALID, "axr_am_recv_header: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  // a rendezvous whose sender has cancelled it in the meantime never shows up
+  while (!ctx->arrived.empty() && ctx->arrived.front()->rndv && ctx->arrived.front()->request->done.load() == -1)
+    ctx->arrived.pop_front();
   if (ctx->arrived.empty()) return fail(AXR_ERR_NO_MESSAGE, "no message queued");
   std::unique_ptr<Message> m = std::move(ctx->arrived.front());
   ctx->arrived.pop_front();
@@ -295,6 +370,16 @@ static int fetch(axr_am_context_t* ctx, uint64_t key, int dst_type, const axr_bu
     if (it == ctx->parked.end()) return fail(AXR_ERR_NO_MESSAGE, "no message with this key");
     if (!it->second->rndv)
       return fail(AXR_ERR_NOT_IMPLEMENTED, "message was eager: its data came with the header");
+    {
+      // claim the payload, unless the sender has cancelled the send in the meantime
+      Request* r = it->second->request.get();
+      std::lock_guard<std::mutex> rl(r->mu);
+      if (r->done.load() == -1) {
+        ctx->parked.erase(it);
+        return fail(AXR_ERR_CANCELED, "the sender cancelled this message");
+      }
+      r->claimed = true;
+    }
     uint64_t room = 0;
     for (size_t i = 0; i < count; ++i) room += vec[i].size;
     if (room < it->second->data_length)
@@ -388,6 +473,37 @@ int axr_am_recv_buffer_iov(axr_am_context_t* ctx,
                            void* stream) {
   return guarded([&] { return am_recv_buffer_iov_body(ctx, key, dst_type, buffer_vec, buffer_count,
                  stream); });
+}
+
+static int am_request_cancel_body(axr_am_context_t* ctx, uint64_t request) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_request_cancel: null context");
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto it = ctx->requests.find(request);
+    if (it == ctx->requests.end()) return fail(AXR_ERR_INVALID, "axr_am_request_cancel: unknown request");
+    // only a send that has not completed can be cancelled; the receiver then finds the message
+    // gone (or fails its fetch), and the sender's buffers are its own again
+    Request* r = it->second.get();
+    std::lock_guard<std::mutex> rl(r->mu);
+    if (!r->claimed && r->done.load() == 0) r->done.store(-1);
+  }
+  progress(ctx);   // room for a waiting send
+  return AXR_OK;
+}
+int axr_am_request_cancel(axr_am_context_t* ctx, uint64_t request) {
+  return guarded([&] { return am_request_cancel_body(ctx, request); });
+}
+
+static int am_progress_body(axr_am_context_t* ctx, size_t* in_flight, size_t* waiting) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_progress: null context");
+  progress(ctx);
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (in_flight) *in_flight = ctx->in_flight.size();
+  if (waiting) *waiting = ctx->waiting.size();
+  return AXR_OK;
+}
+int axr_am_progress(axr_am_context_t* ctx, size_t* in_flight, size_t* waiting) {
+  return guarded([&] { return am_progress_body(ctx, in_flight, waiting); });
 }
 
 static int am_message_release_body(axr_am_context_t* ctx, uint64_t key) {

@@ -334,6 +334,7 @@ const char* axr_status_string(int status) {
     case AXR_ERR_MISMATCH: return "AXR_ERR_MISMATCH";
     case AXR_ERR_NO_DEVICE: return "AXR_ERR_NO_DEVICE";
     case AXR_ERR_BUSY: return "AXR_ERR_BUSY";
+    case AXR_ERR_CANCELED: return "AXR_ERR_CANCELED";
     default: return "AXR_ERR_?";
   }
 }

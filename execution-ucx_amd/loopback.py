@@ -93,6 +93,18 @@ class LoopbackAmContext:
             self._keep.pop(request, None)
         return bool(done.value)
 
+    def cancel(self, request: int) -> None:
+        """Sender-side cancellation of a send that has not completed (a waiting send is
+        dropped, an unfetched rendezvous disappears at the receiver); ``test`` then raises."""
+        _capi.check(self._lib.axr_am_request_cancel(self._h, request))
+
+    def progress(self) -> Tuple[int, int]:
+        """Start waiting sends where completions made room; returns (sends in flight, sends
+        waiting).  A context admits 256 uncompleted sends (ucx_am_context.hpp:94)."""
+        a, b = C.c_size_t(), C.c_size_t()
+        _capi.check(self._lib.axr_am_progress(self._h, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
     # ---- receive
     def pending(self) -> int:
         n = C.c_size_t()

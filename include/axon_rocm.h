@@ -54,7 +54,9 @@ typedef enum axr_status {
   AXR_ERR_HEADER = -8,          /* malformed bundle header                      */
   AXR_ERR_MISMATCH = -9,        /* bound tensors do not match the plan's metas  */
   AXR_ERR_NO_DEVICE = -10,      /* no usable ROCm device in this process        */
-  AXR_ERR_BUSY = -11            /* object still has work in flight              */
+  AXR_ERR_BUSY = -11,           /* object still has work in flight              */
+  AXR_ERR_CANCELED = -12        /* the peer cancelled the operation
+                                   (UCS_ERR_CANCELED)                           */
 } axr_status_t;
 
 /* Human-readable name of a status code (static storage). */
@@ -497,7 +499,22 @@ AXR_API int axr_am_send(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_da
                         void* stream, uint64_t* request);
 AXR_API int axr_am_send_iov(axr_am_context_t* ctx, uint64_t conn_id, const axr_am_iovec_t* data,
                             void* stream, uint64_t* request);
+/* *done: 0 pending, 1 complete, -1 cancelled or failed. */
 AXR_API int axr_am_request_test(axr_am_context_t* ctx, uint64_t request, int* done);
+/* Cancel a send that has not completed (the sender-side stop request of the reference's
+ * send operation, ucx_am_context.hpp:2234-2642): a send that still waits for room is
+ * dropped, a rendezvous that the receiver has not fetched disappears from its queue (a
+ * fetch under way elsewhere fails with AXR_ERR_CANCELED); the request then tests as -1.
+ * A completed send is left as it is. */
+AXR_API int axr_am_request_cancel(axr_am_context_t* ctx, uint64_t request);
+/* A context admits 256 sends that have started and not completed (rendezvous sends whose
+ * payload has not been fetched), the reference's kCompletionQueueEntryCount
+ * (ucx_am_context.hpp:94,836-839).  Further sends are accepted, wait in order, and start as
+ * completions make room (ucx_am_context.cpp:271-274); eager sends behind them wait too, so
+ * the order of delivery is the order of the calls.  Completions are noticed inside
+ * axr_am_send*, axr_am_request_test, axr_am_request_cancel and here.  Either result may be
+ * NULL. */
+AXR_API int axr_am_progress(axr_am_context_t* ctx, size_t* in_flight, size_t* waiting);
 /* Next message in arrival order; AXR_ERR_NO_MESSAGE when none is queued. */
 AXR_API int axr_am_recv_header(axr_am_context_t* ctx, axr_am_message_t* message);
 /* Fetch a rendezvous payload into one contiguous buffer of memory type

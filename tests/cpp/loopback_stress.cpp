@@ -2,7 +2,10 @@
 // meant to be built with ThreadSanitizer (tests/test_host_cpp.py does that): several
 // sender threads, each on a connection of its own, push eager and rendezvous messages
 // at one server context while a receiver thread drains it and checks every payload,
-// and another thread creates, connects and destroys unrelated contexts.  The reference's
+// another sender cancels every other of its rendezvous sends right away, and another
+// thread creates, connects and destroys unrelated contexts.  Two thirds of the messages
+// are rendezvous sends, so that senders run into the 256 sends a context admits and the
+// rest waits its turn.  The reference's
 // context is reached from any thread with the work hopping to the context thread
 // (ucx_context/ucx_am_context/ucx_am_context.hpp:2318-2392); here a mutex per context
 // stands in for that hop.  Prints "loopback_stress ok <messages>" and exits 0.
@@ -41,6 +44,8 @@ int main() {
   if (int rc = axr_am_context_create("server", 4096, &server)) die("create server", rc);
   std::atomic<int> received{0};
   std::atomic<bool> stop_churn{false};
+  std::atomic<bool> canceller_done{false};
+  std::atomic<int> cancelled_seen{0};
 
   std::vector<std::thread> threads;
   for (int s = 0; s < kSenders; ++s) {
@@ -53,7 +58,7 @@ int main() {
       std::vector<std::vector<uint8_t>> live(kPerSender);
       std::vector<uint64_t> requests(kPerSender);
       for (int q = 0; q < kPerSender; ++q) {
-        const uint32_t bytes = (q % 3 == 0) ? 8192u + static_cast<uint32_t>(q) : static_cast<uint32_t>(q % 200);
+        const uint32_t bytes = (q % 3 != 2) ? 8192u + static_cast<uint32_t>(q) : static_cast<uint32_t>(q % 200);
         live[q].resize(bytes);
         for (size_t i = 0; i < bytes; ++i) live[q][i] = byte_of(s, q, i);
         Tag tag{static_cast<uint32_t>(s), static_cast<uint32_t>(q), bytes, 0};
@@ -77,10 +82,49 @@ int main() {
       if (int rc = axr_am_context_destroy(client)) die("destroy client", rc);
     });
   }
-  threads.emplace_back([server, &received] {
-    std::vector<uint32_t> next(kSenders, 0);
+  threads.emplace_back([server, &canceller_done] {   // sends and cancels
+    axr_am_context_t* client = nullptr;
+    if (int rc = axr_am_context_create("canceller", 4096, &client)) die("create canceller", rc);
+    uint64_t conn = 0;
+    if (int rc = axr_am_connect(client, server, &conn)) die("connect canceller", rc);
+    constexpr int kCount = 300;
+    std::vector<std::vector<uint8_t>> live(kCount);
+    std::vector<uint64_t> requests(kCount);
+    for (int q = 0; q < kCount; ++q) {
+      const uint32_t bytes = 8192u + static_cast<uint32_t>(q);
+      live[q].resize(bytes);
+      for (size_t i = 0; i < bytes; ++i) live[q][i] = byte_of(kSenders, q, i);
+      Tag tag{static_cast<uint32_t>(kSenders), static_cast<uint32_t>(q), bytes, 0};
+      axr_am_data_t d;
+      std::memset(&d, 0, sizeof(d));
+      d.header.data = &tag;
+      d.header.size = sizeof(tag);
+      d.buffer.data = live[q].data();
+      d.buffer.size = bytes;
+      d.buffer_type = AXR_MEM_HOST;
+      if (int rc = axr_am_send(client, conn, &d, nullptr, &requests[q])) die("send (canceller)", rc);
+      if (q % 2) {
+        if (int rc = axr_am_request_cancel(client, requests[q])) die("cancel", rc);
+      }
+    }
+    for (int q = 0; q < kCount; ++q) {
+      int done = 0;
+      while (!done) {
+        if (int rc = axr_am_request_test(client, requests[q], &done)) die("request_test (canceller)", rc);
+        if (done < 0 && q % 2 == 0) die("a send that nobody cancelled failed", done);
+        if (!done) std::this_thread::yield();
+      }
+    }
+    size_t in_flight = 1, waiting = 1;
+    if (int rc = axr_am_progress(client, &in_flight, &waiting)) die("progress", rc);
+    if (in_flight || waiting) die("sends left behind", -1);
+    if (int rc = axr_am_context_destroy(client)) die("destroy canceller", rc);
+    canceller_done.store(true);
+  });
+  threads.emplace_back([server, &received, &canceller_done, &cancelled_seen] {
+    std::vector<uint32_t> next(kSenders + 1, 0);
     std::vector<uint8_t> buf(16384);
-    while (received.load() < kSenders * kPerSender) {
+    while (received.load() < kSenders * kPerSender || !canceller_done.load()) {
       axr_am_message_t m;
       const int rc = axr_am_recv_header(server, &m);
       if (rc == AXR_ERR_NO_MESSAGE) {
@@ -91,11 +135,22 @@ int main() {
       Tag tag;
       if (m.header.size != sizeof(tag)) die("header size", -1);
       std::memcpy(&tag, m.header.data, sizeof(tag));
-      if (tag.sender >= static_cast<uint32_t>(kSenders) || tag.seq != next[tag.sender]++) die("order per connection", -1);
+      if (tag.sender > static_cast<uint32_t>(kSenders)) die("sender id", -1);
+      if (tag.sender == static_cast<uint32_t>(kSenders)) {   // the canceller: some are missing, none out of order
+        if (tag.seq < next[tag.sender]) die("order on the canceller's connection", -1);
+        next[tag.sender] = tag.seq + 1;
+      } else if (tag.seq != next[tag.sender]++) {
+        die("order per connection", -1);
+      }
       if (m.data_length != tag.bytes) die("length", -1);
       const uint8_t* got = nullptr;
       if (m.is_rndv) {
-        if (int rc2 = axr_am_recv_buffer(server, m.key, AXR_MEM_HOST, buf.data(), buf.size(), nullptr)) die("recv_buffer", rc2);
+        const int rc2 = axr_am_recv_buffer(server, m.key, AXR_MEM_HOST, buf.data(), buf.size(), nullptr);
+        if (rc2 == AXR_ERR_CANCELED && tag.sender == static_cast<uint32_t>(kSenders) && tag.seq % 2) {
+          cancelled_seen.fetch_add(1);   // cancelled between its header and its fetch
+          continue;
+        }
+        if (rc2) die("recv_buffer", rc2);
         got = buf.data();
       } else {
         got = static_cast<const uint8_t*>(m.eager_data.data);
@@ -105,7 +160,7 @@ int main() {
       if (!m.is_rndv) {
         if (int rc2 = axr_am_message_release(server, m.key)) die("release", rc2);
       }
-      received.fetch_add(1);
+      if (tag.sender < static_cast<uint32_t>(kSenders)) received.fetch_add(1);
     }
   });
   threads.emplace_back([&stop_churn] {   // unrelated contexts come and go

@@ -116,6 +116,89 @@ def test_fifo_order_and_cancel(pkg, pair):
         assert np.array_equal(dst, src[i:i + 5000]) and client.test(reqs[i])
 
 
+def test_at_most_256_sends_in_flight_the_rest_wait_in_order(pkg, pair):
+    """kCompletionQueueEntryCount (ucx_am_context.hpp:94,836-839): 256 operations may be
+    under way; further ones are queued and submitted, first in first out, as completions
+    make room (ucx_am_context.cpp:271-274).  An eager send behind waiting ones keeps its
+    place in the order."""
+    client, server, conn = pair
+    src = pattern(300 * 8 + 5000)
+    total = 300
+    reqs = [client.send(conn, i.to_bytes(2, "little"), src.ctypes.data + 8 * i, 5000, memory_type=HOST)
+            for i in range(total)]
+    assert client.progress() == (256, total - 256)
+    assert server.pending() == 256                           # the others have not been sent yet
+    small = client.send(conn, b"eager", src.ctypes.data, 16, memory_type=HOST)   # below the threshold
+    assert client.progress() == (256, total - 256 + 1) and server.pending() == 256
+    dst = np.zeros(5000, np.uint8)
+    for i in range(10):                                      # ten fetches make room for ten sends
+        m = server.recv_header()
+        assert int.from_bytes(m.header, "little") == i
+        server.recv_into(m, dst.ctypes.data, 5000, memory_type=HOST)
+        assert np.array_equal(dst, src[8 * i:8 * i + 5000])
+    assert server.pending() == 246                           # nothing moves before the sender progresses
+    assert client.test(reqs[0])                              # ... which a test of a request does
+    assert client.progress() == (256, total - 256 + 1 - 10) and server.pending() == 256
+    seen = []
+    while True:
+        m = server.recv_header()
+        if m is None:
+            if client.progress() == (0, 0):
+                break
+            continue
+        if m.is_rndv:
+            seen.append(int.from_bytes(m.header, "little"))
+            server.recv_into(m, dst.ctypes.data, 5000, memory_type=HOST)
+            assert np.array_equal(dst, src[8 * seen[-1]:8 * seen[-1] + 5000])
+        else:
+            seen.append(m.header)
+            assert m.eager_data == bytes(src[:16])
+    assert seen == list(range(10, total)) + [b"eager"]       # the order of the calls
+    assert all(client.test(r) for r in reqs[1:]) and client.test(small)
+
+
+def test_sender_cancels_waiting_and_unfetched_sends(pkg, pair):
+    client, server, conn = pair
+    src = pattern(9000)
+    reqs = [client.send(conn, bytes([i % 251]), src.ctypes.data, 5000, memory_type=HOST) for i in range(260)]
+    assert client.progress() == (256, 4)
+    # a send that still waits for room: dropped before it reaches the peer
+    client.cancel(reqs[258])
+    assert client.progress() == (256, 3)
+    with pytest.raises(pkg.AxonRocmError):
+        client.test(reqs[258])
+    # a rendezvous the receiver has not looked at: it never shows up, and its slot is free again
+    client.cancel(reqs[0])
+    assert client.progress() == (256, 2)                     # 255 + one waiting send started
+    m = server.recv_header()
+    assert m.header == bytes([1])
+    # one the receiver holds the header of: its fetch fails, nothing is copied
+    client.cancel(reqs[1])
+    dst = np.full(5000, 7, np.uint8)
+    with pytest.raises(pkg.AxonRocmError) as e:
+        server.recv_into(m, dst.ctypes.data, 5000, memory_type=HOST)
+    assert e.value.status == pkg._capi.AXR_ERR_CANCELED and (dst == 7).all()
+    # a completed send cannot be cancelled any more
+    m = server.recv_header()
+    assert m.header == bytes([2])
+    server.recv_into(m, dst.ctypes.data, 5000, memory_type=HOST)
+    client.cancel(reqs[2])
+    assert client.test(reqs[2]) and np.array_equal(dst, src[:5000])
+    # the rest arrives in order, without the cancelled ones
+    seen = []
+    while True:
+        m = server.recv_header()
+        if m is None:
+            if client.progress() == (0, 0):
+                break
+            continue
+        seen.append(m.header[0])
+        server.recv_into(m, dst.ctypes.data, 5000, memory_type=HOST)
+    assert seen == [i % 251 for i in range(3, 260) if i != 258]
+    with pytest.raises(pkg.AxonRocmError):
+        client.cancel(10 ** 9)                               # unknown request
+
+
 def test_send_to_a_destroyed_peer_is_an_error(pkg):
     """An endpoint outlives its peer context; sending on it fails cleanly (a closed
     connection is an error_code in the reference, ucx_am_context.hpp:2318-2392) and
