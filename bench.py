@@ -40,7 +40,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--rotate", type=int, default=4,
                     help="independent bundle copies cycled through by the steps (1 = cache resident)")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "transposed"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "transposed", "rows100", "rows250", "rows512", "stepped",
+                             "odd_transposed"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--separate-launches", action="store_true",
                     help="time axr_pack + axr_unpack as two launches per step instead of one axr_submit")
@@ -280,6 +281,52 @@ def make_transposed_sets(h, count, seed=0, n=8, edge=4096):
             workloads.views_of_torch([y.t() for y in dst]), 256, (src, dst),
             check=lambda src=src, dst=dst: all(bool(torch.equal(x.view(torch.int16), y.view(torch.int16)))
                                                for x, y in zip(src, dst))))
+    return sets
+
+
+def _random_storage(torch, shape, dtype, seed):
+    """Random bytes viewed as `dtype` (every bit pattern occurs, NaNs included: the path moves bytes)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    item = torch.empty((), dtype=dtype).element_size()
+    n = 1
+    for e in shape:
+        n *= e
+    return torch.randint(0, 256, (n * item,), dtype=torch.uint8, device="cuda", generator=g).view(dtype).reshape(shape)
+
+
+# Strided views: name -> (description, function(torch, seed) -> list of views of fresh storage)
+VIEW_WORKLOADS = {
+    "rows100": ("fp32 [2M, 64][:, :25]: rows of 100 B at a 256 B pitch (element mode, ragged 16-byte granules)",
+                lambda t, seed: [_random_storage(t, (1 << 21, 64), t.float32, seed)[:, :25]]),
+    "rows250": ("bf16 [1M, 512][:, :125]: rows of 250 B at a 1 KiB pitch (element mode, ragged 16-byte granules)",
+                lambda t, seed: [_random_storage(t, (1 << 20, 512), t.bfloat16, seed)[:, :125]]),
+    "rows512": ("bf16 [512K, 512][:, :256]: rows of 512 B at a 1 KiB pitch (element mode, 16-byte granules)",
+                lambda t, seed: [_random_storage(t, (1 << 19, 512), t.bfloat16, seed)[:, :256]]),
+    "stepped": ("fp32 [16M, 8][:, ::2]: every second element (element mode, 4-byte granules)",
+                lambda t, seed: [_random_storage(t, (1 << 24, 8), t.float32, seed)[:, ::2]]),
+    "odd_transposed": ("4 transposed 4097 x 4099 bf16 matrices (x.t() views; rows straddle 128-byte lines)",
+                       lambda t, seed: [_random_storage(t, (4097, 4099), t.bfloat16, seed + k).t() for k in range(4)]),
+}
+
+
+def make_view_sets(h, count, workload, seed=0):
+    """Bundles of strided torch views, scattered back into views of the same geometry over
+    zeroed storage; the check compares the elements the views address."""
+    import torch
+    from execution_ucx_amd import workloads
+    make = VIEW_WORKLOADS[workload][1]
+    sets = []
+    for k in range(count):
+        src = make(torch, seed + 100 * k)
+        twins = [torch.zeros_like(v._base if v._base is not None else v) for v in src]
+        dst = [tw.as_strided(v.shape, v.stride(), v.storage_offset()) for tw, v in zip(twins, src)]
+
+        def check(src=src, dst=dst):
+            return all(bool(torch.equal(a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8)))
+                       for a, b in zip(src, dst))
+        sets.append(BundleSet(h, workloads.views_of_torch(src), workloads.views_of_torch(dst), 256,
+                              (src, twins, dst), check=check))
     return sets
 
 
@@ -756,6 +803,9 @@ def main():
     elif args.workload == "transposed":
         sets = make_transposed_sets(h, max(1, min(args.rotate, 2)))
         name = "8 transposed 4096 x 4096 bf16 matrices (x.t() views), 256 MiB"
+    elif args.workload in VIEW_WORKLOADS:
+        sets = make_view_sets(h, max(1, min(args.rotate, 2)), args.workload)
+        name = VIEW_WORKLOADS[args.workload][0]
     else:
         sets = make_c5_sets(h, max(1, min(args.rotate, 2)))
         name = "C5 chunk: 64 pitched 2-D views, 256 MiB"
@@ -885,6 +935,16 @@ def main():
                                       "payload_bytes_P": tr[0].data_bytes, "steps": k5}
         del tr
         torch.cuda.empty_cache()
+        strided = {}
+        for wl in VIEW_WORKLOADS:
+            vs = make_view_sets(h, 2, wl)
+            verify_set(h, vs[0])
+            msv = run_sets(h, vs, k5, 5)
+            check_sets(h, vs, wl)
+            strided[wl] = {"GBps": round(rate(vs[0].data_bytes, msv, k5), 1), "payload_bytes_P": vs[0].data_bytes}
+            del vs
+            torch.cuda.empty_cache()
+        extras["strided_views"] = strided
         extras["fresh_small_bundle"] = fresh_small_round_trip(h)
         extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["loopback_iov_vs_bundle"] = iov_against_bundle(h, spec)

@@ -157,7 +157,7 @@ class SegmentInfo(C.Structure):
         ("granule", C.c_uint32),
         ("tiles", C.c_uint32),
         ("head", C.c_uint32),
-        ("reserved", C.c_uint32),
+        ("lanes_per_run", C.c_uint32),
         ("shape", C.c_uint32 * 6),
         ("stride_bytes", C.c_int64 * 6),
     ]

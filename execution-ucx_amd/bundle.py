@@ -171,7 +171,7 @@ class BundlePlan:
             out.append({
                 "tensor": s.tensor, "mode": s.mode, "address": s.address, "offset": s.offset,
                 "run_bytes": s.run_bytes, "nbytes": s.nbytes, "pad": s.pad, "ndim": s.ndim,
-                "granule": s.granule, "tiles": s.tiles, "head": s.head,
+                "granule": s.granule, "tiles": s.tiles, "head": s.head, "lanes_per_run": s.lanes_per_run,
                 "shape": tuple(s.shape[:s.ndim]), "stride_bytes": tuple(s.stride_bytes[:s.ndim]),
             })
         return out

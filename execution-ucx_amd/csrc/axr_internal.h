@@ -91,7 +91,11 @@ struct Dims {             // 176 bytes, one per strided segment
   uint32_t ext_a, ext_b;
   uint32_t tiles_a, tiles_b;
   uint32_t edge_a, edge_b;         // block extent along A and B (elements)
-  uint32_t reserved[2];
+  uint32_t lanes_per_run;          // kModeElements: 0, or the lane slots a ragged run occupies (its
+                                   // 16-byte granules rounded up to a multiple of four)
+  uint32_t nt_allowed;             // kModeTranspose: sides that may keep the launch's non-temporal hint
+                                   // (bit 0 tensor, bit 1 payload); a side whose block rows straddle
+                                   // 128-byte lines shares lines with its neighbours and must stay cacheable
 };
 static_assert(sizeof(Dims) == 176, "Dims layout");
 
@@ -170,7 +174,8 @@ struct Tunables {
   // 16 bytes; other runs of 16 bytes or more up to five eighths of it (ragged
   // granules), anything else up to an eighth (measured crossovers).
   std::atomic<int64_t> gather_run_bytes{2048};
-  std::atomic<int64_t> xcd_remap{0};          // contiguous wave ranges per die (measured slower)
+  std::atomic<int64_t> xcd_remap{-1};         // contiguous wave ranges per die: 1 always, 0 never, -1 when
+                                  // transposed blocks that share lines with their neighbours dominate
   std::atomic<int64_t> transpose{1};          // move transposed views as square blocks through LDS
   std::atomic<int64_t> ragged_runs{1};        // short runs of 16+ bytes that are no multiple of 16 move in
                                   // 16-byte granules (the last one overlapping) instead of narrower ones

@@ -166,13 +166,16 @@ __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32
   for (uint32_t e0 = lane; e0 < ng; e0 += U * kWaveLanes) {
     gbytes tp[U], pp[U];
     T val[U];
+    bool moves[U];
 #pragma unroll
     for (uint32_t u = 0; u < U; ++u) {
       const uint32_t e = e0 + u * kWaveLanes;
-      const uint32_t ec = e < ng ? e : ng - 1u;   // slots past the end repeat the last granule's load
+      const uint32_t ec = e < ng ? e : ng - 1u;   // slots past the end repeat the last slot's load
       uint64_t packed;
-      tp[u] = tbase + decode(ec, &packed);
+      bool live;                                  // false for a slot that pads a run to whole quads
+      tp[u] = tbase + decode(ec, &packed, &live);
       pp[u] = pbase + packed;
+      moves[u] = live && e < ng;
     }
 #pragma unroll
     for (uint32_t u = 0; u < U; ++u)
@@ -183,7 +186,7 @@ __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32
     }
 #pragma unroll
     for (uint32_t u = 0; u < U; ++u) {
-      if (e0 + u * kWaveLanes < ng) *reinterpret_cast<AXR_GLOBAL loose*>(PACK ? pp[u] : tp[u]) = val[u];
+      if (moves[u]) *reinterpret_cast<AXR_GLOBAL loose*>(PACK ? pp[u] : tp[u]) = val[u];
     }
   }
 }
@@ -203,20 +206,26 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   constexpr uint32_t kTile = ROWS * kRowBytes < kMinElementTileBytes ? kMinElementTileBytes : ROWS * kRowBytes;
   const uint32_t g = dm->granule;
   const uint32_t gs = static_cast<uint32_t>(__builtin_ctz(g));
-  // Ragged runs (16 bytes or longer, not a multiple of 16): a run is ceil(run / 16)
-  // granules of 16 bytes and its last granule covers the run's final 16 bytes,
-  // overlapping the one before it with identical data.  Tiles then count
-  // granules, not packed bytes.
-  const bool ragged = dm->tiles_per_run != 0;
+  // Runs of 16 bytes or more that are no whole number of 64-byte quads (ragged runs):
+  // a run is ceil(run / 16) granules of 16 bytes, its last granule covers the run's
+  // final 16 bytes (overlapping the one before it with identical data when the length
+  // is no multiple of 16), and the run occupies `lanes_per_run` lane slots, the granule
+  // count rounded up to a multiple of four: the memory pipeline takes a wave's
+  // 16-byte accesses four lanes at a time, and a group of four that lies in one run
+  // is one 64-byte request where a group that straddles two runs is two.  Slots past a
+  // run's last granule move nothing.  Tiles then count slots, not packed bytes.
+  const uint32_t lpr = dm->lanes_per_run;
+  const bool ragged = lpr != 0;
   const uint32_t run32 = static_cast<uint32_t>(run_bytes);
-  const uint32_t gpr = ragged ? (run32 + 15u) >> 4 : static_cast<uint32_t>(run_bytes >> gs);
+  const uint32_t granules = ragged ? (run32 + 15u) >> 4 : static_cast<uint32_t>(run_bytes >> gs);
+  const uint32_t gpr = ragged ? lpr : granules;   // slots per run
   const uint32_t nd = dm->ndim;
   const uint64_t b0 = static_cast<uint64_t>(q) * kTile;   // exact runs: packed byte of the tile
   uint64_t e0;
   uint32_t ng;
   if (ragged) {
     e0 = static_cast<uint64_t>(q) * (kTile / kVecBytes);
-    const uint64_t left = dm->pstride[0] - e0;            // granules of the whole segment
+    const uint64_t left = dm->pstride[0] - e0;            // slots of the whole segment
     ng = left < kTile / kVecBytes ? static_cast<uint32_t>(left) : kTile / kVecBytes;
   } else {
     const uint64_t left = dm->nbytes - b0;
@@ -250,23 +259,29 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
     }
   }
   const uint32_t gpr_magic = 0xffffffffu / gpr + 1u;
+  const int64_t stride_last = dm->stride[kMaxOuterDims - 1];
   gbytes tbase = as_global(seg_ptr) + base;
   gbytes pbase = ragged ? pay + static_cast<uint64_t>(run0) * run32 : pay + b0;
   // tensor-side byte offset (relative to the tile's first run) of granule e of the
   // tile, and its payload offset (relative to pbase)
-  auto decode = [&](uint32_t e, uint64_t* packed) -> int64_t {
+  auto decode = [&](uint32_t e, uint64_t* packed, bool* live) -> int64_t {
     uint32_t w = w0 + e;
     // w < gpr + tile / g: for gpr <= 2^15, w * gpr < 2^32 and the multiply-high quotient is exact
     uint32_t carry = gpr == 1 ? w : (gpr <= 32768u ? __umulhi(w, gpr_magic) : w / gpr);
     w -= carry * gpr;
     uint32_t in_run = w << gs;
     if (ragged) {
-      in_run = w + 1u == gpr ? run32 - kVecBytes : in_run;
+      *live = w < granules;
+      in_run = w + 1u >= granules ? run32 - kVecBytes : in_run;
       *packed = static_cast<uint64_t>(carry) * run32 + in_run;
     } else {
+      *live = true;
       *packed = static_cast<uint64_t>(e) << gs;
     }
     int64_t toff = static_cast<int64_t>(in_run);
+    if (nd == 1) {   // one strided dimension (rows of a matrix): the run index is the only coordinate
+      return toff + static_cast<int64_t>(carry) * stride_last;
+    }
 #pragma unroll
     for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
       if (static_cast<uint32_t>(d) + nd >= kMaxOuterDims) {
@@ -287,10 +302,9 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
     }
     return toff;
   };
-  // Accesses per lane and round.  16-byte granules measured fastest one at a time
-  // (a 2 KiB tile is two rounds); narrow granules gain from four in flight.
+  // Accesses per lane and round: four in flight.
   switch (g) {
-    case 16: element_moves<PACK, u32x4, 1>(tbase, pbase, ng, lane, decode); break;
+    case 16: element_moves<PACK, u32x4, 4>(tbase, pbase, ng, lane, decode); break;
     case 8: element_moves<PACK, uint64_t, 2>(tbase, pbase, ng, lane, decode); break;
     case 4: element_moves<PACK, uint32_t, 4>(tbase, pbase, ng, lane, decode); break;
     case 2: element_moves<PACK, uint16_t, 4>(tbase, pbase, ng, lane, decode); break;
@@ -656,6 +670,7 @@ __device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_
   const uint32_t E = dm->granule;
   const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
   const uint32_t T = transpose_edge(E);
+  nt_bits &= dm->nt_allowed;   // rows that straddle lines share them with the neighbouring blocks
   const uint32_t edge_a = dm->edge_a, edge_b = dm->edge_b;
   const uint32_t ta = dm->tiles_a, tb = dm->tiles_b;
   const uint32_t per_batch = ta * tb;

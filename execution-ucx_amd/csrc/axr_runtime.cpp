@@ -399,7 +399,7 @@ static int tune_set_body(const char* key, int64_t value) {
       return fail(AXR_ERR_INVALID, "threads must be 0 (auto) or a multiple of 64 in [64, 1024]");
     t.threads = value;
   } else if (k == "xcd_remap") {
-    t.xcd_remap = value ? 1 : 0;
+    t.xcd_remap = value < 0 ? -1 : (value ? 1 : 0);
   } else if (k == "ragged_runs") {
     t.ragged_runs = value ? 1 : 0;
   } else if (k == "host_threads") {

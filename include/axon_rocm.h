@@ -398,7 +398,10 @@ typedef struct axr_segment_info {
   uint32_t head;          /* mode 0: leading bytes (< 128) that the first tile
                              moves on top of its own range, so that the tiles
                              start on a 128-byte line of the written side      */
-  uint32_t reserved;
+  uint32_t lanes_per_run; /* mode 2 with 16-byte granules: lane slots a run occupies
+                             (its granules, the last one covering the run's final 16
+                             bytes, rounded up to a multiple of four); 0: the tiles
+                             count packed bytes                                  */
   uint32_t shape[6];
   int64_t stride_bytes[6];
 } axr_segment_info_t;
@@ -412,7 +415,10 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "tile_rows" (KiB per wavefront tile: 0 auto, 1, 2, 4, 8, 16), "max_tiles",
  * "max_waves", "threads" (workgroup size), "nontemporal" (-1 auto, or bit 0
  * tensor side / bit 1 payload side), "payload_cache_bytes", "gather_run_bytes",
- * "xcd_remap", "transpose" (1: transposed views move as square blocks through
+ * "xcd_remap" (each accelerator die walks one contiguous share of the tiles: 1 always,
+ * 0 never, -1 (default) for bundles made mostly of transposed views whose rows do not
+ * start on 128-byte lines, where neighbouring blocks then meet in one L2),
+ * "transpose" (1: transposed views move as square blocks through
  * LDS; 0: element by element), "ragged_runs" (1: short strided runs whose
  * length is no multiple of 16 bytes still move in 16-byte granules),
  * "head_align" (contiguous tensors longer than a tile start their tiles on a
