@@ -47,6 +47,8 @@ def parse_args():
                     help="time axr_pack + axr_unpack as two launches per step instead of one axr_submit")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--tune", default="", help="comma separated key=value kernel tunables")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="print what the plain copy, fill and row kernels reach on this device and exit")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N plain 256 MiB device copies (axr_copy_reference) so that "
                          "profiler counters can be scaled by a kernel of known traffic")
@@ -761,6 +763,56 @@ def graph_replay(h, sets, P, steps_in_graph=20):
         return f"not measured: {type(e).__name__}: {e}"
 
 
+def ceilings(h):
+    """What plain kernels of the library reach on this device: the copy kernel, the fill kernel
+    and the row gather / scatter kernel (no tables, one 16-byte access per lane) on the row
+    geometries of the strided workloads.  GB/s of bytes read plus bytes written."""
+    torch, lib, check = h.torch, h.lib, h.capi.check
+    out = {"copy_kernel": {}, "fill_kernel": {}, "row_kernel": {}}
+    for label, n in (("48 MB", 47869056), ("405 MB", 404766720), ("1 GiB", 1 << 30)):
+        copies = max(2, int((600 << 20) // (2 * n)) + 1)    # rotating buffers: more than the last-level cache holds
+        a = [torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda") for _ in range(copies)]
+        b = [torch.empty_like(x) for x in a]
+        h.sync()
+        k = max(10, int(4e9 // n))
+        ms = h.time_steps(lambda i: check(lib.axr_copy_reference(b[i % copies].data_ptr(), a[i % copies].data_ptr(),
+                                                                 n, h.stream)), k, 3)
+        out["copy_kernel"][label] = {"GBps": round(2.0 * n * k / (ms * 1e-3) / 1e9, 1), "us_per_launch": round(ms * 1e3 / k, 2),
+                                     "rotating_buffer_pairs": copies}
+        ms = h.time_steps(lambda i: check(lib.axr_memset_async(b[i % copies].data_ptr(), 7, n, h.stream)), k, 3)
+        out["fill_kernel"][label] = {"GBps": round(1.0 * n * k / (ms * 1e-3) / 1e9, 1)}
+        del a, b
+        torch.cuda.empty_cache()
+    for label, run, pitch, rows in (("100 B rows at a 256 B pitch", 100, 256, 1 << 21),
+                                    ("250 B rows at a 1 KiB pitch", 250, 1024, 1 << 20),
+                                    ("512 B rows at a 1 KiB pitch", 512, 1024, 1 << 19),
+                                    ("128 B rows at a 256 B pitch", 128, 256, 1 << 21)):
+        strided = [torch.randint(0, 256, (rows * pitch,), dtype=torch.uint8, device="cuda") for _ in range(2)]
+        packed = [torch.empty(rows * run, dtype=torch.uint8, device="cuda") for _ in range(2)]
+        h.sync()
+        k = 20
+        res = {}
+        for scatter, name in ((0, "gather"), (1, "scatter")):
+            best, every = None, {}
+            for nt in (0, 1, 2, 3):
+                def step(i, scatter=scatter, nt=nt):
+                    check(lib.axr_rows_reference(strided[i % 2].data_ptr(), pitch, packed[i % 2].data_ptr(), run, rows,
+                                                 scatter, nt, h.stream))
+                ms = h.time_steps(step, k, 2)
+                rate_ = 2.0 * rows * run * k / (ms * 1e-3) / 1e9
+                every[str(nt)] = round(rate_, 1)
+                if best is None or rate_ > best[0]:
+                    best = (rate_, nt)
+            res[name] = {"GBps": round(best[0], 1), "nontemporal_bits": best[1], "by_nontemporal_bits": every}
+        g, sc = res["gather"]["GBps"], res["scatter"]["GBps"]
+        res["pair_GBps"] = round(2.0 / (1.0 / g + 1.0 / sc), 1)
+        res["payload_bytes_P"] = rows * run
+        out["row_kernel"][label] = res
+        del strided, packed
+        torch.cuda.empty_cache()
+    return out
+
+
 def load_traffic(kernel_key):
     path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
     try:
@@ -788,6 +840,9 @@ def main():
     h = Harness(pkg)
     from execution_ucx_amd import workloads
 
+    if args.ceilings:
+        print(json.dumps({"ceilings": ceilings(h)}))
+        return
     spec = workloads.mixed_bundle()
     extras = {}
     if args.workload == "c2":

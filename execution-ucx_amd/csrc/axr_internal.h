@@ -93,9 +93,11 @@ struct Dims {             // 176 bytes, one per strided segment
   uint32_t edge_a, edge_b;         // block extent along A and B (elements)
   uint32_t lanes_per_run;          // kModeElements: 0, or the lane slots a ragged run occupies (its
                                    // 16-byte granules rounded up to a multiple of four)
-  uint32_t nt_allowed;             // kModeTranspose: sides that may keep the launch's non-temporal hint
-                                   // (bit 0 tensor, bit 1 payload); a side whose block rows straddle
-                                   // 128-byte lines shares lines with its neighbours and must stay cacheable
+  uint32_t nt_allowed;             // kModeElements, kModeTranspose: sides that may keep the launch's
+                                   // non-temporal hint when packing (bit 0 tensor, bit 1 payload) and when
+                                   // unpacking (bits 2, 3).  Transposed block rows that straddle 128-byte
+                                   // lines share them with the neighbouring blocks and are written through
+                                   // the cache; rows shorter than a line are read and written through it
 };
 static_assert(sizeof(Dims) == 176, "Dims layout");
 
@@ -170,10 +172,10 @@ struct Tunables {
   // last-level cache when the consumer (unpack, or the transport's copy) reads it.
   std::atomic<int64_t> nontemporal{-1};
   std::atomic<int64_t> payload_cache_bytes{256ll << 20};
-  // Strided runs shorter than this use element mode when they are multiples of
-  // 16 bytes; other runs of 16 bytes or more up to five eighths of it (ragged
-  // granules), anything else up to an eighth (measured crossovers).
-  std::atomic<int64_t> gather_run_bytes{2048};
+  // Strided runs shorter than this use element mode when they are 16 bytes or
+  // longer (16-byte granules, exact or ragged), anything else up to a fifth of it
+  // (measured crossovers).
+  std::atomic<int64_t> gather_run_bytes{1280};
   std::atomic<int64_t> xcd_remap{-1};         // contiguous wave ranges per die: 1 always, 0 never, -1 when
                                   // transposed blocks that share lines with their neighbours dominate
   std::atomic<int64_t> transpose{1};          // move transposed views as square blocks through LDS

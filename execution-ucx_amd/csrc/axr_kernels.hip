@@ -15,6 +15,7 @@
 // bundles without them run the small streaming kernels.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstring>
 
 #include "axr_internal.h"
@@ -161,8 +162,11 @@ __device__ __forceinline__ int64_t run_offset(dims_table dm, uint32_t run) {
 // payload offset from pbase.
 template <bool PACK, typename T, uint32_t U, typename DECODE>
 __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32_t ng,
-                                              uint32_t lane, DECODE decode) {
+                                              uint32_t lane, uint32_t nt_bits, DECODE decode) {
   typedef T __attribute__((aligned(1))) loose;   // no alignment promise on either side
+  // cache hints of the side that is read and of the side that is written (wave-uniform; the
+  // empty asm statements keep the arms apart, or the optimizer merges them and drops the hint)
+  const bool nt_rd = (nt_bits & (PACK ? 1u : 2u)) != 0, nt_wr = (nt_bits & (PACK ? 2u : 1u)) != 0;
   for (uint32_t e0 = lane; e0 < ng; e0 += U * kWaveLanes) {
     gbytes tp[U], pp[U];
     T val[U];
@@ -177,16 +181,33 @@ __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32
       pp[u] = pbase + packed;
       moves[u] = live && e < ng;
     }
+    if (nt_rd) {
+      asm volatile("");
 #pragma unroll
-    for (uint32_t u = 0; u < U; ++u)
-      val[u] = *reinterpret_cast<const AXR_GLOBAL loose*>(PACK ? tp[u] : pp[u]);
+      for (uint32_t u = 0; u < U; ++u)
+        val[u] = __builtin_nontemporal_load(reinterpret_cast<const AXR_GLOBAL loose*>(PACK ? tp[u] : pp[u]));
+      asm volatile("");
+    } else {
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u)
+        val[u] = *reinterpret_cast<const AXR_GLOBAL loose*>(PACK ? tp[u] : pp[u]);
+    }
     if constexpr (sizeof(T) == 16) {
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) asm volatile("" : "+v"(val[u])::"memory");
     }
+    if (nt_wr) {
+      asm volatile("");
 #pragma unroll
-    for (uint32_t u = 0; u < U; ++u) {
-      if (moves[u]) *reinterpret_cast<AXR_GLOBAL loose*>(PACK ? pp[u] : tp[u]) = val[u];
+      for (uint32_t u = 0; u < U; ++u) {
+        if (moves[u]) __builtin_nontemporal_store(val[u], reinterpret_cast<AXR_GLOBAL loose*>(PACK ? pp[u] : tp[u]));
+      }
+      asm volatile("");
+    } else {
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u) {
+        if (moves[u]) *reinterpret_cast<AXR_GLOBAL loose*>(PACK ? pp[u] : tp[u]) = val[u];
+      }
     }
   }
 }
@@ -201,7 +222,8 @@ __device__ __forceinline__ void element_moves(gbytes tbase, gbytes pbase, uint32
 // dimension where no lane carries further.
 template <bool PACK, uint32_t ROWS>
 __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_bytes, dims_table dm,
-                                          gbytes pay, uint32_t q, uint32_t lane) {
+                                          gbytes pay, uint32_t q, uint32_t lane, uint32_t nt_bits) {
+  nt_bits &= PACK ? dm->nt_allowed : dm->nt_allowed >> 2;
   // element-mode tiles are at least 8 KiB: the per-tile decode is amortised over more bytes
   constexpr uint32_t kTile = ROWS * kRowBytes < kMinElementTileBytes ? kMinElementTileBytes : ROWS * kRowBytes;
   const uint32_t g = dm->granule;
@@ -304,11 +326,11 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   };
   // Accesses per lane and round: four in flight.
   switch (g) {
-    case 16: element_moves<PACK, u32x4, 4>(tbase, pbase, ng, lane, decode); break;
-    case 8: element_moves<PACK, uint64_t, 2>(tbase, pbase, ng, lane, decode); break;
-    case 4: element_moves<PACK, uint32_t, 4>(tbase, pbase, ng, lane, decode); break;
-    case 2: element_moves<PACK, uint16_t, 4>(tbase, pbase, ng, lane, decode); break;
-    default: element_moves<PACK, uint8_t, 4>(tbase, pbase, ng, lane, decode); break;
+    case 16: element_moves<PACK, u32x4, 4>(tbase, pbase, ng, lane, nt_bits, decode); break;
+    case 8: element_moves<PACK, uint64_t, 2>(tbase, pbase, ng, lane, nt_bits, decode); break;
+    case 4: element_moves<PACK, uint32_t, 4>(tbase, pbase, ng, lane, nt_bits, decode); break;
+    case 2: element_moves<PACK, uint16_t, 4>(tbase, pbase, ng, lane, nt_bits, decode); break;
+    default: element_moves<PACK, uint8_t, 4>(tbase, pbase, ng, lane, nt_bits, decode); break;
   }
 }
 
@@ -670,7 +692,8 @@ __device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_
   const uint32_t E = dm->granule;
   const uint32_t es = static_cast<uint32_t>(__builtin_ctz(E));
   const uint32_t T = transpose_edge(E);
-  nt_bits &= dm->nt_allowed;   // rows that straddle lines share them with the neighbouring blocks
+  // rows that straddle lines share them with the neighbouring blocks
+  nt_bits &= PACK ? dm->nt_allowed : dm->nt_allowed >> 2;
   const uint32_t edge_a = dm->edge_a, edge_b = dm->edge_b;
   const uint32_t ta = dm->tiles_a, tb = dm->tiles_b;
   const uint32_t per_batch = ta * tb;
@@ -692,7 +715,16 @@ __device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_
       o = next;
     }
   }
-  const uint32_t a0 = ia * edge_a, b0 = ib * edge_b;
+  uint32_t a0 = ia * edge_a, b0 = ib * edge_b;
+  if (edge_a == T && edge_b == T) {
+    // Square blocks: the ragged last block of a dimension that holds at least one whole
+    // block is moved back so that it ends at the extent.  It overlaps its neighbour and
+    // moves those elements a second time with the same values, and stays on the vector
+    // path, where the element-per-lane routine would take many times longer than a whole
+    // block (8191 x 8193 bytes: 2.3 -> 5 TB/s).
+    if (a0 + T > dm->ext_a && dm->ext_a >= T) a0 = dm->ext_a - T;
+    if (b0 + T > dm->ext_b && dm->ext_b >= T) b0 = dm->ext_b - T;
+  }
   const uint32_t ra = dm->ext_a - a0, rb = dm->ext_b - b0;
   const uint32_t na = ra < edge_a ? ra : edge_a, nb = rb < edge_b ? rb : edge_b;
   const bool square = na == T && nb == T;   // a whole square block: the vector path
@@ -798,7 +830,7 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
           lbytes lds = (lbytes)lds_slices + (threadIdx.x >> 6) * lds_per_wave;
           transpose_tile<PACK>(seg_ptr, dm, pay, q, lds, lane, nt_bits);
         } else {
-          element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane);
+          element_tile<PACK, ROWS>(seg_ptr, seg_run, dm, pay, q, lane, nt_bits);
         }
       }
       if constexpr (PACK) {
@@ -1023,6 +1055,53 @@ __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__
   const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t nthreads = static_cast<size_t>(gridDim.x) * blockDim.x;
   for (size_t i = tid; i < nvec; i += nthreads) dst[i] = src[i];
+}
+
+// Plain gather or scatter of equally long rows at a constant pitch: one 16-byte access per
+// lane, a row's last access covering its final 16 bytes, every row in a whole number of
+// four-lane groups, four accesses per lane in flight, nothing looked up in a table.  What
+// this kernel reaches is what the access pattern of such a strided view allows.
+template <bool SCATTER, bool NTS, bool NTP>
+__global__ __launch_bounds__(256) void rows_reference_kernel(uint8_t* strided_arg, uint64_t pitch, uint8_t* packed_arg,
+                                                             uint32_t run, uint32_t lanes_per_row,
+                                                             uint32_t rows_per_wave, uint64_t rows) {
+  constexpr uint32_t U = 4;
+  gbytes strided = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(strided_arg));
+  gbytes packed = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(packed_arg));
+  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
+  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const uint64_t row0 = wave * rows_per_wave;
+  if (row0 >= rows) return;
+  const uint32_t granules = (run + kVecBytes - 1) / kVecBytes;
+  const uint32_t magic = 0xffffffffu / lanes_per_row + 1u;   // slots < 2^15: the quotient is exact
+  const uint32_t slots = rows_per_wave * lanes_per_row;
+  for (uint32_t s0 = lane; s0 < slots; s0 += U * kWaveLanes) {
+    gbytes sp[U], pp[U];
+    bool live[U];
+    u32x4 v[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t s = s0 + u * kWaveLanes;
+      const uint32_t r = lanes_per_row == 1 ? s : __umulhi(s, magic);
+      const uint32_t w = s - r * lanes_per_row;
+      const uint64_t row = row0 + r;
+      live[u] = s < slots && w < granules && row < rows;
+      const uint32_t o = (w + 1u >= granules) ? run - kVecBytes : w * kVecBytes;
+      const uint64_t safe_row = live[u] ? row : row0;
+      sp[u] = strided + safe_row * pitch + o;
+      pp[u] = packed + safe_row * run + o;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) v[u] = SCATTER ? load16<NTP>(pp[u]) : load16<NTS>(sp[u]);
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) asm volatile("" : "+v"(v[u])::"memory");
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      if (live[u]) {
+        if constexpr (SCATTER) store16<NTS>(sp[u], v[u]); else store16<NTP>(pp[u], v[u]);
+      }
+    }
+  }
 }
 
 // Tables of a bundle of contiguous device tensors.  The host writes the n + 1 segment
@@ -1362,6 +1441,42 @@ static int copy_reference_body(void* dst, const void* src, size_t bytes, void* s
 }
 int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream) {
   return guarded([&] { return copy_reference_body(dst, src, bytes, stream); });
+}
+
+static int rows_reference_body(void* strided, size_t pitch, void* packed, size_t run_bytes, size_t rows,
+                               int scatter, uint32_t nontemporal, void* stream) {
+  if (rows == 0) return AXR_OK;
+  if (!strided || !packed) return fail(AXR_ERR_INVALID, "axr_rows_reference: null range");
+  if (run_bytes < kVecBytes || run_bytes > 4096 || pitch < run_bytes)
+    return fail(AXR_ERR_INVALID, "axr_rows_reference: rows of 16 to 4096 bytes at a pitch of at least their length");
+  const uint32_t granules = static_cast<uint32_t>((run_bytes + kVecBytes - 1) / kVecBytes);
+  const uint32_t lanes_per_row = (granules + 3u) & ~3u;
+  const uint32_t rows_per_wave = std::max(1u, 512u / lanes_per_row);   // about 8 KiB per wavefront
+  const uint64_t waves = (static_cast<uint64_t>(rows) + rows_per_wave - 1) / rows_per_wave;
+  const uint64_t groups = (waves + 3) / 4;
+  if (groups > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "axr_rows_reference: too many rows for one launch");
+  const dim3 grid(static_cast<uint32_t>(groups)), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define AXR_ROWS(SC, A, B)                                                                              \
+  hipLaunchKernelGGL((rows_reference_kernel<SC, A, B>), grid, block, 0, st, static_cast<uint8_t*>(strided), \
+                     static_cast<uint64_t>(pitch), static_cast<uint8_t*>(packed),                        \
+                     static_cast<uint32_t>(run_bytes), lanes_per_row, rows_per_wave, static_cast<uint64_t>(rows))
+  switch ((scatter ? 4u : 0u) | (nontemporal & 3u)) {
+    case 0: AXR_ROWS(false, false, false); break;
+    case 1: AXR_ROWS(false, true, false); break;
+    case 2: AXR_ROWS(false, false, true); break;
+    case 3: AXR_ROWS(false, true, true); break;
+    case 4: AXR_ROWS(true, false, false); break;
+    case 5: AXR_ROWS(true, true, false); break;
+    case 6: AXR_ROWS(true, false, true); break;
+    default: AXR_ROWS(true, true, true); break;
+  }
+#undef AXR_ROWS
+  return check_hip(hipGetLastError(), "rows_reference launch");
+}
+int axr_rows_reference(void* strided, size_t pitch, void* packed, size_t run_bytes, size_t rows, int scatter,
+                       uint32_t nontemporal, void* stream) {
+  return guarded([&] { return rows_reference_body(strided, pitch, packed, run_bytes, rows, scatter, nontemporal, stream); });
 }
 
 }  // extern "C"

@@ -595,6 +595,17 @@ AXR_API int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_
  * reference for profiler counters and bandwidth. */
 AXR_API int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream);
 
+/* Plain gather (scatter == 0) or scatter of `rows` rows of run_bytes bytes that lie
+ * `pitch` bytes apart at `strided` and back to back at `packed`: one 16-byte access per
+ * lane, no tables, nothing decoded beyond a division.  Calibration reference for what the
+ * access pattern of a strided view allows (rows that cover parts of 128-byte lines cost
+ * whole lines when read and partial-line writes when written), next to which the bundle
+ * kernel's element mode is judged.  16 <= run_bytes <= 4096, pitch >= run_bytes;
+ * `nontemporal` bit 0 marks the strided side's accesses as streaming, bit 1 the packed
+ * side's.  No counterpart in the reference. */
+AXR_API int axr_rows_reference(void* strided, size_t pitch, void* packed, size_t run_bytes,
+                               size_t rows, int scatter, uint32_t nontemporal, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1297,3 +1297,32 @@ def test_pool_and_copy_table(pkg, gpu):
         mr.deallocate(t, ptr, src.size)
     with pkg.rocm(0).activate() as devobj:
         assert devobj.get_type_string() == "rocm" and devobj.get_context_handle() == 0
+
+
+@pytest.mark.parametrize("nontemporal", [0, 3])
+def test_rows_reference_kernel(pkg, gpu, nontemporal):
+    """The plain row gather / scatter kernel (the calibration reference of the strided modes)
+    against numpy slicing: ragged and exact row lengths, rows that fill their pitch, and a
+    scatter that leaves every byte between the rows alone."""
+    import torch
+    lib, check = pkg._capi.load(), pkg._capi.check
+    rng = np.random.default_rng(17)
+    for run, pitch, rows in ((100, 256, 1000), (250, 1024, 333), (16, 16, 7), (4096, 4100, 5),
+                             (48, 64, 129), (17, 33, 1025), (2049, 2304, 3), (128, 128, 4097)):
+        host = rng.integers(0, 256, size=rows * pitch, dtype=np.uint8)
+        strided = torch.from_numpy(host).to(gpu)
+        packed = device_bytes(rows * run + 32, gpu)
+        check(lib.axr_rows_reference(strided.data_ptr(), pitch, packed.data_ptr(), run, rows, 0, nontemporal, None))
+        torch.cuda.synchronize()
+        want = host.reshape(rows, pitch)[:, :run].reshape(-1)
+        got = packed.cpu().numpy()
+        assert np.array_equal(got[:rows * run], want), (run, pitch, rows)
+        assert (got[rows * run:] == POISON).all()
+        twin = device_bytes(rows * pitch, gpu, fill=0xAB)
+        check(lib.axr_rows_reference(twin.data_ptr(), pitch, packed.data_ptr(), run, rows, 1, nontemporal, None))
+        torch.cuda.synchronize()
+        expect = np.full(rows * pitch, 0xAB, np.uint8)
+        expect.reshape(rows, pitch)[:, :run] = want.reshape(rows, run)
+        assert np.array_equal(twin.cpu().numpy(), expect), (run, pitch, rows)
+    with pytest.raises(Exception):
+        check(lib.axr_rows_reference(strided.data_ptr(), 8, packed.data_ptr(), 16, 1, 0, 0, None))

@@ -228,7 +228,7 @@ def seg_of(pkg, view, align=256, **tune):
         return plan.segments(), plan.launch_info()
     finally:
         if tune:
-            pkg.tune(tile_rows=0, gather_run_bytes=2048, transpose=1, ragged_runs=1)
+            pkg.tune(tile_rows=0, gather_run_bytes=1280, transpose=1, ragged_runs=1)
 
 
 def test_compact_tensor_is_one_run(pkg):
@@ -282,22 +282,27 @@ def test_short_runs_use_element_mode(pkg):
     assert segs[0]["mode"] == 1
     segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 304], strides=[1000, 1]), gather_run_bytes=305)
     assert segs[0]["mode"] == 2 and segs[0]["granule"] == 16
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=480)
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=300)
     assert segs[0]["mode"] == 1
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=488)
-    assert segs[0]["mode"] == 2 and segs[0]["granule"] == 16          # ragged: below 5/8 of it
-    # without ragged granules, runs that are no multiple of 16 switch at an eighth of it
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2400,
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=301)
+    assert segs[0]["mode"] == 2 and segs[0]["granule"] == 16          # ragged granules: the same limit
+    assert segs[0]["lanes_per_run"] == 20                             # 19 granules in five groups of four lanes
+    # without ragged granules, runs that are no multiple of 16 switch at a fifth of it
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=1496,
                      ragged_runs=0)
     assert segs[0]["mode"] == 1
-    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=2408,
+    segs, _ = seg_of(pkg, tv(pkg, 0x10000, [5, 300], strides=[1000, 1]), gather_run_bytes=1501,
                      ragged_runs=0)
     assert segs[0]["mode"] == 2 and segs[0]["granule"] == 4
-    # defaults: 2 KiB
-    assert seg_of(pkg, tv(pkg, 0x10000, [5, 2032], strides=[4000, 1]))[0][0]["mode"] == 2
-    assert seg_of(pkg, tv(pkg, 0x10000, [5, 2048], strides=[4000, 1]))[0][0]["mode"] == 1
+    # defaults: 1280 bytes
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 1264], strides=[4000, 1]))[0][0]["mode"] == 2
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 1280], strides=[4000, 1]))[0][0]["mode"] == 1
     assert seg_of(pkg, tv(pkg, 0x10000, [5, 1279], strides=[4000, 1]))[0][0]["mode"] == 2
     assert seg_of(pkg, tv(pkg, 0x10000, [5, 1281], strides=[4000, 1]))[0][0]["mode"] == 1
+    # runs of a whole number of 64-byte groups keep counting packed bytes; others pad to four lanes
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 128], strides=[4000, 1]))[0][0]["lanes_per_run"] == 0
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 112], strides=[4000, 1]))[0][0]["lanes_per_run"] == 8
+    assert seg_of(pkg, tv(pkg, 0x10000, [5, 100], strides=[4000, 1]))[0][0]["lanes_per_run"] == 8
     assert seg_of(pkg, tv(pkg, 0x10000, [5, 260], strides=[4000, 1]), ragged_runs=0)[0][0]["mode"] == 1
 
 
