@@ -216,6 +216,15 @@ void host_copy(const HostCopyJob* jobs, size_t count);
 // True for a handle that axr_stream_destroy has destroyed (and no later
 // axr_stream_create has returned again).
 bool stream_retired(void* stream);
+// Launch marks order what the library enqueues, process-wide.  A launch takes a mark after
+// it has been enqueued; a wait reads the current mark before it starts, and once it has seen
+// the stream drain, every launch on that stream with a mark up to that value is known to be
+// finished, so that a plan released next need not wait for the stream again.
+uint64_t stream_mark_launch();
+uint64_t stream_launch_mark();
+void stream_note_drained(void* stream, uint64_t mark);
+bool stream_drained(void* stream, uint64_t mark);
+void stream_forget(void* stream);   // the stream is being destroyed
 int fail_nothrow(int status, const char* message) noexcept;
 
 // Every extern "C" entry point runs its body through this: no C++ exception
@@ -268,6 +277,11 @@ struct TableBlock {
 };
 int table_block_acquire(size_t bytes, TableBlock* block);
 void table_block_release(TableBlock* block);
+// Events without timing for the current device, recycled: creating one costs more than a
+// microsecond, and every fresh plan that uploads tables needs one.  An event goes back
+// only once it has fired (or was never recorded).
+int event_acquire(void** event, int* device);
+void event_release(void* event, int device);
 
 }  // namespace axr
 

@@ -19,6 +19,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -29,6 +30,55 @@
 using namespace axr;
 
 namespace {
+
+// Storage the planner fills itself: growing it initialises nothing (a std::vector would
+// clear hundreds of kilobytes per plan that the next loop overwrites), and elements are
+// plain records.
+template <typename T>
+class RawVec {
+ public:
+  RawVec() = default;
+  RawVec(const RawVec&) = delete;
+  RawVec& operator=(const RawVec&) = delete;
+  ~RawVec() { std::free(ptr_); }
+  size_t size() const { return n_; }
+  size_t capacity() const { return cap_; }
+  bool empty() const { return n_ == 0; }
+  T* data() { return ptr_; }
+  const T* data() const { return ptr_; }
+  T& operator[](size_t i) { return ptr_[i]; }
+  const T& operator[](size_t i) const { return ptr_[i]; }
+  T* begin() { return ptr_; }
+  T* end() { return ptr_ + n_; }
+  const T* begin() const { return ptr_; }
+  const T* end() const { return ptr_ + n_; }
+  void clear() { n_ = 0; }
+  void reserve(size_t m) {
+    if (m <= cap_) return;
+    if (m > SIZE_MAX / sizeof(T)) throw std::bad_alloc();
+    T* q = static_cast<T*>(std::realloc(ptr_, m * sizeof(T)));
+    if (!q) throw std::bad_alloc();
+    ptr_ = q;
+    cap_ = m;
+  }
+  void resize(size_t m) {   // new elements hold whatever the memory held
+    reserve(m);
+    n_ = m;
+  }
+  void assign(const T* first, const T* last) {
+    resize(static_cast<size_t>(last - first));
+    if (n_) std::memcpy(ptr_, first, n_ * sizeof(T));
+  }
+  void swap(RawVec& o) {
+    std::swap(ptr_, o.ptr_);
+    std::swap(n_, o.n_);
+    std::swap(cap_, o.cap_);
+  }
+
+ private:
+  T* ptr_ = nullptr;
+  size_t n_ = 0, cap_ = 0;
+};
 
 constexpr uint32_t kMagic = 0x42545841u;
 constexpr uint16_t kVersion = 1;
@@ -113,12 +163,12 @@ inline int nbytes_rule(int32_t ndim, const int64_t* shape, uint8_t bits, uint64_
 
 struct axr_plan {
   uint32_t align = 1;
-  std::vector<TensorRec> tensors;
+  RawVec<TensorRec> tensors;
   std::vector<int64_t> dims64;       // shapes and strides of all tensors
-  std::vector<TensorRec> staged_tensors;   // axr_plan_bind fills these and swaps on success
+  RawVec<TensorRec> staged_tensors;  // axr_plan_bind fills these and swaps on success
   std::vector<int64_t> staged_dims64;
   uint64_t payload_bytes = 0, data_bytes = 0;
-  std::vector<uint8_t> header;
+  RawVec<uint8_t> header;
   bool bound = false;
   bool receiver = false;             // made by axr_plan_from_header: tiles are anchored on the tensor side
 
@@ -146,9 +196,14 @@ struct axr_plan {
   std::unique_ptr<InlineTables> inline_tables;   // the tables as a kernel argument (small bundles)
   bool inline_ready = false;
   uint64_t launches = 0;             // kernel launches since the tables were built
-  hipEvent_t upload_event = nullptr;
+  hipEvent_t upload_event = nullptr;   // from event_acquire
+  int upload_event_device = -1;
   hipStream_t upload_stream = nullptr;
-  std::vector<hipStream_t> busy_streams;   // streams with launches since the last quiesce
+  struct BusyStream {
+    hipStream_t stream;
+    uint64_t mark;   // stream_mark_launch() of the plan's latest launch there
+  };
+  std::vector<BusyStream> busy_streams;    // streams with launches since the last quiesce
 
   const int64_t* shape_of(const TensorRec& t) const { return dims64.data() + t.shape_at; }
   const int64_t* strides_of(const TensorRec& t) const {
@@ -194,9 +249,9 @@ void plan_delete(axr_plan* p) {
     v.clear();
     return v.capacity() * sizeof(v[0]);
   };
-  std::vector<TensorRec> tensors, tensors2;
+  RawVec<TensorRec> tensors, tensors2;
   std::vector<int64_t> dims64, dims64_2;
-  std::vector<uint8_t> header;
+  RawVec<uint8_t> header;
   std::vector<Seg> segs;
   std::vector<Dims> dims;
   std::vector<uint32_t> wave_seg;
@@ -292,16 +347,36 @@ void invalidate_tables(axr_plan* p) {
 // stream's work has finished, so the whole device is drained for it.
 void quiesce(axr_plan* p) {
   bool whole_device = false;
-  for (hipStream_t s : p->busy_streams) {
+  for (const axr_plan::BusyStream& b : p->busy_streams) {
+    hipStream_t s = b.stream;
     if (s && stream_retired(s)) {
       whole_device = true;
-    } else if (hipStreamSynchronize(s) != hipSuccess) {
-      (void)hipGetLastError();
-      whole_device = true;
+    } else if (stream_drained(s, b.mark)) {
+      // axr_stream_synchronize has seen the stream pass the plan's last launch
+    } else {
+      const uint64_t reached = stream_launch_mark();
+      if (hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        whole_device = true;
+      } else {
+        stream_note_drained(s, reached);
+      }
     }
   }
   if (whole_device) (void)hipDeviceSynchronize();
   p->busy_streams.clear();
+}
+
+// The plan has just enqueued work on `stream`.
+void remember_stream(axr_plan* p, hipStream_t stream) {
+  const uint64_t mark = stream_mark_launch();
+  for (axr_plan::BusyStream& b : p->busy_streams) {
+    if (b.stream == stream) {
+      b.mark = mark;
+      return;
+    }
+  }
+  p->busy_streams.push_back({stream, mark});
 }
 
 // ------------------------------------------------------------ table building
@@ -743,13 +818,12 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
                                 reinterpret_cast<uint32_t*>(d + wave_at), p->cfg.seg_shift, stream);
   if (rc) return rc;
   if (!p->upload_event) {
-    rc = check_hip(hipEventCreateWithFlags(&p->upload_event, hipEventDisableTiming), "hipEventCreate");
+    rc = event_acquire(reinterpret_cast<void**>(&p->upload_event), &p->upload_event_device);
     if (rc) return rc;
   }
   rc = check_hip(hipEventRecord(p->upload_event, stream), "hipEventRecord");
   if (rc) return rc;
-  if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
-    p->busy_streams.push_back(stream);
+  remember_stream(p, stream);
   p->upload_stream = stream;
   p->uploaded = true;
   p->device_built = true;
@@ -921,8 +995,7 @@ int ensure_uploaded(axr_plan* p, hipStream_t stream) {
                        "hipMemcpyAsync(plan tables)");
     if (rc) return rc;
     if (!p->upload_event) {
-      rc = check_hip(hipEventCreateWithFlags(&p->upload_event, hipEventDisableTiming),
-                     "hipEventCreate");
+      rc = event_acquire(reinterpret_cast<void**>(&p->upload_event), &p->upload_event_device);
       if (rc) return rc;
     }
     rc = check_hip(hipEventRecord(p->upload_event, stream), "hipEventRecord");
@@ -1082,8 +1155,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
     if (delta != 0)
       return fail(AXR_ERR_UNSUPPORTED, "a tensor address delta cannot be applied to host (kDLCPU) tensors");
     rc = move_host_tensors(p, pack, static_cast<uint8_t*>(payload), stream);
-    if (std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
-      p->busy_streams.push_back(stream);
+    remember_stream(p, stream);
     if (rc) return rc;
   }
   if (p->ntiles == 0) return AXR_OK;
@@ -1113,9 +1185,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
     // The launch needs nothing of the plan any more, but callers rely on axr_plan_free and
     // axr_plan_bind returning only when the plan's launches are done (they release the
     // payload or the tensors next), so the stream is remembered all the same.
-    if (!capturing &&
-        std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
-      p->busy_streams.push_back(stream);
+    if (!capturing) remember_stream(p, stream);
     return AXR_OK;
   }
   if (capturing && !p->resident)
@@ -1133,9 +1203,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   ++p->launches;
   // a capturing stream cannot be drained later; the caller keeps the plan alive
   // for as long as the graph can run
-  if (!capturing &&
-      std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
-    p->busy_streams.push_back(stream);
+  if (!capturing) remember_stream(p, stream);
   return AXR_OK;
 }
 
@@ -1149,6 +1217,7 @@ int store_tensor(std::vector<int64_t>& dims64, const axr_tensor_t& in, TensorRec
   int rc = nbytes_rule(in.ndim, in.shape, in.dtype_bits, &rec->nbytes);
   if (rc) return rc;
   rec->shape_at = static_cast<uint32_t>(dims64.size());
+  rec->strides_at = 0;
   rec->has_strides = in.strides != nullptr && in.ndim > 0;
   if (in.ndim == 1) {
     dims64.push_back(in.shape[0]);
@@ -1194,18 +1263,11 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_create: out of host memory");
   p->align = align;
   p->tensors.resize(n);
-  size_t ndims = 0, shape_words = 0;
-  for (size_t i = 0; i < n; ++i) {
-    if (tensors[i].ndim > 0 && tensors[i].ndim <= kMaxNdim) {
-      shape_words += static_cast<size_t>(tensors[i].ndim);
-      ndims += (tensors[i].strides ? 2 : 1) * static_cast<size_t>(tensors[i].ndim);
-    }
-  }
   p->dims64.clear();
-  p->dims64.reserve(ndims);
-  // one pass: tensor record, layout and header record
-  std::vector<uint8_t>& h = p->header;
-  h.resize(kFixedHeader + n * kTensorHeader + 8 * shape_words);
+  p->dims64.reserve(2 * n);
+  // one pass: tensor record, layout and header record (the header grows as shapes come in)
+  RawVec<uint8_t>& h = p->header;
+  h.resize(kFixedHeader + n * (kTensorHeader + 16));
   uint8_t* w = h.data() + kFixedHeader;
   uint64_t off = 0, data = 0, end = 0;
   const uint64_t mask = static_cast<uint64_t>(align) - 1;
@@ -1215,6 +1277,15 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
     if (rc) {
       plan_delete(p);
       return rc;
+    }
+    {
+      // room for this record and every fixed part still to come
+      const size_t at = static_cast<size_t>(w - h.data());
+      const size_t need = at + 8 * static_cast<size_t>(t.ndim) + (n - i) * kTensorHeader;
+      if (need > h.size()) {
+        h.resize(std::max(need, h.size() + h.size() / 2));
+        w = h.data() + at;
+      }
     }
     if (__builtin_add_overflow(off, mask, &off) || (off &= ~mask, __builtin_add_overflow(off, t.nbytes, &end))) {
       plan_delete(p);
@@ -1235,11 +1306,15 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
     rec.byte_offset = 0;   // the packed copy starts at its offset
     std::memcpy(w, &rec, kTensorHeader);
     w += kTensorHeader;
-    if (t.ndim) {
+    if (t.ndim == 1) {   // the common case without a call
+      std::memcpy(w, tensors[i].shape, 8);
+      w += 8;
+    } else if (t.ndim) {
       std::memcpy(w, tensors[i].shape, 8 * static_cast<size_t>(t.ndim));
       w += 8 * static_cast<size_t>(t.ndim);
     }
   }
+  h.resize(static_cast<size_t>(w - h.data()));
   p->payload_bytes = end;
   p->data_bytes = data;
   encode_preamble(p);
@@ -1260,7 +1335,8 @@ static int plan_free_body(axr_plan_t* plan) {
   quiesce(plan);
   if (plan->uploaded && plan->upload_event) (void)hipEventSynchronize(plan->upload_event);
   table_block_release(&plan->block);
-  if (plan->upload_event) (void)hipEventDestroy(plan->upload_event);
+  event_release(plan->upload_event, plan->upload_event_device);   // fired, or never recorded
+  plan->upload_event = nullptr;
   for (HostStage& st : plan->stage) {
     table_block_release(&st.block);
     if (st.ready) (void)hipEventDestroy(st.ready);
@@ -1399,6 +1475,9 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
     uint64_t rule = 0;
     int sized;
     if (!binding) {
+      t.address = 0;
+      t.strides_at = 0;
+      t.has_strides = false;
       t.shape_at = static_cast<uint32_t>(p->dims64.size());
       if (t.ndim == 1) {
         p->dims64.push_back(get<int64_t>(h + at));
@@ -1409,7 +1488,11 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
       sized = nbytes_rule(t.ndim, p->dims64.data() + t.shape_at, t.bits, &rule);
     } else {
       int64_t sent_shape[kMaxNdim];   // the record's shape is only checked; the bound tensor's is kept
-      std::memcpy(sent_shape, h + at, 8 * static_cast<size_t>(t.ndim));
+      if (t.ndim == 1) {
+        std::memcpy(sent_shape, h + at, 8);
+      } else {
+        std::memcpy(sent_shape, h + at, 8 * static_cast<size_t>(t.ndim));
+      }
       sized = nbytes_rule(t.ndim, sent_shape, t.bits, &rule);
     }
     at += static_cast<size_t>(t.ndim) * 8;
@@ -1473,7 +1556,7 @@ static int plan_bind_body(axr_plan_t* plan, const axr_tensor_t* tensors, size_t 
   if (n && !tensors) return fail(AXR_ERR_INVALID, "axr_plan_bind: null tensor array");
   // Everything is validated and staged first (in vectors the plan keeps for this): a
   // failure leaves the plan as it was.
-  std::vector<TensorRec>& recs = plan->staged_tensors;
+  RawVec<TensorRec>& recs = plan->staged_tensors;
   std::vector<int64_t>& dims64 = plan->staged_dims64;
   recs.resize(n);
   dims64.clear();
@@ -1566,9 +1649,7 @@ static int pack_noalloc_body(axr_plan_t* p, void* payload, size_t payload_bytes,
   a.xcd_remap = p->cfg.xcd_remap ? p->cfg.workgroups / kXcds : 0;
   a.seg_shift = p->cfg.seg_shift;
   auto remember = [&] {
-    if (!capturing &&
-        std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
-      p->busy_streams.push_back(stream);
+    if (!capturing) remember_stream(p, stream);
   };
   if (tables_fit_kernel_arguments(p)) {
     if (!p->inline_ready) fill_inline_tables(p);
@@ -1726,9 +1807,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     for (size_t k = i; k < end; ++k) {
       axr_plan* p = jobs[k].plan;
       ++p->launches;
-      if (!capturing &&
-          std::find(p->busy_streams.begin(), p->busy_streams.end(), stream) == p->busy_streams.end())
-        p->busy_streams.push_back(stream);
+      if (!capturing) remember_stream(p, stream);
     }
     i = end;
   }

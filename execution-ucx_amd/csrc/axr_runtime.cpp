@@ -97,6 +97,47 @@ size_t bucket_bytes(size_t bytes) {
 }
 }  // namespace
 
+namespace {
+std::mutex g_event_mutex;
+std::unordered_map<int, std::vector<hipEvent_t>> g_idle_events;   // per device
+constexpr size_t kMaxIdleEvents = 64;
+}  // namespace
+
+int event_acquire(void** event, int* device) {
+  int dev = -1;
+  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc) return rc;
+  {
+    std::lock_guard<std::mutex> lock(g_event_mutex);
+    std::vector<hipEvent_t>& idle = g_idle_events[dev];
+    if (!idle.empty()) {
+      *event = idle.back();
+      *device = dev;
+      idle.pop_back();
+      return AXR_OK;
+    }
+  }
+  hipEvent_t e = nullptr;
+  rc = check_hip(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
+  if (rc) return rc;
+  *event = e;
+  *device = dev;
+  return AXR_OK;
+}
+
+void event_release(void* event, int device) {
+  if (!event) return;
+  {
+    std::lock_guard<std::mutex> lock(g_event_mutex);
+    std::vector<hipEvent_t>& idle = g_idle_events[device];
+    if (idle.size() < kMaxIdleEvents) {
+      idle.push_back(static_cast<hipEvent_t>(event));
+      return;
+    }
+  }
+  (void)hipEventDestroy(static_cast<hipEvent_t>(event));
+}
+
 int table_block_acquire(size_t bytes, TableBlock* block) {
   int dev = 0;
   int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
@@ -199,6 +240,30 @@ namespace {
 std::mutex g_stream_mutex;
 std::unordered_set<void*> g_retired_streams;
 }  // namespace
+
+namespace axr {
+namespace {
+std::atomic<uint64_t> g_launch_mark{0};
+std::mutex g_drained_mutex;
+std::unordered_map<void*, uint64_t> g_drained;   // stream -> highest mark seen drained
+}  // namespace
+uint64_t stream_mark_launch() { return g_launch_mark.fetch_add(1, std::memory_order_seq_cst) + 1; }
+uint64_t stream_launch_mark() { return g_launch_mark.load(std::memory_order_seq_cst); }
+void stream_note_drained(void* stream, uint64_t mark) {
+  std::lock_guard<std::mutex> lock(g_drained_mutex);
+  uint64_t& seen = g_drained[stream];
+  if (mark > seen) seen = mark;
+}
+bool stream_drained(void* stream, uint64_t mark) {
+  std::lock_guard<std::mutex> lock(g_drained_mutex);
+  auto it = g_drained.find(stream);
+  return it != g_drained.end() && it->second >= mark;
+}
+void stream_forget(void* stream) {
+  std::lock_guard<std::mutex> lock(g_drained_mutex);
+  g_drained.erase(stream);
+}
+}  // namespace axr
 
 namespace axr {
 bool stream_retired(void* stream) {
@@ -554,15 +619,20 @@ static int stream_destroy_body(void* stream) {
     std::lock_guard<std::mutex> lock(g_stream_mutex);
     g_retired_streams.insert(stream);
   }
+  stream_forget(stream);
   return check_hip(hipStreamDestroy(static_cast<hipStream_t>(stream)), "hipStreamDestroy");
 }
 int axr_stream_destroy(void* stream) {
   return guarded([&] { return stream_destroy_body(stream); });
 }
 
+
 static int stream_synchronize_body(void* stream) {
-  return check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)),
-                   "hipStreamSynchronize");
+  const uint64_t reached = stream_launch_mark();
+  int rc = check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "hipStreamSynchronize");
+  if (rc) return rc;
+  stream_note_drained(stream, reached);   // plans released next need not wait for this stream again
+  return AXR_OK;
 }
 int axr_stream_synchronize(void* stream) {
   return guarded([&] { return stream_synchronize_body(stream); });
