@@ -48,6 +48,13 @@ class BundlePlan {
     Check(axr_plan_from_header(header, length, &p.plan_), "axr_plan_from_header");
     return p;
   }
+  // The receiver's plan in one pass over the header: decoded and bound to the destination
+  // tensors (a memory policy that answers from buffers it already holds).
+  static BundlePlan FromHeaderBind(const void* header, size_t length, const axr_tensor_t* tensors, size_t n) {
+    BundlePlan p;
+    Check(axr_plan_from_header_bind(header, length, tensors, n, &p.plan_), "axr_plan_from_header_bind");
+    return p;
+  }
   ~BundlePlan() { reset(); }
   BundlePlan(BundlePlan&& o) noexcept : plan_(o.plan_) { o.plan_ = nullptr; }
   BundlePlan& operator=(BundlePlan&& o) noexcept {
@@ -218,6 +225,46 @@ inline std::vector<std::vector<uint8_t>> PayloadToHost(const void* header, size_
   plan.unpack(payload, payload_bytes, stream);
   return out;
 }
+
+// Several gathers and scatters handed over together (a worker with requests to send and
+// responses to scatter at the same moment, axon/src/axon_worker.cpp:1424-1490 next to
+// :1098-1219): neighbouring jobs share one kernel launch.  The jobs must not depend on each
+// other.
+inline void SubmitBundles(const std::vector<axr_job_t>& jobs, void* stream) {
+  Check(axr_submit(jobs.data(), jobs.size(), stream), "axr_submit");
+}
+inline axr_job_t PackJob(const BundlePlan& plan, void* payload, size_t bytes, int64_t tensor_delta = 0) {
+  return axr_job_t{plan.get(), 0, payload, bytes, tensor_delta, 0, 0};
+}
+inline axr_job_t UnpackJob(const BundlePlan& plan, const void* payload, size_t bytes, int64_t tensor_delta = 0) {
+  return axr_job_t{plan.get(), 1, const_cast<void*>(payload), bytes, tensor_delta, 0, 0};
+}
+
+// A large payload moved in chunks of one geometry: pack -> connection_send ->
+// connection_recv_buffer -> unpack per chunk, the chunks double-buffered over `lanes` pairs
+// of slots from the manager's pool (ucx_am_context.hpp:2234-2642 and :1511-1844 are the two
+// ends of the wire; here a loopback pair stands in for it).  ONE sender plan and ONE receiver
+// plan serve every chunk: Submit says how far this chunk's tensors lie from the ones the
+// plans are bound to, and never plans, uploads or allocates.
+class StreamedTransfer {
+ public:
+  StreamedTransfer(ucxx::UcxRocmMemoryResourceManager& mr, size_t slot_bytes, int lanes = 2, int streams = 1) {
+    Check(axr_transfer_create(mr.pool(), slot_bytes, lanes, streams, &transfer_), "axr_transfer_create");
+  }
+  ~StreamedTransfer() {
+    if (transfer_) (void)axr_transfer_destroy(transfer_);
+  }
+  StreamedTransfer(const StreamedTransfer&) = delete;
+  StreamedTransfer& operator=(const StreamedTransfer&) = delete;
+  void Submit(const BundlePlan& send, int64_t send_delta, const BundlePlan& recv, int64_t recv_delta) {
+    Check(axr_transfer_submit(transfer_, send.get(), send_delta, recv.get(), recv_delta), "axr_transfer_submit");
+  }
+  // Returns when every submitted chunk has arrived in its destination tensors.
+  void Finish() { Check(axr_transfer_finish(transfer_), "axr_transfer_finish"); }
+
+ private:
+  axr_transfer_t* transfer_ = nullptr;
+};
 
 // Zero-copy receive: views into the payload at the header's offsets.
 inline std::vector<ucx_buffer_t> SplitPayload(const void* header, size_t header_length, void* payload,

@@ -3,6 +3,7 @@
 // behaviour on a machine without one.  Prints "host_selftest ok" and exits 0.
 #include <cstdio>
 #include <cstdlib>
+#include <algorithm>
 #include <cstring>
 #include <numeric>
 #include <thread>
@@ -192,6 +193,61 @@ int main(int argc, char** argv) {
       EXPECT(mr.stats().live_blocks == 2);
       mr.deallocate(ucx_memory_type::ROCM, kept, kept_bytes);
       mr.deallocate(ucx_memory_type::ROCM, seg, fill.size());
+      EXPECT(mr.stats().live_blocks == 0);
+    }
+
+    // a payload streamed in chunks of one geometry: one pair of plans, moved over the
+    // chunks by address deltas; then two independent bundles in one launch
+    {
+      const size_t chunk = 1u << 20, chunks = 6, parts = 4, part = chunk / parts;
+      std::vector<uint8_t> pattern(chunk * chunks);
+      for (size_t i = 0; i < pattern.size(); ++i) pattern[i] = static_cast<uint8_t>((i * 7 + i / 4099) % 251);
+      void* src = mr.allocate(ucx_memory_type::ROCM, pattern.size());
+      void* dst = mr.allocate(ucx_memory_type::ROCM, pattern.size());
+      mr.memcpy(ucx_memory_type::ROCM, src, ucx_memory_type::HOST, pattern.data(), pattern.size());
+      std::vector<uint8_t> zeros(pattern.size(), 0);
+      mr.memcpy(ucx_memory_type::ROCM, dst, ucx_memory_type::HOST, zeros.data(), zeros.size());
+      int64_t shape = static_cast<int64_t>(part);
+      std::vector<axr_tensor_t> from(parts), to(parts);
+      for (size_t k = 0; k < parts; ++k) {
+        from[k] = Tensor1D(static_cast<uint8_t*>(src) + k * part, &shape, 10, 1, 8);
+        to[k] = Tensor1D(static_cast<uint8_t*>(dst) + k * part, &shape, 10, 1, 8);
+      }
+      {
+        bundle::BundlePlan send = bundle::BundlePlan::Create(from.data(), parts, 256);
+        const std::vector<uint8_t> header = send.header();
+        bundle::BundlePlan recv = bundle::BundlePlan::FromHeaderBind(header.data(), header.size(), to.data(), parts);
+        bundle::StreamedTransfer transfer(mr, send.payload_bytes(), /*lanes=*/2, /*streams=*/1);
+        for (size_t c = 0; c < chunks; ++c)
+          transfer.Submit(send, static_cast<int64_t>(c * chunk), recv, static_cast<int64_t>(c * chunk));
+        transfer.Finish();
+      }
+      std::vector<uint8_t> got(pattern.size());
+      mr.memcpy(ucx_memory_type::HOST, got.data(), ucx_memory_type::ROCM, dst, got.size());
+      EXPECT(got == pattern);
+
+      // pack of chunk 1 and unpack of chunk 0's payload in ONE launch
+      mr.memcpy(ucx_memory_type::ROCM, dst, ucx_memory_type::HOST, zeros.data(), zeros.size());
+      bundle::BundlePlan send = bundle::BundlePlan::Create(from.data(), parts, 256);
+      const std::vector<uint8_t> header = send.header();
+      bundle::BundlePlan recv = bundle::BundlePlan::FromHeaderBind(header.data(), header.size(), to.data(), parts);
+      const size_t bytes = send.payload_bytes();
+      void* pay0 = mr.allocate(ucx_memory_type::ROCM, bytes);
+      void* pay1 = mr.allocate(ucx_memory_type::ROCM, bytes);
+      send.pack(pay0, bytes, nullptr);
+      EXPECT(axr_device_synchronize() == AXR_OK);
+      bundle::SubmitBundles({bundle::PackJob(send, pay1, bytes, static_cast<int64_t>(chunk)),
+                             bundle::UnpackJob(recv, pay0, bytes, 0)}, nullptr);
+      bundle::SubmitBundles({bundle::UnpackJob(recv, pay1, bytes, static_cast<int64_t>(chunk))}, nullptr);
+      EXPECT(axr_device_synchronize() == AXR_OK);
+      mr.memcpy(ucx_memory_type::HOST, got.data(), ucx_memory_type::ROCM, dst, 2 * chunk);
+      EXPECT(std::equal(got.begin(), got.begin() + 2 * chunk, pattern.begin()));
+      send.reset();
+      recv.reset();
+      mr.deallocate(ucx_memory_type::ROCM, pay0, bytes);
+      mr.deallocate(ucx_memory_type::ROCM, pay1, bytes);
+      mr.deallocate(ucx_memory_type::ROCM, src, pattern.size());
+      mr.deallocate(ucx_memory_type::ROCM, dst, pattern.size());
       EXPECT(mr.stats().live_blocks == 0);
     }
 
