@@ -1326,3 +1326,57 @@ def test_rows_reference_kernel(pkg, gpu, nontemporal):
         assert np.array_equal(twin.cpu().numpy(), expect), (run, pitch, rows)
     with pytest.raises(Exception):
         check(lib.axr_rows_reference(strided.data_ptr(), 8, packed.data_ptr(), 16, 1, 0, 0, None))
+
+
+@pytest.mark.parametrize("nontemporal", [-1, 3, 0])
+def test_short_rows_of_every_length(pkg, orc, gpu, nontemporal):
+    """Element mode over its whole range of run lengths: every length from 16 to 160 bytes and
+    a few up to the crossover with run tiles, enough rows for several work units (so that units
+    begin inside a run whenever the lane slots per run do not divide 512), with one and with two
+    strided dimensions, bases and pitches on and off the 16-byte grid, and every cache-hint
+    setting.  Gather against numpy slicing (the oracle for a sample), scatter into poisoned twins."""
+    import torch
+    rng = np.random.default_rng(31 + nontemporal)
+    lengths = list(range(16, 161)) + [250, 500, 1001, 1279]
+    pkg.tune(nontemporal=nontemporal)
+    try:
+        for batch in range(0, len(lengths), 25):
+            cases = []
+            for run in lengths[batch:batch + 25]:
+                pitch = run + int(rng.choice([0, 1, 7, 16, 100, 256 - run % 256]))
+                rows = int(rng.integers(600, 1400))
+                lead = int(rng.choice([0, 1, 3, 16]))
+                if rng.random() < 0.4:                       # two strided dimensions: [planes, rows, run]
+                    planes = int(rng.integers(2, 5))
+                    host = rng.integers(0, 256, size=lead + planes * (rows + 3) * pitch, dtype=np.uint8)
+                    dev = torch.from_numpy(host).to(gpu)
+                    view = dev[lead:].reshape(planes, rows + 3, pitch)[:, 1:rows + 1, :run]
+                    want = host[lead:].reshape(planes, rows + 3, pitch)[:, 1:rows + 1, :run]
+                else:
+                    host = rng.integers(0, 256, size=lead + rows * pitch, dtype=np.uint8)
+                    dev = torch.from_numpy(host).to(gpu)
+                    view = dev[lead:].reshape(rows, pitch)[:, :run]
+                    want = host[lead:].reshape(rows, pitch)[:, :run]
+                cases.append((host, dev, view, np.ascontiguousarray(want).reshape(-1)))
+            views = [c[2] for c in cases]
+            chunks = [c[3] for c in cases]
+            host0, _, v0, c0 = cases[0]
+            assert np.array_equal(c0, orc.gather_strided(host0, v0.storage_offset(), tuple(v0.shape),
+                                                         tuple(v0.stride()), 1))
+            for align in (1, 256):
+                got, plan, buf = run_pack(pkg, views, align, gpu)
+                modes = [s["mode"] for s in plan.segments()]      # pitch == run: one contiguous run
+                assert set(modes) <= {0, 1, 2} and modes.count(2) >= len(modes) // 2, modes
+                assert np.array_equal(got, orc.pack(chunks, align)), (batch, align)
+                twins = [device_bytes(c[1].numel(), gpu, fill=0x5C) for c in cases]
+                tviews = [t.as_strided(c[2].shape, c[2].stride(), c[2].storage_offset())
+                          for t, c in zip(twins, cases)]
+                pkg.BundlePlan.from_header(plan.header).bind(tviews).unpack(buf.data_ptr(), plan.payload_bytes)
+                torch.cuda.synchronize()
+                for twin, (host, _, view, chunk) in zip(twins, cases):
+                    expect = np.full(host.size, 0x5C, np.uint8)
+                    orc.scatter_strided(chunk, expect, view.storage_offset(), tuple(view.shape),
+                                        tuple(view.stride()), 1)
+                    assert np.array_equal(twin.cpu().numpy(), expect), (batch, align, tuple(view.shape))
+    finally:
+        pkg.tune(nontemporal=-1)
