@@ -139,23 +139,27 @@ def run_sets(h: Harness, sets, steps, warmup):
     return ms
 
 
-def run_sets_one_launch(h: Harness, sets, steps, warmup):
-    """Step i = axr_submit({pack of set i+1, unpack of set i}): one kernel launch."""
+def run_sets_one_launch(h: Harness, sets, steps, warmup, width=1):
+    """Step i = axr_submit({packs of the next `width` sets, unpacks of the `width` sets packed
+    by the step before}): one kernel launch that moves `width` bundles each way."""
     lib, stream, capi = h.lib, h.stream, h.capi
     n = len(sets)
-    if n < 2:
-        raise ValueError("the pipelined steps need at least two bundle copies")
+    if n < 2 * width or n % width:
+        raise ValueError("the pipelined steps need two groups of bundle copies")
+    groups = n // width
     jobs = []
-    for i in range(n):
-        a, b = sets[(i + 1) % n], sets[i]
-        arr = (capi.Job * 2)()
-        arr[0] = capi.Job(a.pp, 0, a.ptr, a.nbytes, 0)
-        arr[1] = capi.Job(b.up, 1, b.ptr, b.nbytes, 0)
+    for g in range(groups):
+        arr = (capi.Job * (2 * width))()
+        for k in range(width):
+            a, b = sets[((g + 1) % groups) * width + k], sets[g * width + k]
+            arr[k] = capi.Job(a.pp, 0, a.ptr, a.nbytes, 0)
+            arr[width + k] = capi.Job(b.up, 1, b.ptr, b.nbytes, 0)
         jobs.append(arr)
-    capi.check(lib.axr_pack(sets[0].pp, sets[0].ptr, sets[0].nbytes, stream))   # fills the pipeline
+    for k in range(width):      # fills the pipeline
+        capi.check(lib.axr_pack(sets[k].pp, sets[k].ptr, sets[k].nbytes, stream))
 
     def step(i):
-        rc = lib.axr_submit(jobs[i % n], 2, stream)
+        rc = lib.axr_submit(jobs[i % groups], 2 * width, stream)
         if rc:
             capi.check(rc)
 
@@ -955,6 +959,12 @@ def main():
         ms2 = run_sets_two_streams(h, sets, args.steps, args.warmup)
         extras["c2_two_streams_GBps"] = round(rate(P, ms2, args.steps), 1)
         extras["c2_graph_replay_GBps"] = graph_replay(h, sets, P)
+        if len(sets) >= 4 and len(sets) % 2 == 0:
+            # not `value`: two bundles each way per launch (four jobs), the fixed cost of a launch paid once
+            clear_sets(h, sets)
+            ms4 = run_sets_one_launch(h, sets, max(1, args.steps // 2), args.warmup, width=2)
+            check_sets(h, sets, "the four-job steps")
+            extras["c2_two_bundles_per_launch_GBps"] = round(rate(P, ms4, 2 * max(1, args.steps // 2)), 1)
         # the reference's own layout (tight concatenation) and a payload that bypasses the
         # last-level cache on both sides
         extras["c2_tight"] = c2_variant(align=1)
