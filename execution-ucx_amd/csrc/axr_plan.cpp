@@ -288,6 +288,23 @@ void plan_delete(axr_plan* p) {
   delete p;   // (under the lock: rare, and the plan is empty)
 }
 
+// A plan under construction: given back to the shells unless it is released to the caller,
+// also when an allocation throws on the way.
+struct PlanInProgress {
+  axr_plan* p;
+  explicit PlanInProgress(axr_plan* plan) : p(plan) {}
+  PlanInProgress(const PlanInProgress&) = delete;
+  PlanInProgress& operator=(const PlanInProgress&) = delete;
+  ~PlanInProgress() {
+    if (p) plan_delete(p);
+  }
+  axr_plan* release() {
+    axr_plan* out = p;
+    p = nullptr;
+    return out;
+  }
+};
+
 // One tensor's record of the header, as it lies on the wire (little-endian targets only).
 #pragma pack(push, 1)
 struct WireTensor {
@@ -1259,7 +1276,8 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   if (flags != 0) return fail(AXR_ERR_INVALID, "axr_plan_create: flags are reserved and must be 0");
   int rc = check_align(align);
   if (rc) return rc;
-  axr_plan* p = plan_new();
+  PlanInProgress guard(plan_new());
+  axr_plan* p = guard.p;
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_create: out of host memory");
   p->align = align;
   p->tensors.resize(n);
@@ -1275,7 +1293,6 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
     TensorRec& t = p->tensors[i];
     rc = store_tensor(p->dims64, tensors[i], &t);
     if (rc) {
-      plan_delete(p);
       return rc;
     }
     {
@@ -1288,7 +1305,6 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
       }
     }
     if (__builtin_add_overflow(off, mask, &off) || (off &= ~mask, __builtin_add_overflow(off, t.nbytes, &end))) {
-      plan_delete(p);
       return fail(AXR_ERR_INVALID, "axr_plan_create: bundle size overflows 64 bits");
     }
     t.offset = off;
@@ -1319,7 +1335,7 @@ static int plan_create_body(const axr_tensor_t* tensors, size_t n, uint32_t alig
   p->data_bytes = data;
   encode_preamble(p);
   p->bound = true;
-  *plan = p;
+  *plan = guard.release();
   return AXR_OK;
 }
 int axr_plan_create(const axr_tensor_t* tensors,
@@ -1439,7 +1455,8 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
     if (nbound != n) return fail(AXR_ERR_MISMATCH, "axr_plan_from_header_bind: tensor count differs from the header");
     if (n && !bound) return fail(AXR_ERR_INVALID, "axr_plan_from_header_bind: null tensor array");
   }
-  axr_plan* p = plan_new();
+  PlanInProgress guard(plan_new());
+  axr_plan* p = guard.p;
   if (!p) return fail(AXR_ERR_NOMEM, "axr_plan_from_header: out of host memory");
   p->align = align;
   p->tensors.resize(n);
@@ -1448,12 +1465,10 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
   uint64_t expect = 0, end = 0, data = 0;
   const uint64_t mask = static_cast<uint64_t>(align) - 1;
   if ((length - kFixedHeader - static_cast<size_t>(n) * kTensorHeader) / 8 > 0xffffffffull) {
-    plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header too long");
   }
   for (uint32_t i = 0; i < n; ++i) {
     if (length - at < kTensorHeader) {
-      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header truncated");
     }
     TensorRec& t = p->tensors[i];
@@ -1469,7 +1484,6 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
     at += kTensorHeader;
     if (t.ndim < 0 || t.ndim > kMaxNdim ||
         static_cast<size_t>(t.ndim) * 8 > length - at || byte_offset != 0) {
-      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header has a bad tensor record");
     }
     uint64_t rule = 0;
@@ -1497,18 +1511,15 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
     }
     at += static_cast<size_t>(t.ndim) * 8;
     if (sized != AXR_OK || rule != nb) {
-      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header tensor size does not follow from its shape");
     }
     if (binding) {
       const uint32_t sent_item = (static_cast<uint32_t>(t.bits) + 7) / 8;
       int rc = store_tensor(p->dims64, bound[i], &t);   // size rule, null checks; replaces the record
       if (rc) {
-        plan_delete(p);
         return rc;
       }
       if (t.nbytes != nb || (nb != 0 && (static_cast<uint32_t>(t.bits) + 7) / 8 != sent_item)) {
-        plan_delete(p);
         return fail(AXR_ERR_MISMATCH, "axr_plan_from_header_bind: tensor " + std::to_string(i) +
                                           " does not match the header's size or element width");
       }
@@ -1517,7 +1528,6 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
     uint64_t stop = 0;
     if (__builtin_add_overflow(expect, mask, &expect) || (expect &= ~mask, expect != off) ||
         __builtin_add_overflow(off, nb, &stop)) {
-      plan_delete(p);
       return fail(AXR_ERR_HEADER, "bundle header offsets do not follow the layout rule");
     }
     expect = end = stop;
@@ -1526,11 +1536,9 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
     t.offset = off;
   }
   if (at != length) {
-    plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header has trailing bytes");
   }
   if (end != payload) {
-    plan_delete(p);
     return fail(AXR_ERR_HEADER, "bundle header offsets do not follow the layout rule");
   }
   p->payload_bytes = end;
@@ -1538,7 +1546,7 @@ static int plan_from_header_body(const void* header, size_t length, const axr_te
   p->header.assign(h, h + length);
   p->bound = binding;
   p->receiver = true;
-  *plan = p;
+  *plan = guard.release();
   return AXR_OK;
 }
 int axr_plan_from_header(const void* header, size_t length, axr_plan_t** plan) {
