@@ -817,6 +817,54 @@ def ceilings(h):
     return out
 
 
+def small_bundles_batched(h, bundles=16, tensors=4, each=16 * 1024, steps=200):
+    """Sixteen small bundles (4 tensors of 16 KiB: the size of an RPC argument list) packed and
+    unpacked with kept plans: one axr_pack / axr_unpack launch per bundle against ONE
+    axr_submit launch for all sixteen packs and one for all unpacks.  us per bundle round trip."""
+    torch, lib, capi = h.torch, h.lib, h.capi
+    src = [[torch.randint(0, 255, (each,), dtype=torch.uint8, device="cuda") for _ in range(tensors)]
+           for _ in range(bundles)]
+    dst = [[torch.zeros_like(t) for t in b] for b in src]
+    plans = [h.pkg.BundlePlan.create(b, align=256) for b in src]
+    rplans = [h.pkg.BundlePlan.from_header(p.header).bind(d) for p, d in zip(plans, dst)]
+    nbytes = plans[0].payload_bytes
+    payloads = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(bundles)]
+    for p in plans + rplans:
+        p.prepare(h.stream)
+    packs = (capi.Job * bundles)(*[capi.Job(p._h, 0, b.data_ptr(), nbytes, 0) for p, b in zip(plans, payloads)])
+    unpacks = (capi.Job * bundles)(*[capi.Job(r._h, 1, b.data_ptr(), nbytes, 0) for r, b in zip(rplans, payloads)])
+    calls = [(p._h, r._h, b.data_ptr()) for p, r, b in zip(plans, rplans, payloads)]
+
+    def separate(i):
+        rc = 0
+        for pp, up, ptr in calls:
+            rc |= lib.axr_pack(pp, ptr, nbytes, h.stream)
+        for pp, up, ptr in calls:
+            rc |= lib.axr_unpack(up, ptr, nbytes, h.stream)
+        if rc:
+            capi.check(rc)
+
+    def batched(i):
+        rc = lib.axr_submit(packs, bundles, h.stream) | lib.axr_submit(unpacks, bundles, h.stream)
+        if rc:
+            capi.check(rc)
+
+    ms_sep = h.time_steps(separate, steps, 5)
+    for d in dst:
+        for t in d:
+            t.zero_()
+    h.sync()
+    ms_bat = h.time_steps(batched, steps, 5)
+    h.sync()
+    if not all(bool(torch.equal(a, b)) for s_, d_ in zip(src, dst) for a, b in zip(s_, d_)):
+        raise SystemExit("bench.py: batched small bundles did not reproduce the tensors")
+    for p in plans + rplans:
+        p.close()
+    return {"bundles": bundles, "tensors_per_bundle": tensors, "bytes_per_tensor": each,
+            "one_launch_per_bundle_us": round(ms_sep * 1e3 / (steps * bundles), 2),
+            "sixteen_bundles_per_launch_us": round(ms_bat * 1e3 / (steps * bundles), 2)}
+
+
 def load_traffic(kernel_key):
     path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
     try:
@@ -1011,6 +1059,7 @@ def main():
             torch.cuda.empty_cache()
         extras["strided_views"] = strided
         extras["fresh_small_bundle"] = fresh_small_round_trip(h)
+        extras["small_bundles_batched"] = small_bundles_batched(h)
         extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["loopback_iov_vs_bundle"] = iov_against_bundle(h, spec)
         extras["python_plan_us_per_1k_tensors"] = python_boundary(h, spec)

@@ -115,7 +115,7 @@ struct KernelArgs {
 };
 
 // One launch serving several bundles: job k owns the workgroups [wg_begin[k], wg_begin[k+1]).
-constexpr uint32_t kMaxJobs = 4;
+constexpr uint32_t kMaxJobs = 16;   // 1 KiB of kernel arguments
 struct JobDesc {              // 64 bytes
   uint64_t segs, dims, wave_seg, payload;   // device addresses
   int64_t tensor_delta;

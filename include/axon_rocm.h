@@ -320,7 +320,7 @@ AXR_API int axr_plan_prepare(axr_plan_t* plan, void* stream);
  * ProcessRndvBuffer_, axon/src/axon_worker.cpp:1424-1490 and :1098-1219, run by
  * independent coroutines in the reference) submits the gathers and scatters
  * together: neighbouring jobs of one launch geometry share ONE kernel launch
- * (up to four per launch; a short kernel's fixed cost is paid once), the rest run
+ * (up to sixteen per launch; a short kernel's fixed cost is paid once), the rest run
  * one after the other, all on `stream`.  The jobs of one call must not depend on
  * each other (no job may read what another one writes) and no plan may appear
  * twice.  `tensor_delta` is added to every bound tensor address of that job: a

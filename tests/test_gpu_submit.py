@@ -366,3 +366,34 @@ def test_tables_built_on_the_device_match_the_oracle(pkg, orc, gpu, align):
         plan.close()
     finally:
         pkg.tune(device_tables=before.value)
+
+
+def test_many_small_bundles_in_one_call(pkg, orc, gpu):
+    """Forty small bundles (the size of an RPC argument list) gathered by one axr_submit and
+    scattered by another: sixteen jobs share a launch, so the call is three launches, and
+    every bundle equals the oracle's pack and comes back whole."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    rng = np.random.default_rng(77)
+    bundles = [random_tensors(rng, gpu, int(rng.integers(1, 9)), lo=64, hi=70000) for _ in range(40)]
+    torch.cuda.synchronize()
+    plans = [pkg.BundlePlan.create(t, align=256) for t in bundles]
+    bufs = [torch.full((p.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu) for p in plans]
+    outs = [zeros_like_views(t) for t in bundles]
+    rplans = [pkg.BundlePlan.from_header(p.header).bind(o) for p, o in zip(plans, outs)]
+    torch.cuda.synchronize()
+    try:
+        arr = job_array(capi, [(p, 0, b.data_ptr(), p.payload_bytes, 0) for p, b in zip(plans, bufs)])
+        capi.check(lib.axr_submit(arr, len(plans), None))
+        arr = job_array(capi, [(r, 1, b.data_ptr(), p.payload_bytes, 0) for r, p, b in zip(rplans, plans, bufs)])
+        capi.check(lib.axr_submit(arr, len(plans), None))
+        capi.check(lib.axr_device_synchronize())
+        for tensors, p, b, o in zip(bundles, plans, bufs, outs):
+            got = b.cpu().numpy()
+            assert np.array_equal(got[:p.payload_bytes], orc.pack([chunk_of(t) for t in tensors], 256))
+            assert (got[p.payload_bytes:] == POISON).all()
+            for x, y in zip(tensors, o):
+                assert np.array_equal(chunk_of(x), chunk_of(y))
+    finally:
+        for p in plans + rplans:
+            p.close()
