@@ -415,6 +415,20 @@ def end_to_end_us(h, spec, steps=20):
             "round_trip_us": times[len(times) // 2] * 1e6}
 
 
+def end_to_end_from_cpp():
+    """The same fresh-bundle round trip timed inside a C++ caller of the C ABI
+    (execution-ucx_amd/lib/fresh_bundle_bench, built by `make`): no ctypes calls in the timed
+    region.  It checks its own result and prints one JSON line."""
+    import subprocess
+    exe = os.path.join(ROOT, "execution-ucx_amd", "lib", "fresh_bundle_bench")
+    if not os.path.exists(exe):
+        return "not measured: lib/fresh_bundle_bench is not built"
+    out = subprocess.run([exe, "100"], capture_output=True, text=True, timeout=120)
+    if out.returncode != 0:
+        raise SystemExit("bench.py: fresh_bundle_bench failed: " + out.stderr.strip()[-400:])
+    return json.loads(out.stdout.strip().splitlines()[-1])
+
+
 def fresh_small_round_trip(h, tensors=4, each=64 * 1024, steps=200):
     """Wall time of plan -> pack -> sync -> plan-from-header -> bind -> unpack -> sync for a
     fresh bundle of a few tensors (the size of a typical RPC argument list), C ABI only."""
@@ -1018,6 +1032,7 @@ def main():
         extras["c2_tight"] = c2_variant(align=1)
         extras["c2_payload_streaming"] = c2_variant(payload_cache_bytes=0)
         extras.update({k: round(v, 2) for k, v in end_to_end_us(h, spec).items()})
+        extras["fresh_bundle_from_cpp"] = end_to_end_from_cpp()
         del sets
         torch.cuda.empty_cache()
         c3 = make_c3_sets(h, 2)
