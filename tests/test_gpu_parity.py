@@ -1380,3 +1380,44 @@ def test_short_rows_of_every_length(pkg, orc, gpu, nontemporal):
                     assert np.array_equal(twin.cpu().numpy(), expect), (batch, align, tuple(view.shape))
     finally:
         pkg.tune(nontemporal=-1)
+
+
+@pytest.mark.parametrize("dtype_name", ["uint8", "int16", "float32", "float64", "complex128"])
+def test_transposed_views_of_random_extents(pkg, orc, gpu, dtype_name):
+    """Transposed matrices whose extents fall anywhere around the block edge: shorter than a
+    block, one element past a whole number of blocks, one short of it (the last block of such
+    a dimension is moved back over its neighbour and stays on the vector path), with row
+    pitches and bases off every power-of-two grid.  Gather against the oracle, scatter into
+    poisoned twins."""
+    import torch
+    dt = getattr(torch, dtype_name)
+    item = torch.empty((), dtype=dt).element_size()
+    t = (128 if item <= 4 else 256) // item
+    rng = np.random.default_rng(500 + item)
+    extents = [1, 2, t - 1, t, t + 1, 2 * t - 1, 2 * t + 1, 3 * t - 5, int(rng.integers(1, 3 * t)),
+               int(rng.integers(1, 3 * t))]
+    cases = []
+    for _ in range(14):
+        rows, cols = int(rng.choice(extents)), int(rng.choice(extents))
+        pad_r, pad_c = int(rng.integers(0, 3)), int(rng.integers(0, 4))
+        parent = rand_bytes_tensor(rng, (rows + pad_r) * (cols + pad_c) * item, gpu).view(dt).reshape(rows + pad_r, cols + pad_c)
+        cases.append((parent, parent[pad_r:, pad_c:].t()))
+    b = rand_bytes_tensor(rng, 3 * (t + 3) * (2 * t + 1) * item, gpu).view(dt).reshape(3, t + 3, 2 * t + 1)
+    cases.append((b, b.transpose(1, 2)))                       # a batch of ragged transposes
+    views = [v for _, v in cases]
+    chunks = []
+    for parent, v in cases:
+        host_parent = parent.reshape(-1).view(torch.uint8).cpu().numpy()
+        chunks.append(orc.gather_strided(host_parent, (v.data_ptr() - parent.data_ptr()),
+                                         tuple(v.shape), tuple(v.stride()), item))
+    for align in (256, 1):
+        got, plan, buf = run_pack(pkg, views, align, gpu)
+        assert np.array_equal(got, orc.pack(chunks, align)), align
+        twins = [device_bytes(p.numel() * item, gpu, fill=0x3B).view(dt).reshape(p.shape) for p, _ in cases]
+        tviews = [tw.as_strided(v.shape, v.stride(), v.storage_offset()) for tw, (_, v) in zip(twins, cases)]
+        pkg.BundlePlan.from_header(plan.header).bind(tviews).unpack(buf.data_ptr(), plan.payload_bytes)
+        torch.cuda.synchronize()
+        for tw, (parent, v), c in zip(twins, cases, chunks):
+            expect = np.full(parent.numel() * item, 0x3B, np.uint8)
+            orc.scatter_strided(c, expect, v.data_ptr() - parent.data_ptr(), tuple(v.shape), tuple(v.stride()), item)
+            assert np.array_equal(tw.reshape(-1).view(torch.uint8).cpu().numpy(), expect), (align, tuple(v.shape))
