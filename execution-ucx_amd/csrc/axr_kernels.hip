@@ -282,6 +282,9 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
   }
   const uint32_t gpr_magic = 0xffffffffu / gpr + 1u;
   const int64_t stride_last = dm->stride[kMaxOuterDims - 1];
+  const int64_t stride_prev = dm->stride[kMaxOuterDims - 2];
+  const uint32_t extent_last = dm->shape[kMaxOuterDims - 1];
+  const uint32_t magic_last = 0xffffffffu / extent_last + 1u;
   gbytes tbase = as_global(seg_ptr) + base;
   gbytes pbase = ragged ? pay + static_cast<uint64_t>(run0) * run32 : pay + b0;
   // tensor-side byte offset (relative to the tile's first run) of granule e of the
@@ -303,6 +306,17 @@ __device__ __forceinline__ void element_tile(uint64_t seg_ptr, uint64_t run_byte
     int64_t toff = static_cast<int64_t>(in_run);
     if (nd == 1) {   // one strided dimension (rows of a matrix): the run index is the only coordinate
       return toff + static_cast<int64_t>(carry) * stride_last;
+    }
+    if (nd == 2) {
+      // two strided dimensions (every k-th element of the rows of a matrix, a slice of a
+      // 3-d tensor): one quotient, no carry beyond the outer one, nothing to vote on.
+      // v < extent + 2^14, so the multiply-high quotient is exact for extents below 2^15.
+      uint32_t v = idx0[kMaxOuterDims - 1] + carry;
+      uint32_t c = extent_last < 32768u ? __umulhi(v, magic_last) : v / extent_last;
+      c = extent_last == 1 ? v : c;
+      v -= c * extent_last;
+      return toff + static_cast<int64_t>(static_cast<int32_t>(v - idx0[kMaxOuterDims - 1])) * stride_last +
+             static_cast<int64_t>(c) * stride_prev;
     }
 #pragma unroll
     for (int d = static_cast<int>(kMaxOuterDims) - 1; d >= 0; --d) {
