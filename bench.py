@@ -1074,6 +1074,12 @@ def main():
             torch.cuda.empty_cache()
         extras["strided_views"] = strided
         extras["fresh_small_bundle"] = fresh_small_round_trip(h)
+        # the same with axr_stream_synchronize polling a word of pinned memory first (opt-in)
+        pkg.tune(spin_wait_us=200)
+        try:
+            extras["fresh_small_bundle"]["round_trip_us_with_polled_wait"] = fresh_small_round_trip(h)["round_trip_us"]
+        finally:
+            pkg.tune(spin_wait_us=0)
         extras["small_bundles_batched"] = small_bundles_batched(h)
         extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["loopback_iov_vs_bundle"] = iov_against_bundle(h, spec)

@@ -193,6 +193,10 @@ struct Tunables {
   // tables in one pass over the tensors into pinned memory plus a kernel that brings them to
   // the device and writes the tile-block index (0: the general host path always).
   std::atomic<int64_t> device_tables{512};
+  // axr_stream_synchronize may first poll, for up to this many microseconds, a word of pinned
+  // memory that a one-wave kernel enqueued behind the stream's work writes, before it falls
+  // back to the runtime's wait (0, the default: the runtime's wait only).  See the header.
+  std::atomic<int64_t> spin_wait_us{0};
   std::atomic<int64_t> host_threads{4};       // threads (the caller included) for host-side staging copies
   std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
@@ -253,6 +257,8 @@ int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchC
 // hints; cfg.workgroups is the whole grid, cfg.lds_per_wave the largest need of any job).
 int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stream);
 int launch_fill(void* dst, int value, size_t bytes, void* stream);
+// Enqueues a one-wave kernel that stores `value` into *flag (pinned host memory).
+int launch_notify(uint32_t* flag, uint32_t value, void* stream);
 // staged: n + 1 segment records in device-accessible memory (pinned host memory will do);
 // segs and wave_seg are device memory.  Copies the records and writes the tile-block index.
 int launch_expand_tables(const Seg* staged, uint32_t n, Seg* segs, uint32_t* wave_seg, uint32_t seg_shift,

@@ -1357,6 +1357,19 @@ int launch_stream_copy(void* dst, const void* src, size_t bytes, bool nontempora
   return check_hip(hipGetLastError(), "stream copy launch");
 }
 
+// One lane stores `value` into a word of pinned host memory: a host thread that polls the
+// word learns that the stream has reached this point without waiting for the runtime's
+// completion signal.  A vector store at system scope; nothing is released with it (the
+// kernels ahead of this one in the stream have ended by then).
+__global__ void notify_kernel(uint32_t* flag, uint32_t value) {
+  if (threadIdx.x == 0) __hip_atomic_store(flag, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+int launch_notify(uint32_t* flag, uint32_t value, void* stream) {
+  hipLaunchKernelGGL(notify_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), flag, value);
+  return check_hip(hipGetLastError(), "notify kernel launch");
+}
+
 int launch_fill(void* dst, int value, size_t bytes, void* stream) {
   if (bytes == 0) return AXR_OK;
   hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(bytes / 16 + 1, 1u << 16)), dim3(256), 0,

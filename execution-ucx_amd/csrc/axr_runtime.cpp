@@ -3,6 +3,8 @@
 // headers; host code above the C ABI never does.
 #include <hip/hip_runtime_api.h>
 
+#include <chrono>
+
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -467,6 +469,9 @@ static int tune_set_body(const char* key, int64_t value) {
     t.xcd_remap = value < 0 ? -1 : (value ? 1 : 0);
   } else if (k == "ragged_runs") {
     t.ragged_runs = value ? 1 : 0;
+  } else if (k == "spin_wait_us") {
+    if (value < 0 || value > 1000000) return fail(AXR_ERR_INVALID, "spin_wait_us must be in [0, 1000000]");
+    t.spin_wait_us = value;
   } else if (k == "host_threads") {
     if (value < 1 || value > 64) return fail(AXR_ERR_INVALID, "host_threads must be in [1, 64]");
     t.host_threads = value;
@@ -509,6 +514,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "ragged_runs") *value = t.ragged_runs;
   else if (k == "inline_tables") *value = t.inline_tables;
   else if (k == "host_threads") *value = t.host_threads;
+  else if (k == "spin_wait_us") *value = t.spin_wait_us;
   else if (k == "head_align") *value = t.head_align;
   else if (k == "loopback_copy_kernel") *value = t.loopback_copy_kernel;
   else if (k == "device_tables") *value = t.device_tables;
@@ -627,10 +633,77 @@ int axr_stream_destroy(void* stream) {
 }
 
 
+namespace {
+// Words of pinned host memory, per device, that notify kernels write and waiting threads
+// poll ("spin_wait_us").  Each wait takes the next word in turn and a value of its own;
+// should two waits ever share a word (more than kNotifySlots under way at once), the loser
+// merely runs out of time and falls back to the runtime's wait.
+constexpr int kNotifyDevices = 64;
+constexpr uint32_t kNotifySlots = 256;
+constexpr uint32_t kNotifyStride = 16;   // words: one 64-byte line per slot
+std::atomic<uint32_t*> g_notify_words[kNotifyDevices];
+std::atomic<uint32_t> g_notify_ticket{0};
+
+uint32_t* notify_words(int device) {
+  if (device < 0 || device >= kNotifyDevices) return nullptr;
+  uint32_t* words = g_notify_words[device].load(std::memory_order_acquire);
+  if (words) return words;
+  void* fresh = nullptr;
+  if (hipHostMalloc(&fresh, kNotifySlots * kNotifyStride * sizeof(uint32_t), hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::memset(fresh, 0, kNotifySlots * kNotifyStride * sizeof(uint32_t));
+  uint32_t* expected = nullptr;
+  if (!g_notify_words[device].compare_exchange_strong(expected, static_cast<uint32_t*>(fresh),
+                                                      std::memory_order_acq_rel)) {
+    (void)hipHostFree(fresh);   // another thread was first
+    return expected;
+  }
+  return static_cast<uint32_t*>(fresh);   // kept until the process ends
+}
+
+// True when the stream was seen to reach its end by polling; false: the caller waits through
+// the runtime (capturing stream, no pinned memory, launch refused, time budget spent).
+bool spin_until_stream_end(hipStream_t stream, int64_t budget_us) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (status != hipStreamCaptureStatusNone) return false;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  uint32_t* words = notify_words(device);
+  if (!words) return false;
+  const uint32_t ticket = g_notify_ticket.fetch_add(1, std::memory_order_relaxed) + 1;
+  volatile uint32_t* word = words + (ticket % kNotifySlots) * kNotifyStride;
+  const uint32_t value = ticket | 0x80000000u;   // never the zero the words start with
+  if (launch_notify(const_cast<uint32_t*>(word), value, stream) != AXR_OK) return false;
+  const auto deadline = std::chrono::steady_clock::now() + std::chrono::microseconds(budget_us);
+  for (;;) {
+    for (int i = 0; i < 64; ++i) {
+      if (*word == value) {
+        std::atomic_thread_fence(std::memory_order_acquire);
+        return true;
+      }
+      __builtin_ia32_pause();
+    }
+    if (std::chrono::steady_clock::now() >= deadline) return false;
+  }
+}
+}  // namespace
+
 static int stream_synchronize_body(void* stream) {
   const uint64_t reached = stream_launch_mark();
-  int rc = check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "hipStreamSynchronize");
-  if (rc) return rc;
+  const int64_t budget = tunables().spin_wait_us;
+  if (!(budget > 0 && spin_until_stream_end(static_cast<hipStream_t>(stream), budget))) {
+    int rc = check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "hipStreamSynchronize");
+    if (rc) return rc;
+  }
   stream_note_drained(stream, reached);   // plans released next need not wait for this stream again
   return AXR_OK;
 }

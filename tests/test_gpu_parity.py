@@ -1421,3 +1421,37 @@ def test_transposed_views_of_random_extents(pkg, orc, gpu, dtype_name):
             expect = np.full(parent.numel() * item, 0x3B, np.uint8)
             orc.scatter_strided(c, expect, v.data_ptr() - parent.data_ptr(), tuple(v.shape), tuple(v.stride()), item)
             assert np.array_equal(tw.reshape(-1).view(torch.uint8).cpu().numpy(), expect), (align, tuple(v.shape))
+
+
+def test_polled_stream_wait(pkg, orc, gpu):
+    """axr_stream_synchronize with "spin_wait_us": the wait that polls a word of pinned memory
+    returns only when the stream's work is done (a pack's payload is complete right after it),
+    a budget too short for the kernel falls back to the runtime's wait with the same result,
+    and plans freed afterwards do not trip over the notify kernels."""
+    import torch
+    lib, check = pkg._capi.load(), pkg._capi.check
+    rng = np.random.default_rng(12)
+    stream = C.c_void_p()
+    check(lib.axr_stream_create(C.byref(stream)))
+    big = [rand_bytes_tensor(rng, 64 << 20, gpu) for _ in range(4)]        # a launch of ~100 us
+    small = [rand_bytes_tensor(rng, int(n), gpu) for n in rng.integers(1, 5000, size=9)]
+    want_big = orc.pack([t.cpu().numpy() for t in big], 256)
+    want_small = orc.pack([t.cpu().numpy() for t in small], 256)
+    torch.cuda.synchronize()
+    try:
+        for budget in (200, 1, 0):
+            pkg.tune(spin_wait_us=budget)
+            for tensors, want in ((big, want_big), (small, want_small)):
+                for _ in range(3):
+                    plan = pkg.BundlePlan.create(tensors, align=256)
+                    buf = device_bytes(plan.payload_bytes, gpu)
+                    torch.cuda.synchronize()
+                    plan.pack(buf.data_ptr(), plan.payload_bytes, stream.value)
+                    check(lib.axr_stream_synchronize(stream))
+                    host = torch.empty(plan.payload_bytes, dtype=torch.uint8).pin_memory()
+                    host.copy_(buf)                            # a blocking copy on another stream: no extra wait for ours
+                    plan.close()
+                    assert np.array_equal(host.numpy(), want), (budget, len(tensors))
+    finally:
+        pkg.tune(spin_wait_us=0)
+        check(lib.axr_stream_destroy(stream))

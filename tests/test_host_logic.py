@@ -68,7 +68,8 @@ def test_tunables(pkg):
     lib = pkg._capi.load()
     v = C.c_int64()
     for key, good, bad in ((b"tile_rows", 4, 3), (b"threads", 512, 100), (b"max_waves", 99, 0),
-                           (b"gather_run_bytes", 64, 0), (b"max_tiles", 1000, 0)):
+                           (b"gather_run_bytes", 64, 0), (b"max_tiles", 1000, 0),
+                           (b"spin_wait_us", 150, -1)):
         before = C.c_int64()
         assert lib.axr_tune_get(key, C.byref(before)) == 0
         assert lib.axr_tune_set(key, good) == 0
