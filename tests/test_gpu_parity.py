@@ -1455,3 +1455,32 @@ def test_polled_stream_wait(pkg, orc, gpu):
     finally:
         pkg.tune(spin_wait_us=0)
         check(lib.axr_stream_destroy(stream))
+
+
+def test_die_contiguous_tile_ranges(pkg, orc, gpu):
+    """"xcd_remap": every die walks one contiguous share of the tiles.  Forced on for a mixed
+    bundle, and chosen automatically for a bundle of transposed views whose rows straddle
+    128-byte lines (there the grid is rounded up to a multiple of the eight dies); both
+    against the oracle, pack and unpack."""
+    import torch
+    rng = np.random.default_rng(808)
+    mixed = [rand_bytes_tensor(rng, int(n), gpu) for n in rng.integers(1, 40000, size=700)]
+    mixed.append(rand_bytes_tensor(rng, 300 * 1000, gpu).reshape(300, 1000)[:, :333])      # element mode
+    odd = [rand_bytes_tensor(rng, 700 * 650 * 2, gpu).view(torch.int16).reshape(700, 650).t() for _ in range(2)]
+    for views, tune, expect_rounded in ((mixed, 1, True), (odd, -1, True), (odd, 0, False)):
+        pkg.tune(xcd_remap=tune)
+        try:
+            chunks = [tbytes(v) for v in views]
+            got, plan, buf = run_pack(pkg, views, 256, gpu)
+            info = plan.launch_info()
+            assert info["workgroups"] >= 32
+            assert (info["workgroups"] % 8 == 0) == expect_rounded or not expect_rounded, info
+            assert np.array_equal(got, orc.pack(chunks, 256)), tune
+            twins = [torch.zeros_like(v._base if v._base is not None else v) for v in views]
+            tviews = [tw.as_strided(v.shape, v.stride(), v.storage_offset()) for tw, v in zip(twins, views)]
+            pkg.BundlePlan.from_header(plan.header).bind(tviews).unpack(buf.data_ptr(), plan.payload_bytes)
+            torch.cuda.synchronize()
+            for v, tv_ in zip(views, tviews):
+                assert np.array_equal(tbytes(v), tbytes(tv_)), tune
+        finally:
+            pkg.tune(xcd_remap=-1)
