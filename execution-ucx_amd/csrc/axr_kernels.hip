@@ -892,10 +892,11 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   const AXR_CONST JobTable* jt =
       (const AXR_CONST JobTable*)__builtin_amdgcn_kernarg_segment_ptr();
   const uint32_t wg = blockIdx.x;
+  // the job whose workgroup range holds this workgroup (the ranges ascend; a launch of two
+  // jobs reads one entry beyond its own)
   uint32_t j = 0;
-#pragma unroll
-  for (uint32_t k = 1; k < kMaxJobs; ++k)
-    if (k < jt->count && wg >= jt->job[k].wg_begin) j = k;
+  const uint32_t count = jt->count;
+  for (uint32_t k = 1; k < count && wg >= jt->job[k].wg_begin; ++k) j = k;
   const AXR_CONST JobDesc* d = &jt->job[j];
   KernelArgs a;
   a.ntiles = d->ntiles;
