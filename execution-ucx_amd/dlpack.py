@@ -192,7 +192,14 @@ class TensorArray:
     def from_objects(cls, objs: Sequence[Any]) -> "TensorArray":
         """Descriptors of DLPack producers (or ``TensorView``s)."""
         native = _native()
-        described = native.describe(objs, *_torch_exporter()) if native is not None else None
+        exporter = _torch_exporter()
+        described = None
+        if exporter:   # a bundle of plain torch tensors is read without one capsule per tensor
+            direct = _native_torch()
+            if direct is not None:
+                described = direct.describe(objs, exporter[2])
+        if described is None and native is not None:
+            described = native.describe(objs, *exporter)
         if described is None:   # no helper, or something that is not a DLPack producer
             return cls(extract_many(objs))
         descs, dims, owners = described
@@ -271,6 +278,35 @@ def _native():
                 _NATIVE = mod
             break
     return _NATIVE
+
+
+_NATIVE_TORCH: Any = False
+
+
+def _native_torch():
+    """The helper that reads torch tensors' fields through torch's own non-owning DLPack
+    converter, or None when it has not been built or does not load against this torch.
+    Only called once torch has been imported (its libraries are the module's dependencies)."""
+    global _NATIVE_TORCH
+    if _NATIVE_TORCH is False:
+        import glob
+        import importlib.machinery
+        import importlib.util
+        import os
+        _NATIVE_TORCH = None
+        here = os.path.dirname(os.path.abspath(__file__))
+        for path in glob.glob(os.path.join(here, "lib", "_axr_torch*.so")):
+            try:
+                loader = importlib.machinery.ExtensionFileLoader("_axr_torch", path)
+                spec = importlib.util.spec_from_loader("_axr_torch", loader)
+                mod = importlib.util.module_from_spec(spec)
+                loader.exec_module(mod)
+            except ImportError:   # built against another torch
+                break
+            if mod.TENSOR_BYTES == C.sizeof(_capi.Tensor):
+                _NATIVE_TORCH = mod
+            break
+    return _NATIVE_TORCH
 
 
 # ---------------------------------------------------------------- export

@@ -854,6 +854,24 @@ def test_torch_device_tensors_through_the_short_export_route(pkg, orc, gpu):
     plain = dlpack.extract_many(tensors)
     assert [(x.data, x.device_type, x.shape, x.strides, x.dtype) for x in short] == \
         [(x.data, x.device_type, x.shape, x.strides, x.dtype) for x in plain]
+    # the reader that makes no capsules took them (device and pinned host tensors alike), and
+    # declines GPU tensors when asked for another device than theirs
+    direct = dlpack._native_torch()
+    assert direct is not None, "build lib/_axr_torch*.so with `make -C execution-ucx_amd`"
+    with_pinned = tensors + [torch.arange(12, dtype=torch.float32).pin_memory().view(3, 4)[:, 1:]]
+    described = direct.describe(with_pinned, fast[2])
+    assert described is not None and described[2] == with_pinned
+    again = dlpack._native().describe(with_pinned, *fast)
+    count = len(with_pinned)
+    ta = (dlpack._capi.Tensor * count).from_buffer(described[0])
+    tb = (dlpack._capi.Tensor * count).from_buffer(again[0])
+    for i in range(count):
+        for f in ("data", "device_type", "device_id", "ndim", "dtype_code", "dtype_bits", "dtype_lanes",
+                  "byte_offset"):
+            assert getattr(ta[i], f) == getattr(tb[i], f), (i, f)
+    del ta, tb
+    assert bytes(described[1]) == bytes(again[1])
+    assert direct.describe(tensors, fast[2] + 1) is None and direct.describe(tensors, -1) is None
     want = orc.pack([tbytes(t) for t in tensors], 64)
     got, plan, _ = run_pack(pkg, tensors, 64, gpu)
     assert np.array_equal(got, want)

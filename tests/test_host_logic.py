@@ -635,6 +635,75 @@ def test_torch_tensors_skip_the_python_wrapper_but_keep_its_refusals(pkg):
     # hands out GPU memory through the short route (checked on the capsule in C)
 
 
+def test_torch_tensors_read_without_capsules_match_the_capsule_route(pkg):
+    """lib/_axr_torch reads plain torch tensors through torch's non-owning DLPack converter:
+    every descriptor field equals what a capsule from torch.utils.dlpack.to_dlpack carries, for
+    each dtype torch exports and for views with size-1, size-0, stepped and permuted dimensions;
+    anything Tensor.__dlpack__ would refuse, a subclass or a foreign producer makes it decline
+    (None), and the bundle then takes the capsule route with that route's verdict."""
+    import torch
+    from execution_ucx_amd import dlpack
+    direct = dlpack._native_torch()
+    native = dlpack._native()
+    assert direct is not None, "build lib/_axr_torch*.so with `make -C execution-ucx_amd`"
+    to_dlpack = torch.utils.dlpack.to_dlpack
+    tensors = []
+    for dt in (torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64, torch.float16,
+               torch.bfloat16, torch.float32, torch.float64, torch.bool, torch.complex64,
+               torch.complex128, torch.uint16, torch.uint32, torch.uint64):
+        base = torch.zeros(4 * 6 * 8, dtype=dt)
+        cube = base.view(4, 6, 8)
+        tensors += [base, cube, cube[:, ::2, 1:], cube.permute(2, 0, 1), cube[1], base.view(4, 1, 48),
+                    base.view(4, 1, 48)[:, :, ::3], base[:0], cube[:, :0], base[3:4].reshape(()),
+                    base.view(1, 192), base.view(192, 1).t()]
+    for dt in (torch.float8_e4m3fn, torch.float8_e5m2):   # exported or not, both routes agree
+        try:
+            to_dlpack(torch.zeros(4, dtype=dt))
+            tensors.append(torch.zeros(4, 6, dtype=dt)[:, ::2])
+        except (BufferError, RuntimeError, TypeError):
+            assert direct.describe([torch.zeros(4, dtype=dt)], -1) is None
+    a = direct.describe(tensors, -1)
+    b = native.describe(tensors, torch.Tensor, to_dlpack, -1)
+    assert a is not None and a[2] == tensors                       # the owners are the tensors
+    assert len(a[0]) == len(b[0]) and bytes(a[1]) == bytes(b[1])   # shapes and strides
+    ta = (dlpack._capi.Tensor * len(tensors)).from_buffer(a[0])
+    tb = (dlpack._capi.Tensor * len(tensors)).from_buffer(b[0])
+    fields = ("data", "device_type", "device_id", "ndim", "dtype_code", "dtype_bits", "dtype_lanes",
+              "byte_offset")
+    dims_a = C.addressof((C.c_char * len(a[1])).from_buffer(a[1])) if len(a[1]) else 0
+    dims_b = C.addressof((C.c_char * len(b[1])).from_buffer(b[1])) if len(b[1]) else 0
+    for i in range(len(tensors)):
+        assert [getattr(ta[i], f) for f in fields] == [getattr(tb[i], f) for f in fields], i
+        for name in ("shape", "strides"):   # the pointers name the same places of the two dims blocks
+            pa = C.cast(getattr(ta[i], name), C.c_void_p).value
+            pb = C.cast(getattr(tb[i], name), C.c_void_p).value
+            assert (pa is None) == (pb is None), (i, name)
+            if pa is not None:
+                assert pa - dims_a == pb - dims_b, (i, name)
+    del ta, tb
+    assert pkg.BundlePlan.create(tensors[:40], align=64).header == \
+        pkg.BundlePlan.create(dlpack.extract_many(tensors[:40]), align=64).header
+
+    class Wrapped(torch.Tensor):
+        pass
+    good = tensors[1]
+    for other in (good.as_subclass(Wrapped), torch.zeros(3, requires_grad=True),
+                  torch.zeros(3, dtype=torch.complex64).conj(), torch.zeros(3, 3).to_sparse(),
+                  torch.nn.Parameter(torch.zeros(3)), np.zeros(3), object(),
+                  torch.zeros(3, device="meta")):
+        assert direct.describe([good, other], -1) is None, type(other)
+    # a Parameter that requires no gradient is a Tensor as far as the export goes
+    frozen = torch.nn.Parameter(torch.arange(6.0).view(2, 3), requires_grad=False)
+    assert bytes(direct.describe([frozen], -1)[0])[:24] == \
+        bytes(native.describe([frozen], torch.Tensor, to_dlpack, -1)[0])[:24]   # up to the shape pointer
+    assert direct.describe([], -1) is not None and direct.describe((good,), -1) is not None
+    # the capsule route still has the last word on what was declined
+    with pytest.raises(BufferError, match="gradient"):
+        dlpack.TensorArray.from_objects([good, torch.zeros(3, requires_grad=True)])
+    mixed = dlpack.TensorArray.from_objects([good, np.zeros(3, np.float32)])
+    assert mixed.count == 2 and mixed.views[1].shape == (3,)
+
+
 # ------------------------------------------------------------------ bench.py contract (no GPU needed)
 
 def test_bench_refuses_more_than_one_gpu():
