@@ -164,18 +164,28 @@ static int transfer_submit_body(axr_transfer_t* t, axr_plan_t* send_plan, int64_
     am.mem_h = lane.send_mem_h;
     rc = axr_am_send(t->client, t->conn, &am, lane.stream, &lane.request);
     if (rc) return rc;
+    // From here on a failure must not leave the send parked or its message queued: the
+    // slot is reused by the chunk after next.
     axr_am_message_t msg;
     rc = axr_am_recv_header(t->server, &msg);
-    if (rc) return rc;
+    if (rc) {
+      (void)axr_am_request_cancel(t->client, lane.request);
+      return rc;
+    }
     // what arrived is what the receiver planned for
     if (!msg.is_rndv || msg.data_length != nbytes || msg.header.size != recv_header_bytes ||
         std::memcmp(msg.header.data, recv_header, recv_header_bytes) != 0) {
       (void)axr_am_message_release(t->server, msg.key);
+      (void)axr_am_request_cancel(t->client, lane.request);
       return fail(AXR_ERR_MISMATCH, "the received message does not match the receiver's plan");
     }
     rc = axr_am_recv_buffer_async(t->server, msg.key, AXR_MEM_ROCM, lane.recv_slot, t->slot_bytes,
                                   lane.stream);
-    if (rc) return rc;
+    if (rc) {
+      (void)axr_am_message_release(t->server, msg.key);
+      (void)axr_am_request_cancel(t->client, lane.request);
+      return rc;
+    }
     lane.in_flight = true;
   }
   job.plan = recv_plan;
