@@ -22,7 +22,7 @@
  * C exporter that Tensor.__dlpack__ ends in, minus a dozen Python-level checks
  * per tensor (about 0.15 us instead of 1.7 us).  Whatever fails one of the
  * conditions, or makes `fast_export` raise, goes through `__dlpack__()` and
- * gets that method's verdict.
+ * gets that method's answer.
  */
 #define PY_SSIZE_T_CLEAN
 #include <Python.h>

@@ -12,7 +12,7 @@
 //   owners  the tensors themselves (they own the memory the descriptors name)
 // None when any element is not exactly a torch.Tensor, requires grad, carries the conjugate or
 // negative bit, is not strided, lives on another GPU than `device_id`, or is refused by the
-// converter: the caller then takes the capsule route, which gives Tensor.__dlpack__'s verdict.
+// converter: the caller then takes the capsule route, which gives Tensor.__dlpack__'s answer.
 //
 // Built against the torch that is installed; importable only after `import torch`.
 #include <torch/csrc/autograd/python_variable.h>

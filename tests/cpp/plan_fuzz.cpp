@@ -141,10 +141,10 @@ int main(int argc, char** argv) {
     rc = axr_plan_bind(back, n ? c.tensors.data() : nullptr, n);
     if (rc != AXR_OK && rc != AXR_ERR_MISMATCH) die("bind", rc);
     if (rc == AXR_OK) inspect(back, n);
-    {   // the same in one pass: same verdict, same tables
+    {   // the same in one pass: same result, same tables
       axr_plan_t* fused = nullptr;
       const int rc1 = axr_plan_from_header_bind(bytes.data(), bytes.size(), n ? c.tensors.data() : nullptr, n, &fused);
-      if (rc1 != rc) die("from_header_bind verdict differs from from_header + bind", rc1);
+      if (rc1 != rc) die("from_header_bind result differs from from_header + bind", rc1);
       if (rc1 == AXR_OK) {
         inspect(fused, n);
         size_t c1 = 0, c2 = 0;

@@ -640,7 +640,7 @@ def test_torch_tensors_read_without_capsules_match_the_capsule_route(pkg):
     every descriptor field equals what a capsule from torch.utils.dlpack.to_dlpack carries, for
     each dtype torch exports and for views with size-1, size-0, stepped and permuted dimensions;
     anything Tensor.__dlpack__ would refuse, a subclass or a foreign producer makes it decline
-    (None), and the bundle then takes the capsule route with that route's verdict."""
+    (None), and the bundle then takes the capsule route with that route's answer."""
     import torch
     from execution_ucx_amd import dlpack
     direct = dlpack._native_torch()
