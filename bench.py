@@ -40,8 +40,11 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--rotate", type=int, default=4,
                     help="independent bundle copies cycled through by the steps (1 = cache resident)")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "transposed", "rows100", "rows250", "rows512", "stepped",
-                             "odd_transposed"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "small", "transposed", "rows100", "rows250", "rows512",
+                             "stepped", "odd_transposed"])
+    ap.add_argument("--align", type=int, default=256, help="pack alignment of the c2 and small workloads")
+    ap.add_argument("--direction", default="both", choices=["both", "pack", "unpack"],
+                    help="with --separate-launches: time only the packs or only the unpacks")
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--separate-launches", action="store_true",
                     help="time axr_pack + axr_unpack as two launches per step instead of one axr_submit")
@@ -139,6 +142,38 @@ def run_sets(h: Harness, sets, steps, warmup):
     return ms
 
 
+def run_sets_one_direction(h: Harness, sets, steps, warmup, unpack):
+    """Only the packs (unpack == False) or only the unpacks of the rotating sets, one launch
+    per step: what a sender and a receiver in different processes each see.  The payloads
+    must hold packed data before the unpacks are timed."""
+    lib, stream = h.lib, h.stream
+    n = len(sets)
+    calls = [(s.up if unpack else s.pp, s.ptr, s.nbytes) for s in sets]
+    fn = lib.axr_unpack if unpack else lib.axr_pack
+
+    def step(i):
+        plan, ptr, nb = calls[i % n]
+        rc = fn(plan, ptr, nb, stream)
+        if rc:
+            h.capi.check(rc)
+
+    return h.time_steps(step, steps, warmup)
+
+
+def half_rates(h: Harness, sets, steps, warmup):
+    """Pack-only and unpack-only figures of a workload: GB/s over the 2P bytes one
+    direction reads and writes, fraction of the HBM peak, microseconds per launch."""
+    P = sets[0].data_bytes
+    out = {}
+    for name, unpack in (("pack_only", False), ("unpack_only", True)):
+        ms = run_sets_one_direction(h, sets, steps, warmup, unpack)
+        us = ms * 1e3 / steps
+        gbps = 2.0 * P / (us * 1e-6) / 1e9
+        out[name] = {"GBps_2P": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "avg_launch_us": round(us, 3)}
+    return out
+
+
 def run_sets_one_launch(h: Harness, sets, steps, warmup, width=1):
     """Step i = axr_submit({packs of the next `width` sets, unpacks of the `width` sets packed
     by the step before}): one kernel launch that moves `width` bundles each way."""
@@ -205,13 +240,23 @@ def run_sets_two_streams(h: Harness, sets, steps, warmup):
     return times[len(times) // 2]
 
 
-def make_c2_sets(h, count, seed=0, align=256):
+def tensor_byte_mask(h, spec):
+    """Boolean device tensor over the arena: True for bytes that belong to a tensor."""
+    import numpy as np
+    edges = np.zeros(spec.arena_bytes + 1, dtype=np.int32)
+    starts = np.fromiter((s.arena_offset for s in spec.segments), dtype=np.int64, count=len(spec.segments))
+    sizes = np.fromiter((s.nbytes for s in spec.segments), dtype=np.int64, count=len(spec.segments))
+    np.add.at(edges, starts, 1)
+    np.add.at(edges, starts + sizes, -1)
+    return h.torch.from_numpy(np.cumsum(edges[:-1]) > 0).cuda()
+
+
+def make_c2_sets(h, count, seed=0, align=256, spec=None):
     from execution_ucx_amd import workloads
-    spec = workloads.mixed_bundle(seed=seed)
+    if spec is None:
+        spec = workloads.mixed_bundle(seed=seed)
     sets = []
-    mask = h.torch.zeros(spec.arena_bytes, dtype=h.torch.bool, device="cuda")
-    for s in spec.segments:
-        mask[s.arena_offset:s.arena_offset + s.nbytes] = True
+    mask = tensor_byte_mask(h, spec)
     for k in range(count):
         arena, _ = workloads.materialize_mixed(spec, "cuda", seed=seed + k)
         arena.mul_(mask)      # bytes between tensors are not part of the bundle: zero them
@@ -879,6 +924,51 @@ def small_bundles_batched(h, bundles=16, tensors=4, each=16 * 1024, steps=200):
             "sixteen_bundles_per_launch_us": round(ms_bat * 1e3 / (steps * bundles), 2)}
 
 
+def small_segments(h, tensors=65536, lo=8, hi=512, copies=4, steps=400):
+    """Bundles of many short tensors (RPC argument lists, norm scales, biases, optimizer
+    scalars): `tensors` contiguous 1-D tensors of lo..hi bytes, log-uniform, five dtypes, at
+    the benchmark's 256-byte alignment and in the reference's tight layout.  Pack-only,
+    unpack-only and pack + unpack rates next to a plain device copy of the same byte count
+    under the same rotation; launch geometry (wavefronts launched, device table bytes)."""
+    from execution_ucx_amd import workloads
+    torch, lib, check = h.torch, h.lib, h.capi.check
+    spec = workloads.mixed_bundle(n=tensors, lo=lo, hi=hi, seed=3)
+    out = {"tensors": tensors, "size_range_bytes": [lo, hi], "rotating_copies": copies}
+    for align in (256, 1):
+        _, sets = make_c2_sets(h, copies, seed=3, align=align, spec=spec)
+        for s_ in sets:
+            verify_set(h, s_)
+        P = sets[0].data_bytes
+        clear_sets(h, sets)
+        pair = run_sets(h, sets, steps, 20)
+        check_sets(h, sets, "the small-segment steps")
+        one = run_sets_one_launch(h, sets, steps, 20)
+        res = half_rates(h, sets, steps, 20)
+        info = sets[0].pack_plan.launch_info()
+        res.update({"payload_bytes_P": P, "packed_bytes": sets[0].nbytes,
+                    "pack_unpack_GBps_4P": round(rate(P, pair, steps), 1),
+                    "one_launch_GBps_4P": round(rate(P, one, steps), 1),
+                    "wavefronts": info["tiles"], "segments": info["segments"],
+                    "table_bytes": info["table_bytes"]})
+        out[f"align{align}"] = res
+        del sets
+        torch.cuda.empty_cache()
+    n = (out["align1"]["payload_bytes_P"] + 15) // 16 * 16
+    a = [torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda") for _ in range(copies)]
+    b = [torch.empty_like(x) for x in a]
+    h.sync()
+    ms = h.time_steps(lambda i: check(lib.axr_copy_reference(b[i % copies].data_ptr(), a[i % copies].data_ptr(),
+                                                             n, h.stream)), steps, 20)
+    us = ms * 1e3 / steps
+    out["plain_copy_same_bytes"] = {"bytes": n, "GBps_2n": round(2.0 * n / (us * 1e-6) / 1e9, 1),
+                                    "avg_launch_us": round(us, 3)}
+    for align in (256, 1):
+        r = out[f"align{align}"]
+        r["pack_vs_plain_copy"] = round(r["pack_only"]["GBps_2P"] / out["plain_copy_same_bytes"]["GBps_2n"], 3)
+        r["unpack_vs_plain_copy"] = round(r["unpack_only"]["GBps_2P"] / out["plain_copy_same_bytes"]["GBps_2n"], 3)
+    return out
+
+
 def load_traffic(kernel_key):
     path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
     try:
@@ -912,9 +1002,14 @@ def main():
     spec = workloads.mixed_bundle()
     extras = {}
     if args.workload == "c2":
-        _, sets = make_c2_sets(h, max(1, args.rotate))
+        _, sets = make_c2_sets(h, max(1, args.rotate), align=args.align)
         name = ("C2 mixed small-tensor bundle: 4096 contiguous 1-D tensors, log-uniform "
-                "256 B-64 KiB, fp16/bf16/fp32/int32/int8, 256 B aligned offsets")
+                f"256 B-64 KiB, fp16/bf16/fp32/int32/int8, {args.align} B aligned offsets")
+    elif args.workload == "small":
+        small_spec = workloads.mixed_bundle(n=65536, lo=8, hi=512, seed=3)
+        _, sets = make_c2_sets(h, max(1, args.rotate), seed=3, align=args.align, spec=small_spec)
+        name = ("65,536 contiguous 1-D tensors, log-uniform 8 B-512 B, five dtypes, "
+                f"{args.align} B aligned offsets")
     elif args.workload == "c3":
         sets = make_c3_sets(h, max(1, args.rotate))
         name = "C3 Llama-7B single-layer weight bundle, bf16, 9 tensors"
@@ -939,14 +1034,18 @@ def main():
         ms = run_sets_one_launch(h, sets, args.steps, args.warmup)
         launches_per_step, bytes_per_launch = 1, 4 * P
         kernel = "axr::bundle_jobs_kernel (one launch: pack of bundle i+1 and unpack of bundle i)"
+    elif args.direction != "both":
+        ms = run_sets_one_direction(h, sets, args.steps, args.warmup, args.direction == "unpack")
+        launches_per_step, bytes_per_launch = 1, 2 * P
+        kernel = f"axr::bundle_kernel ({args.direction} instantiation only)"
     else:
         ms = run_sets(h, sets, args.steps, args.warmup)
         launches_per_step, bytes_per_launch = 2, 2 * P
         kernel = "axr::bundle_kernel (pack and unpack instantiations)"
     batches = h.batches
-    if all(s.clear is not None for s in sets):
+    if all(s.clear is not None for s in sets) and (pipelined or args.direction == "both"):
         check_sets(h, sets, "the timed steps")
-    value = rate(P, ms, args.steps)
+    value = rate(P, ms, args.steps) * (0.5 if (not pipelined and args.direction != "both") else 1.0)
     info = sets[0].pack_plan.launch_info()
     launch_us = ms * 1e3 / (launches_per_step * args.steps)
     achieved = bytes_per_launch / (launch_us * 1e-6) / 1e9
@@ -1007,13 +1106,18 @@ def main():
                 one = run_sets_one_launch(h, vs, args.steps, args.warmup)
                 check_sets(h, vs, "a C2 variant")
                 two = run_sets(h, vs, args.steps, args.warmup)
-                return {"one_launch_GBps": round(rate(P, one, args.steps), 1),
-                        "separate_launches_GBps": round(rate(P, two, args.steps), 1)}
+                res = {"one_launch_GBps": round(rate(P, one, args.steps), 1),
+                       "separate_launches_GBps": round(rate(P, two, args.steps), 1)}
+                res.update(half_rates(h, vs, args.steps, args.warmup))
+                return res
             finally:
                 pkg.tune(**defaults)
 
         ms_sep = run_sets(h, sets, args.steps, args.warmup)
         extras["c2_separate_launches_GBps"] = round(rate(P, ms_sep, args.steps), 1)
+        # a deployed sender and receiver are different processes: each half on its own
+        halves = half_rates(h, sets, args.steps, args.warmup)
+        extras["c2_pack_only"], extras["c2_unpack_only"] = halves["pack_only"], halves["unpack_only"]
         # cache-resident rate of the same bundle (one copy only: pack then unpack)
         ms1 = run_sets(h, sets[:1], args.steps, args.warmup)
         extras["c2_cache_resident_GBps"] = round(rate(P, ms1, args.steps), 1)
@@ -1041,6 +1145,8 @@ def main():
         ms3 = run_sets(h, c3, k3, 5)
         ms3b = run_sets_one_launch(h, c3, k3, 5)
         check_sets(h, c3, "C3")
+        halves = half_rates(h, c3, k3, 5)
+        extras["c3_pack_only"], extras["c3_unpack_only"] = halves["pack_only"], halves["unpack_only"]
         extras["c3_llama_layer"] = {"GBps": round(rate(c3[0].data_bytes, ms3, k3), 1),
                                     "pct_of_hbm_peak": round(100 * rate(c3[0].data_bytes, ms3, k3) / HBM_PEAK_GBPS, 2),
                                     "one_launch_GBps": round(rate(c3[0].data_bytes, ms3b, k3), 1),
@@ -1081,6 +1187,7 @@ def main():
         finally:
             pkg.tune(spin_wait_us=0)
         extras["small_bundles_batched"] = small_bundles_batched(h)
+        extras["small_segments"] = small_segments(h)
         extras["c1_host_bundle"] = host_bundle_c1(h)
         extras["loopback_iov_vs_bundle"] = iov_against_bundle(h, spec)
         extras["python_plan_us_per_1k_tensors"] = python_boundary(h, spec)
@@ -1093,6 +1200,8 @@ def main():
         ms4 = run_sets(h, [c4], k4, 3)
         extras["c4_kv_gather"] = {"GBps": round(rate(c4.data_bytes, ms4, k4), 1),
                                   "payload_bytes_P": c4.data_bytes, "steps": k4}
+        halves = half_rates(h, [c4], k4, 3)
+        extras["c4_pack_only"], extras["c4_unpack_only"] = halves["pack_only"], halves["unpack_only"]
         del c4
         torch.cuda.empty_cache()
     if args.calibrate_copy:
