@@ -52,6 +52,8 @@ def parse_args():
     ap.add_argument("--tune", default="", help="comma separated key=value kernel tunables")
     ap.add_argument("--ceilings", action="store_true",
                     help="print what the plain copy, fill and row kernels reach on this device and exit")
+    ap.add_argument("--small-segments", action="store_true",
+                    help="print the report of the many-short-tensors workload (65,536 tensors of 8-512 B) and exit")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N plain 256 MiB device copies (axr_copy_reference) so that "
                          "profiler counters can be scaled by a kernel of known traffic")
@@ -998,6 +1000,9 @@ def main():
 
     if args.ceilings:
         print(json.dumps({"ceilings": ceilings(h)}))
+        return
+    if args.small_segments:
+        print(json.dumps({"small_segments": small_segments(h)}))
         return
     spec = workloads.mixed_bundle()
     extras = {}

@@ -35,7 +35,10 @@ constexpr uint32_t kMaxOuterDims = 6;
 constexpr uint32_t kSegPadMask = 0xfffu;         // meta bits 0..11: zero bytes after segment
 constexpr uint32_t kSegDimsShift = 12;           // meta bits 12..31: 1 + dims index
 constexpr uint32_t kSegFillOnly = 0xfffffu;      // dims field value: segment only writes zeros
+constexpr uint32_t kSegGroup = 0xffffeu;         // dims field value: one tile that holds several short tensors
 constexpr uint32_t kMaxAlign = 4096;
+constexpr uint32_t kDirectSegShift = 0xffu;      // seg_shift value: every segment is exactly one tile
+constexpr uint32_t kGroupBlocksShift = 0xfeu;    // seg_shift value: every tile is a group block at a fixed stride
 // run_bytes of a contiguous (not strided) segment carries, in its top byte, the number
 // of leading bytes (< 128) that tile 0 moves in addition to its own range: with them
 // peeled off, every tile of the segment starts on a 128-byte line of the written side.
@@ -51,6 +54,42 @@ struct Seg {              // 32 bytes
   uint32_t meta;          // pad | (dims index + 1) << 12
 };
 static_assert(sizeof(Seg) == 32, "Seg layout");
+
+// A group tile: several whole short contiguous tensors that follow each other in the bundle
+// are moved by ONE wavefront.  Every group has a block of kGroupBlockBytes in the table block
+// (behind the tile-block index): a GroupHead, then up to kGroupMaxMembers Member records.  The
+// group's Seg carries, in `ptr`, the byte offset of that block from the start of the segment
+// table.  A bundle that consists of group tiles only needs neither its Seg records nor the
+// index on the device: tile t's block lies at t * kGroupBlockBytes (seg_shift ==
+// kGroupBlocksShift; the kernel's `dims` argument then points at the blocks), which takes
+// one dependent memory access out of every wavefront's path.
+// A member of n bytes followed by `pad` zero bytes occupies max(1, ceil(n / 16)) data slots,
+// then ceil(pad / 16) zero slots when pad >= 16; a slot is one 16-byte access of one lane, the
+// last data (zero) slot covering the member's (gap's) final 16 bytes.  Members shorter than 16
+// bytes and gaps shorter than 16 bytes move in pieces of 8, 4, 2 and 1 bytes in the lane of
+// the member's last data slot.
+constexpr uint32_t kGroupMaxMembers = 16;
+constexpr uint32_t kGroupMaxSlots = 128;         // two 16-byte accesses per lane
+constexpr uint32_t kGroupMaxMemberBytes = 1023;
+struct Member {           // 16 bytes
+  uint64_t ptr;           // tensor-side address
+  uint32_t off_pad;       // bits 0-19: payload offset from the group's first byte; bits 20-31: pad
+  uint16_t nbytes;        // 1 .. kGroupMaxMemberBytes
+  uint16_t begin;         // first slot of the member
+};
+static_assert(sizeof(Member) == 16, "Member layout");
+struct GroupHead {        // 32 bytes
+  uint64_t starts[2];     // bit j of starts[r]: lane slot 64 r + j is the first slot of a member, so
+                          // that a slot finds its member by counting bits instead of searching
+  uint64_t off;           // payload offset of the group's first member
+  uint32_t members;
+  uint32_t slots;
+};
+static_assert(sizeof(GroupHead) == 32, "GroupHead layout");
+constexpr uint32_t kGroupBlockBytes = sizeof(GroupHead) + kGroupMaxMembers * sizeof(Member);   // 288
+constexpr uint32_t kMemberOffBits = 20;
+constexpr uint32_t group_data_slots(uint32_t nbytes) { return nbytes >= kVecBytes ? (nbytes + kVecBytes - 1) / kVecBytes : 1u; }
+constexpr uint32_t group_pad_slots(uint32_t pad) { return pad >= kVecBytes ? (pad + kVecBytes - 1) / kVecBytes : 0u; }
 
 constexpr uint32_t kModeRunTiles = 0;   // every tile is a piece of one contiguous run
 constexpr uint32_t kModeElements = 1;   // tile covers packed bytes; lanes decode granules
@@ -198,6 +237,11 @@ struct Tunables {
   // back to the runtime's wait (0, the default: the runtime's wait only).  See the header.
   std::atomic<int64_t> spin_wait_us{0};
   std::atomic<int64_t> host_threads{4};       // threads (the caller included) for host-side staging copies
+  // Contiguous device tensors of at most this many bytes that follow each other in a bundle
+  // share wavefronts (group tiles, up to 64 tensors or 2 KiB of lane slots each); 0: every
+  // tensor gets its own wavefronts.
+  std::atomic<int64_t> group_bytes{512};
+  std::atomic<int64_t> group_slots{kGroupMaxSlots};   // lane slots per group tile: 64 or 128
   std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
 };

@@ -756,6 +756,172 @@ __device__ __attribute__((noinline)) void transpose_tile(uint64_t seg_ptr, dims_
   }
 }
 
+// ---------------------------------------------------------------- group tiles
+//
+// Several whole short tensors moved by one wavefront.  A group's block in the table holds
+// one 64-bit mask per round of 64 lane slots (bit j: slot j is the first slot of a member),
+// the group's payload offset and counts, and then the member records.  Lane l loads member
+// l's record while the head arrives by scalar load; slot s finds its member by counting the mask bits up to s (two ALU
+// instructions), fetches that member's record from the lane that holds it through the
+// cross-lane permute, and moves its 16 bytes: the last data slot of a member covers the
+// member's final 16 bytes, the zero slots behind it clear the gap to the next aligned
+// offset.  Members and gaps shorter than 16 bytes move in pieces of 8, 4, 2 and 1 bytes.
+// Both rounds of 64 slots are in flight together: record fetches, then loads, then stores.
+__device__ __forceinline__ uint32_t lane_value(uint32_t from_lane, uint32_t value) {
+  return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(static_cast<int>(from_lane << 2), static_cast<int>(value)));
+}
+
+template <bool PACK>
+__device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* head, gbytes payload,
+                                                     uint64_t delta, uint32_t lane) {
+  typedef uint64_t __attribute__((aligned(1))) loose64;
+  typedef uint32_t __attribute__((aligned(1))) loose32;
+  typedef uint16_t __attribute__((aligned(1))) loose16;
+  constexpr uint32_t R = kGroupMaxSlots / kWaveLanes;
+  static_assert(R == 2, "two masks per group head");
+  uint32_t my_lo = 0, my_hi = 0, my_off_pad = 0, my_nb = 0;
+  if (lane < kGroupMaxMembers) {   // (records past the group's last member are zero)
+    const AXR_CONST Member* recs = reinterpret_cast<const AXR_CONST Member*>(head + 1);
+    const u32x4 r = *reinterpret_cast<const AXR_CONST u32x4*>(recs + lane);
+    my_lo = r.x;
+    my_hi = r.y;
+    my_off_pad = r.z;
+    my_nb = r.w;
+  }
+  // member of slot s: the number of members that begin at or before s, minus one
+  const uint64_t mask0 = head->starts[0], mask1 = head->starts[1];
+  gbytes pay = payload + head->off;
+  const uint32_t slots = head->slots;
+  uint32_t m[R];
+  {
+    const uint32_t lo0 = static_cast<uint32_t>(mask0), hi0 = static_cast<uint32_t>(mask0 >> 32);
+    const uint32_t lo1 = static_cast<uint32_t>(mask1), hi1 = static_cast<uint32_t>(mask1 >> 32);
+    // mbcnt counts the mask bits below this lane; the lane's own bit is added
+    m[0] = __builtin_amdgcn_mbcnt_hi(hi0, __builtin_amdgcn_mbcnt_lo(lo0, 0)) +
+           static_cast<uint32_t>((mask0 >> lane) & 1u) - 1u;
+    m[1] = static_cast<uint32_t>(__builtin_popcountll(mask0)) +
+           __builtin_amdgcn_mbcnt_hi(hi1, __builtin_amdgcn_mbcnt_lo(lo1, 0)) +
+           static_cast<uint32_t>((mask1 >> lane) & 1u) - 1u;
+  }
+  uint32_t f_lo[R], f_hi[R], f_off_pad[R], f_nb[R];
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) {
+    const uint32_t from = m[r] & (kGroupMaxMembers - 1u);
+    f_lo[r] = lane_value(from, my_lo);
+    f_hi[r] = lane_value(from, my_hi);
+    f_off_pad[r] = lane_value(from, my_off_pad);
+    f_nb[r] = lane_value(from, my_nb);
+  }
+  gbytes ten[R], pp[R];
+  uint32_t kind[R];      // 0 nothing, 1 sixteen data bytes, 2 sixteen zero bytes (pack)
+  uint32_t small_n[R];   // a member shorter than 16 bytes: its length, in the lane of its only data slot
+  uint32_t small_pad[R]; // a gap shorter than 16 bytes, in the lane of the member's last data slot
+  gbytes gap_at[R], small_pp[R];
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) {
+    const uint32_t s = r * kWaveLanes + lane;
+    const uint64_t ptr = (static_cast<uint64_t>(f_hi[r]) << 32 | f_lo[r]) + delta;
+    const uint32_t off_pad = f_off_pad[r], nb = f_nb[r];
+    const uint32_t n = nb & 0xffffu, k = s - (nb >> 16);
+    const uint32_t rel = off_pad & ((1u << kMemberOffBits) - 1u), pad = off_pad >> kMemberOffBits;
+    const uint32_t dslots = group_data_slots(n), pslots = group_pad_slots(pad);
+    const bool live = s < slots;
+    gbytes t0 = as_global(ptr), p0 = pay + rel;
+    kind[r] = 0;
+    small_n[r] = 0;
+    small_pad[r] = 0;
+    ten[r] = t0;
+    pp[r] = p0;
+    gap_at[r] = p0;
+    small_pp[r] = p0;
+    if (live && k < dslots) {
+      if (n >= kVecBytes) {
+        const uint32_t o = (k + 1u == dslots) ? n - kVecBytes : k * kVecBytes;
+        ten[r] = t0 + o;
+        pp[r] = p0 + o;
+        kind[r] = 1;
+      } else {
+        small_n[r] = n;
+      }
+      if (PACK && k + 1u == dslots && pad && pad < kVecBytes) small_pad[r] = pad;
+    } else if (PACK && live && k < dslots + pslots) {
+      const uint32_t j = k - dslots;
+      pp[r] = p0 + n + ((j + 1u == pslots) ? pad - kVecBytes : j * kVecBytes);
+      kind[r] = 2;
+    }
+    if (PACK && small_pad[r]) gap_at[r] = p0 + n;   // where the short gap begins (payload side)
+  }
+  // Ordinary (cacheable) accesses on both sides whatever the launch's hints: short tensors
+  // share their 128-byte lines with their neighbours, and a line marked as streaming is fetched
+  // again for the next member (measured: 5 to 15 % slower with either hint).
+  // Every load of the tile, the pieces of members shorter than 16 bytes included, is issued
+  // before the first store: one memory round trip for the whole tile.
+  bool any_small = false;
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) any_small = any_small || small_n[r] != 0;
+  const bool wave_has_small = __builtin_amdgcn_ballot_w64(any_small) != 0;   // wave-uniform: most groups have none
+  u32x4 v[R];
+  uint64_t a8[R];
+  uint32_t b4[R];
+  uint16_t c2[R];
+  uint8_t d1[R];
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) {
+    v[r] = u32x4{0u, 0u, 0u, 0u};
+    if (kind[r] == 1) v[r] = load16<false>(PACK ? ten[r] : pp[r]);
+  }
+  if (wave_has_small) {
+#pragma unroll
+    for (uint32_t r = 0; r < R; ++r) {
+      const uint32_t n = small_n[r];
+      gcbytes src = PACK ? ten[r] : small_pp[r];
+      a8[r] = 0;
+      b4[r] = 0;
+      c2[r] = 0;
+      d1[r] = 0;
+      if (n & 8u) a8[r] = *reinterpret_cast<const AXR_GLOBAL loose64*>(src);
+      if (n & 4u) b4[r] = *reinterpret_cast<const AXR_GLOBAL loose32*>(src + (n & 8u));
+      if (n & 2u) c2[r] = *reinterpret_cast<const AXR_GLOBAL loose16*>(src + (n & 12u));
+      if (n & 1u) d1[r] = src[n & 14u];
+    }
+  }
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) asm volatile("" : "+v"(v[r])::"memory");
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) {
+    if (kind[r] == 1) store16<false>(PACK ? pp[r] : ten[r], v[r]);
+    else if (kind[r] == 2) store16<false>(pp[r], v[r]);
+  }
+  if (wave_has_small) {
+#pragma unroll
+    for (uint32_t r = 0; r < R; ++r) {
+      const uint32_t n = small_n[r];
+      gbytes dst = PACK ? small_pp[r] : ten[r];
+      if (n & 8u) *reinterpret_cast<AXR_GLOBAL loose64*>(dst) = a8[r];
+      if (n & 4u) *reinterpret_cast<AXR_GLOBAL loose32*>(dst + (n & 8u)) = b4[r];
+      if (n & 2u) *reinterpret_cast<AXR_GLOBAL loose16*>(dst + (n & 12u)) = c2[r];
+      if (n & 1u) dst[n & 14u] = d1[r];
+    }
+  }
+  if constexpr (PACK) {
+    // gaps shorter than 16 bytes (tight layouts have none)
+    bool any_gap = false;
+#pragma unroll
+    for (uint32_t r = 0; r < R; ++r) any_gap = any_gap || small_pad[r] != 0;
+    if (__builtin_amdgcn_ballot_w64(any_gap) != 0) {
+#pragma unroll
+      for (uint32_t r = 0; r < R; ++r) {
+        const uint32_t z = small_pad[r];
+        gbytes dst = gap_at[r];
+        if (z & 8u) *reinterpret_cast<AXR_GLOBAL loose64*>(dst) = 0;
+        if (z & 4u) *reinterpret_cast<AXR_GLOBAL loose32*>(dst + (z & 8u)) = 0;
+        if (z & 2u) *reinterpret_cast<AXR_GLOBAL loose16*>(dst + (z & 12u)) = 0;
+        if (z & 1u) dst[z & 14u] = 0;
+      }
+    }
+  }
+}
+
 // The whole pack or unpack of a bundle: every wavefront finds the segment of its
 // first tile through the tile-block index and walks forward from there.  `wg` is the
 // workgroup's index within this bundle's share of the grid; `a.tensor_delta` is added to
@@ -779,10 +945,19 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
   const uint32_t t_end =
       (a.ntiles - t > a.tiles_per_wave) ? t + a.tiles_per_wave : a.ntiles;
   const uint64_t delta = static_cast<uint64_t>(a.tensor_delta);
+  if (a.seg_shift == kGroupBlocksShift) {
+    // a bundle of group tiles only: tile t's block lies at a fixed stride behind `dims`
+    const AXR_CONST uint8_t* blocks = reinterpret_cast<const AXR_CONST uint8_t*>(dims);
+    for (; t < t_end; ++t)
+      group_tile<PACK>(reinterpret_cast<const AXR_CONST GroupHead*>(blocks + static_cast<uint64_t>(t) * kGroupBlockBytes),
+                       payload, delta, lane);
+    return;
+  }
   // The index has one entry per block of 2^seg_shift tiles (the planner sizes
   // blocks so that they rarely hold more than one segment); the loop below
   // walks forward from there to the segment of this wave's first tile.
-  uint32_t s = wave_seg[t >> a.seg_shift];
+  // (a bundle whose segments are one tile each needs no index: tile t is segment t)
+  uint32_t s = a.seg_shift == kDirectSegShift ? t : wave_seg[t >> a.seg_shift];
   uint64_t seg_ptr = segs[s].ptr + delta, seg_off = segs[s].off, seg_run = segs[s].run_bytes;
   uint32_t seg_begin = segs[s].tile_begin, seg_meta = segs[s].meta;
   uint32_t seg_end = segs[s + 1].tile_begin;
@@ -822,6 +997,11 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
       }
     } else if (dsel == kSegFillOnly) {
       if constexpr (PACK) wave_zero(pay, pad, lane);
+    } else if (dsel == kSegGroup) {
+      // seg_ptr is an offset into the table block here, not a tensor address
+      const AXR_CONST GroupHead* head = reinterpret_cast<const AXR_CONST GroupHead*>(
+          reinterpret_cast<const AXR_CONST uint8_t*>(segs) + (seg_ptr - delta));
+      group_tile<PACK>(head, payload, delta, lane);
     } else {
       dims_table dm = dims + (dsel - 1);
       if (dm->mode == kModeRunTiles) {

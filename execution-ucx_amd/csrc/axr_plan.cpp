@@ -179,6 +179,9 @@ struct axr_plan {
   std::vector<Dims> dims;
   std::vector<uint32_t> wave_seg;
   std::vector<uint32_t> seg_tensor;  // tensor index per segment (inspection)
+  std::vector<uint8_t> group_blocks; // kGroupBlockBytes per group tile: GroupHead, then Member records
+  std::vector<uint32_t> member_tensor;   // kGroupMaxMembers tensor indices per block (inspection)
+  bool groups_only = false;          // every tile is a group tile: the kernel walks the blocks directly
   std::vector<HostCopy> host_copies;
   std::vector<uint32_t> host_copy_tensor;
   std::vector<HostChunk> host_chunks;
@@ -189,7 +192,7 @@ struct axr_plan {
   LaunchConfig cfg;
   TableBlock block;
   size_t table_bytes = 0;
-  size_t dims_at = 0, wave_at = 0;
+  size_t dims_at = 0, wave_at = 0, members_at = 0;
   bool uploaded = false;
   bool resident = false;             // upload known to be complete (axr_plan_prepare)
   size_t stage_bytes = 0;            // longest host chunk: size of the staging blocks
@@ -347,6 +350,9 @@ void invalidate_tables(axr_plan* p) {
   p->dims.clear();
   p->wave_seg.clear();
   p->seg_tensor.clear();
+  p->group_blocks.clear();
+  p->member_tensor.clear();
+  p->groups_only = false;
   p->host_copies.clear();
   p->host_copy_tensor.clear();
   p->host_chunks.clear();
@@ -471,6 +477,79 @@ struct Builder {
   uint64_t head_align;    // 0 or a power of two up to 128
   uint64_t tiles = 0;
   uint64_t shared_line_tiles = 0;   // transposed blocks whose rows straddle 128-byte lines
+  uint64_t group_bytes = 0;         // longest tensor that may share a wavefront (0: none)
+  uint32_t slots_per_group = kGroupMaxSlots;
+  // the group being collected (when open): the last block of p->group_blocks
+  bool group_open = false;
+  uint32_t group_count = 0;
+  uint32_t group_slots = 0;
+  uint64_t group_off = 0;
+  uint64_t group_starts[2] = {0, 0};
+
+  uint8_t* open_block() { return p->group_blocks.data() + p->group_blocks.size() - kGroupBlockBytes; }
+
+  // A short contiguous device tensor joins the open group, which is closed first when the
+  // tensor does not fit (16 members, 128 lane slots, offsets within 1 MiB of the first).
+  // Returns false for a tensor that cannot be a member at all.
+  bool add_member(uint32_t tensor, uint64_t ptr, uint64_t off, uint64_t nbytes, uint64_t pad, int* rc) {
+    *rc = AXR_OK;
+    if (group_bytes == 0 || nbytes == 0 || nbytes > group_bytes || nbytes > kGroupMaxMemberBytes || pad >= kMaxAlign)
+      return false;
+    const uint32_t need = group_data_slots(static_cast<uint32_t>(nbytes)) + group_pad_slots(static_cast<uint32_t>(pad));
+    if (need > slots_per_group / 2) return false;
+    if (group_open && (group_count >= kGroupMaxMembers || group_slots + need > slots_per_group ||
+                       off < group_off || off - group_off >= (1ull << kMemberOffBits))) {
+      *rc = close_group();
+      if (*rc) return true;
+    }
+    if (!group_open) {
+      group_open = true;
+      group_count = 0;
+      group_slots = 0;
+      group_off = off;
+      group_starts[0] = group_starts[1] = 0;
+      p->group_blocks.resize(p->group_blocks.size() + kGroupBlockBytes, 0);
+      p->member_tensor.resize(p->member_tensor.size() + kGroupMaxMembers, 0);
+    }
+    Member m;
+    m.ptr = ptr;
+    m.off_pad = static_cast<uint32_t>(off - group_off) | static_cast<uint32_t>(pad) << kMemberOffBits;
+    m.nbytes = static_cast<uint16_t>(nbytes);
+    m.begin = static_cast<uint16_t>(group_slots);
+    std::memcpy(open_block() + sizeof(GroupHead) + group_count * sizeof(Member), &m, sizeof(m));
+    p->member_tensor[p->member_tensor.size() - kGroupMaxMembers + group_count] = tensor;
+    group_starts[group_slots >> 6] |= 1ull << (group_slots & 63u);
+    ++group_count;
+    group_slots += need;
+    return true;
+  }
+
+  // Ends the open group: one tile for two members or more, an ordinary segment for one.
+  int close_group() {
+    if (!group_open) return AXR_OK;
+    group_open = false;
+    if (group_count == 1) {
+      Member m;
+      std::memcpy(&m, open_block() + sizeof(GroupHead), sizeof(m));
+      const uint32_t tensor = p->member_tensor[p->member_tensor.size() - kGroupMaxMembers];
+      p->group_blocks.resize(p->group_blocks.size() - kGroupBlockBytes);
+      p->member_tensor.resize(p->member_tensor.size() - kGroupMaxMembers);
+      int rc = add_seg(tensor, m.ptr, group_off, m.nbytes, 1, 0);
+      if (!rc) p->segs.back().meta |= m.off_pad >> kMemberOffBits;
+      return rc;
+    }
+    GroupHead head;
+    head.starts[0] = group_starts[0];
+    head.starts[1] = group_starts[1];
+    head.off = group_off;
+    head.members = group_count;
+    head.slots = group_slots;
+    std::memcpy(open_block(), &head, sizeof(head));
+    const size_t index = p->group_blocks.size() / kGroupBlockBytes - 1;
+    // `ptr` holds the index of the group's block until the table sections are laid out
+    return add_seg(p->member_tensor[index * kGroupMaxMembers], index, group_off,
+                   static_cast<uint64_t>(group_count) | static_cast<uint64_t>(group_slots) << 8, 1, kSegGroup);
+  }
 
   int add_seg(uint32_t tensor, uint64_t ptr, uint64_t off, uint64_t run_bytes, uint64_t ntile,
               uint32_t dsel) {
@@ -702,7 +781,7 @@ int build_tables(axr_plan* p);
 // the grid would exceed max_waves, workgroup size, cache hints, and the size of the blocks of
 // the tile-block index (about one segment each, a power of two up to 256 tiles: a bundle of
 // few large tensors gets a tiny index, a bundle of many small ones an entry per few tiles).
-void finish_geometry(axr_plan* p, uint32_t rows, size_t nseg) {
+void finish_geometry(axr_plan* p, uint32_t rows, size_t nseg, bool may_be_direct = false) {
   const Tunables& tn = tunables();
   uint64_t tpw = (p->ntiles + static_cast<uint64_t>(tn.max_waves) - 1) /
                  static_cast<uint64_t>(tn.max_waves);
@@ -735,7 +814,8 @@ void finish_geometry(axr_plan* p, uint32_t rows, size_t nseg) {
   }
   uint32_t shift = 0;
   while (shift < 8 && (static_cast<uint64_t>(nseg) << (shift + 1)) <= p->ntiles) ++shift;
-  p->cfg.seg_shift = shift;
+  // as many tiles as segments (none without a tile): tile t is segment t, no index to consult
+  p->cfg.seg_shift = may_be_direct && nseg == p->ntiles ? kDirectSegShift : shift;
 }
 
 // Tile rows of a bundle whose tensors are all compact: 2 KiB tiles, doubled while the bundle
@@ -773,6 +853,14 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   const size_t n = p->tensors.size();
   const int64_t least = tn.device_tables;
   if (least <= 0 || n < static_cast<uint64_t>(least) || n > (1u << 20) || !p->bound) return AXR_OK;
+  if (tn.group_bytes > 0) {
+    // a bundle in which a quarter of the tensors are short enough to share wavefronts takes the
+    // general path, which builds group tiles
+    const uint64_t limit = static_cast<uint64_t>(tn.group_bytes);
+    size_t small = 0;
+    for (size_t i = 0; i < n; ++i) small += (p->tensors[i].nbytes - 1) < limit ? 1 : 0;   // 1 .. limit
+    if (small * 4 >= n) return AXR_OK;
+  }
   const uint32_t rows = rows_for_compact_bundle(p);
   const uint32_t tile_bytes = rows * kRowBytes;
   const uint32_t tile_shift = static_cast<uint32_t>(__builtin_ctz(tile_bytes));
@@ -898,6 +986,8 @@ int build_tables(axr_plan* p) {
   }
   Builder b{p, rows * kRowBytes, static_cast<uint32_t>(__builtin_ctz(rows * kRowBytes)),
             static_cast<uint64_t>(tn.head_align)};
+  b.group_bytes = static_cast<uint64_t>(tn.group_bytes);
+  b.slots_per_group = static_cast<uint32_t>(tn.group_slots);
   p->segs.reserve(p->tensors.size() + 1);
   p->seg_tensor.reserve(p->tensors.size());
 
@@ -922,11 +1012,19 @@ int build_tables(axr_plan* p) {
     }
     int rc;
     if (t.device_type == kDLROCM || t.device_type == kDLROCMHost) {
+      if (c.nd == 0 && b.add_member(static_cast<uint32_t>(i), t.address, t.offset, t.nbytes, pad, &rc)) {
+        if (rc) return rc;
+        continue;
+      }
+      rc = b.close_group();
+      if (rc) return rc;
       rc = b.add_strided(static_cast<uint32_t>(i), t.address, t.offset, c.extent, c.stride, c.nd,
                          c.run_bytes);
       if (rc) return rc;
       if (pad) p->segs.back().meta |= static_cast<uint32_t>(pad);
     } else if (t.device_type == kDLCPU) {
+      rc = b.close_group();
+      if (rc) return rc;
       rc = b.add_host(static_cast<uint32_t>(i), t.address, t.offset, c.extent, c.stride, c.nd,
                       c.run_bytes);
       if (rc) return rc;
@@ -939,6 +1037,10 @@ int build_tables(axr_plan* p) {
       return fail(AXR_ERR_UNSUPPORTED,
                   "Unsupported memory type: DLPack device " + std::to_string(t.device_type));
     }
+  }
+  {
+    int rc = b.close_group();
+    if (rc) return rc;
   }
   // Group neighbouring host pieces (in payload order, at most an alignment gap
   // apart) into chunks that fit one staging block.
@@ -966,17 +1068,25 @@ int build_tables(axr_plan* p) {
   p->segs.push_back(sentinel);
 
   const size_t nseg = p->segs.size() - 1;
-  finish_geometry(p, rows, nseg);
+  bool one_tile_each = true;
+  for (size_t i = 0; i < nseg && one_tile_each; ++i)
+    one_tile_each = p->segs[i + 1].tile_begin - p->segs[i].tile_begin == 1;
+  finish_geometry(p, rows, nseg, one_tile_each);
+  // group tiles only: the kernel finds tile t's block at a fixed stride, without the segment
+  // records and the index
+  p->groups_only = nseg != 0 && p->group_blocks.size() == nseg * kGroupBlockBytes;
+  if (p->groups_only) p->cfg.seg_shift = kGroupBlocksShift;
 
   // Tile-block index: entry k = segment that holds tile k << seg_shift.  Blocks
   // are sized to about one segment each (a power of two, at most 256 tiles), so
   // a bundle of few large tensors gets a tiny index and a bundle of many small
   // ones one entry per few tiles; a wave walks at most a segment or two forward.
   const uint32_t shift = p->cfg.seg_shift;
-  const size_t nblocks = (static_cast<size_t>(p->ntiles) >> shift) + 1;
+  const bool no_index = shift == kDirectSegShift || shift == kGroupBlocksShift;
+  const size_t nblocks = no_index ? 1 : (static_cast<size_t>(p->ntiles) >> shift) + 1;
   p->wave_seg.assign(nblocks, 0);
   size_t s = 0;
-  for (size_t k = 0; k < nblocks; ++k) {
+  for (size_t k = 0; k < nblocks && !no_index; ++k) {
     const uint64_t t0 = static_cast<uint64_t>(k) << shift;
     if (t0 >= p->ntiles) break;
     while (s + 1 < nseg && p->segs[s + 1].tile_begin <= t0) ++s;
@@ -985,9 +1095,30 @@ int build_tables(axr_plan* p) {
 
   p->dims_at = align_up(p->segs.size() * sizeof(Seg), 16);
   p->wave_at = align_up(p->dims_at + p->dims.size() * sizeof(Dims), 16);
-  p->table_bytes = p->wave_at + p->wave_seg.size() * sizeof(uint32_t);
+  p->members_at = align_up(p->wave_at + p->wave_seg.size() * sizeof(uint32_t), 16);
+  p->table_bytes = p->members_at + p->group_blocks.size();
+  if (!p->group_blocks.empty()) {
+    // a group's segment names its block by the block's offset in the table block
+    if (p->table_bytes > 0xffffffffull) return fail(AXR_ERR_UNSUPPORTED, "bundle tables exceed 4 GiB");
+    for (size_t i = 0; i < nseg; ++i) {
+      Seg& sg = p->segs[i];
+      if ((sg.meta >> kSegDimsShift) == kSegGroup) sg.ptr = p->members_at + sg.ptr * kGroupBlockBytes;
+    }
+  }
   p->tables_built = true;
   return AXR_OK;
+}
+
+// Where the kernel's `dims` argument points inside the table block: at the Dims records, or,
+// for a bundle of group tiles only, at the group blocks.
+size_t dims_arg_at(const axr_plan* p) { return p->groups_only ? p->members_at : p->dims_at; }
+
+// The host-built tables laid out as one block (segments, dims, tile-block index, group blocks).
+void write_tables(const axr_plan* p, uint8_t* h) {
+  std::memcpy(h, p->segs.data(), p->segs.size() * sizeof(Seg));
+  if (!p->dims.empty()) std::memcpy(h + p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims));
+  std::memcpy(h + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t));
+  if (!p->group_blocks.empty()) std::memcpy(h + p->members_at, p->group_blocks.data(), p->group_blocks.size());
 }
 
 int ensure_uploaded(axr_plan* p, hipStream_t stream) {
@@ -1004,9 +1135,7 @@ int ensure_uploaded(axr_plan* p, hipStream_t stream) {
       quiesce(p);   // previous launches may still read the old tables
     }
     uint8_t* h = static_cast<uint8_t*>(p->block.host);
-    std::memcpy(h, p->segs.data(), p->segs.size() * sizeof(Seg));
-    if (!p->dims.empty()) std::memcpy(h + p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims));
-    std::memcpy(h + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t));
+    write_tables(p, h);
     int rc = check_hip(hipMemcpyAsync(p->block.device, h, p->table_bytes, hipMemcpyHostToDevice,
                                       stream),
                        "hipMemcpyAsync(plan tables)");
@@ -1126,10 +1255,7 @@ void fill_inline_tables(axr_plan* p) {
   uint8_t* b = p->inline_tables->bytes;
   std::memset(b, 0, kInlineTablesHead);
   std::memcpy(b, &kInlineTablesMark, sizeof(kInlineTablesMark));
-  uint8_t* h = b + kInlineTablesHead;
-  std::memcpy(h, p->segs.data(), p->segs.size() * sizeof(Seg));
-  if (!p->dims.empty()) std::memcpy(h + p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims));
-  std::memcpy(h + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t));
+  write_tables(p, b + kInlineTablesHead);
   p->inline_ready = true;
 }
 
@@ -1195,7 +1321,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
     // host and 4 us on the device, once).
     if (!p->inline_ready) fill_inline_tables(p);
     rc = launch_bundle_kernel_inline(pack, a, p->cfg, *p->inline_tables,
-                                     static_cast<uint32_t>(p->dims_at),
+                                     static_cast<uint32_t>(dims_arg_at(p)),
                                      static_cast<uint32_t>(p->wave_at), stream);
     if (rc) return rc;
     ++p->launches;
@@ -1213,7 +1339,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   }
   uint8_t* d = static_cast<uint8_t*>(p->block.device);
   a.segs = reinterpret_cast<const Seg*>(d);
-  a.dims = reinterpret_cast<const Dims*>(d + p->dims_at);
+  a.dims = reinterpret_cast<const Dims*>(d + dims_arg_at(p));
   a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
   rc = launch_bundle_kernel(pack, a, cfg, stream);
   if (rc) return rc;
@@ -1662,7 +1788,7 @@ static int pack_noalloc_body(axr_plan_t* p, void* payload, size_t payload_bytes,
   if (tables_fit_kernel_arguments(p)) {
     if (!p->inline_ready) fill_inline_tables(p);
     rc = launch_bundle_kernel_inline(true, a, p->cfg, *p->inline_tables,
-                                     static_cast<uint32_t>(p->dims_at),
+                                     static_cast<uint32_t>(dims_arg_at(p)),
                                      static_cast<uint32_t>(p->wave_at), stream);
     if (rc) return rc;
     ++p->launches;
@@ -1694,9 +1820,13 @@ static int pack_noalloc_body(axr_plan_t* p, void* payload, size_t payload_bytes,
     rc = check_hip(hipMemcpyAsync(d + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t),
                                   hipMemcpyHostToDevice, stream),
                    "hipMemcpyAsync(tile index -> static area)");
+  if (!rc && !p->group_blocks.empty())
+    rc = check_hip(hipMemcpyAsync(d + p->members_at, p->group_blocks.data(), p->group_blocks.size(),
+                                  hipMemcpyHostToDevice, stream),
+                   "hipMemcpyAsync(member records -> static area)");
   if (rc) return rc;
   a.segs = reinterpret_cast<const Seg*>(d);
-  a.dims = reinterpret_cast<const Dims*>(d + p->dims_at);
+  a.dims = reinterpret_cast<const Dims*>(d + dims_arg_at(p));
   a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
   rc = launch_bundle_kernel(true, a, p->cfg, stream);
   if (rc) return rc;
@@ -1785,7 +1915,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
       const uint8_t* d = static_cast<const uint8_t*>(p->block.device);
       JobDesc& jd = table.job[k - i];
       jd.segs = reinterpret_cast<uint64_t>(d);
-      jd.dims = reinterpret_cast<uint64_t>(d + p->dims_at);
+      jd.dims = reinterpret_cast<uint64_t>(d + dims_arg_at(p));
       jd.wave_seg = reinterpret_cast<uint64_t>(d + p->wave_at);
       jd.payload = reinterpret_cast<uint64_t>(j.payload);
       jd.tensor_delta = j.tensor_delta;
@@ -1872,10 +2002,40 @@ static int plan_segments_body(axr_plan_t* plan, axr_segment_info_t* out, size_t 
   int rc = build_tables(plan);
   if (rc) return rc;
   const size_t nseg = plan->segs.size() - 1;
-  *count = nseg + plan->host_copies.size();
+  size_t groups = 0;
+  for (size_t i = 0; i < nseg; ++i) groups += (plan->segs[i].meta >> kSegDimsShift) == kSegGroup ? 1 : 0;
+  size_t members = 0;
+  for (size_t g = 0; g < groups; ++g) {
+    GroupHead head;
+    std::memcpy(&head, plan->group_blocks.data() + g * kGroupBlockBytes, sizeof(head));
+    members += head.members;
+  }
+  *count = nseg - groups + members + plan->host_copies.size();
   size_t w = 0;
   for (size_t i = 0; i < nseg && out && w < capacity; ++i, ++w) {
     const Seg& s = plan->segs[i];
+    if ((s.meta >> kSegDimsShift) == kSegGroup) {
+      // one entry per member; the group's single tile is counted with its first member
+      const size_t block = (s.ptr - plan->members_at) / kGroupBlockBytes, n = s.run_bytes & 0xffu;
+      for (size_t k = 0; k < n && w < capacity; ++k, ++w) {
+        Member m;
+        std::memcpy(&m, plan->group_blocks.data() + block * kGroupBlockBytes + sizeof(GroupHead) + k * sizeof(Member),
+                    sizeof(m));
+        axr_segment_info_t& o = out[w];
+        std::memset(&o, 0, sizeof(o));
+        o.tensor = plan->member_tensor[block * kGroupMaxMembers + k];
+        o.mode = 6;
+        o.address = m.ptr;
+        o.offset = s.off + (m.off_pad & ((1u << kMemberOffBits) - 1u));
+        o.run_bytes = o.nbytes = m.nbytes;
+        o.pad = m.off_pad >> kMemberOffBits;
+        o.tiles = k == 0 ? 1u : 0u;
+        o.granule = m.begin;
+        o.lanes_per_run = group_data_slots(m.nbytes) + group_pad_slots(o.pad);
+      }
+      --w;   // the loop header steps once more
+      continue;
+    }
     axr_segment_info_t& o = out[w];
     std::memset(&o, 0, sizeof(o));
     o.tensor = plan->seg_tensor[i];

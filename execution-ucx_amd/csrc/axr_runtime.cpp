@@ -480,6 +480,13 @@ static int tune_set_body(const char* key, int64_t value) {
     t.inline_tables = value;
   } else if (k == "transpose") {
     t.transpose = value ? 1 : 0;
+  } else if (k == "group_bytes") {
+    if (value < 0 || value > static_cast<int64_t>(kGroupMaxMemberBytes))
+      return fail(AXR_ERR_INVALID, "group_bytes must be in [0, 1023]");
+    t.group_bytes = value;
+  } else if (k == "group_slots") {
+    if (value != 64 && value != 128) return fail(AXR_ERR_INVALID, "group_slots must be 64 or 128");
+    t.group_slots = value;
   } else if (k == "device_tables") {
     if (value < 0) return fail(AXR_ERR_INVALID, "device_tables must not be negative");
     t.device_tables = value;
@@ -518,6 +525,8 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "head_align") *value = t.head_align;
   else if (k == "loopback_copy_kernel") *value = t.loopback_copy_kernel;
   else if (k == "device_tables") *value = t.device_tables;
+  else if (k == "group_bytes") *value = t.group_bytes;
+  else if (k == "group_slots") *value = t.group_slots;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;
 }

@@ -386,7 +386,11 @@ typedef struct axr_segment_info {
                              elements, 3 zero fill only, 4 host copy,
                              5 transposed blocks (all dims in packed order;
                              the one whose stride equals `granule` is
-                             contiguous in the tensor)                        */
+                             contiguous in the tensor), 6 a short tensor that
+                             shares one wavefront's tile with its neighbours
+                             (`granule` = its first lane slot in the tile,
+                             `lanes_per_run` = the slots it occupies, `tiles`
+                             = 1 for the first tensor of a tile, else 0)      */
   uint64_t address;       /* tensor-side address of the first element         */
   uint64_t offset;        /* payload offset                                   */
   uint64_t run_bytes;     /* contiguous bytes per run                         */
@@ -444,6 +448,10 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * 0: never),
  * "loopback_copy_kernel" (1, default: the loopback context moves a device payload
  * to device memory with the library's copy kernel; 0: with hipMemcpyAsync),
+ * "group_bytes" (contiguous device tensors of at most this many bytes that follow each
+ * other in the bundle share wavefronts: up to 64 tensors or 128 sixteen-byte lane slots
+ * per wavefront, so that wavefronts and table bytes scale with the payload and not with
+ * the tensor count; default 512, at most 1023, 0: every tensor gets wavefronts of its own),
  * "inline_tables" (the first launch of a bundle of at most this many tiles
  * whose tables fit into 3.5 KiB carries the tables inside the kernel arguments:
  * no table block and no upload; a plan that is launched again uploads its

@@ -368,7 +368,7 @@ def test_small_bundles_carry_their_tables_in_the_kernel_arguments(pkg):
         try:
             return pkg.BundlePlan.create(views, align=256).launch_info()
         finally:
-            pkg.tune(tile_rows=0, inline_tables=16384, nontemporal=-1)
+            pkg.tune(tile_rows=0, inline_tables=16384, nontemporal=-1, group_bytes=512)
     few = [tv(pkg, 0x10000 * (i + 1), [5000]) for i in range(4)]
     i = info(few)
     assert i["inline_tables"] == 1 and i["table_bytes"] + 16 <= 3584
@@ -378,8 +378,11 @@ def test_small_bundles_carry_their_tables_in_the_kernel_arguments(pkg):
     assert info([tv(pkg, 0x10000, [3 * 2048])], inline_tables=2)["inline_tables"] == 0   # 3 tiles > 2
     assert info([tv(pkg, 0x10000, [3 * 2048])], inline_tables=3)["inline_tables"] == 1
     many = [tv(pkg, 0x1000 * (i + 1), [100]) for i in range(120)]  # 121 x 32 B of segments alone
-    assert info(many)["inline_tables"] == 0
-    assert info(many[:90])["inline_tables"] == 1
+    assert info(many, group_bytes=0)["inline_tables"] == 0
+    assert info(many[:90], group_bytes=0)["inline_tables"] == 1
+    grouped = info(many)                                           # short tensors share tiles
+    assert grouped["tiles"] <= 20 and grouped["inline_tables"] == 0     # 18 blocks of 288 B
+    assert info(many[:60])["inline_tables"] == 1
     big = [tv(pkg, 0x10000000, [64 << 20])]                        # 32768 tiles
     assert info(big)["inline_tables"] == 0
     strided = [tv(pkg, 0x10000, [64, 64], strides=[1, 64], dtype=(2, 32, 1)),
@@ -398,7 +401,9 @@ def test_pads_fill_segments_and_host_copies(pkg):
     segs = plan.segments()
     dev = [s for s in segs if s["mode"] != 4]
     host = [s for s in segs if s["mode"] == 4]
-    assert [(s["tensor"], s["mode"], s["pad"]) for s in dev] == [(0, 0, 156), (2, 0, 0), (3, 3, 226), (4, 0, 0)]
+    # the two short device tensors share one group tile; the last one has no neighbour
+    assert [(s["tensor"], s["mode"], s["pad"]) for s in dev] == [(0, 6, 156), (2, 6, 0), (3, 3, 226), (4, 0, 0)]
+    assert [s["tiles"] for s in dev] == [1, 0, 1, 1]
     assert dev[2]["offset"] == 512 + 30
     assert [(s["address"], s["offset"], s["nbytes"]) for s in host] == [
         (0x40000, 512, 10), (0x40000 + 20, 522, 10), (0x40000 + 40, 532, 10)]

@@ -20,7 +20,7 @@ def interpret(segments, memory, payload_bytes):
     out = np.full(payload_bytes, 0xEE, np.uint8)
     for s in segments:
         off, run = s["offset"], s["run_bytes"]
-        if s["mode"] in (0, 4):
+        if s["mode"] in (0, 4, 6):
             a = s["address"] - BASE
             out[off:off + run] = memory[a:a + run]
             end = off + run
@@ -117,3 +117,111 @@ def test_host_pieces_and_fill_segments(pkg, orc):
     got = interpret(segs, memory, plan.payload_bytes)
     want = orc.pack([np.ascontiguousarray(host).reshape(-1), memory[0x4000:0x4000 + 1000]], 256)
     assert np.array_equal(got, want)
+
+
+def move_group_slots(members, memory, out):
+    """One group tile moved slot by slot, the way a wavefront does it: slot s belongs to the
+    last member whose first slot is <= s; a member of n >= 16 bytes moves 16 bytes per data
+    slot, the last one covering its final 16 bytes; shorter members and gaps under 16 bytes move
+    in pieces of 8, 4, 2 and 1 bytes; gaps of 16 bytes or more are zero slots."""
+    begins = [m["granule"] for m in members]
+    total = members[-1]["granule"] + members[-1]["lanes_per_run"]
+    assert begins[0] == 0 and total <= 128 and len(members) <= 64
+    for a, b in zip(members, members[1:]):
+        assert b["granule"] == a["granule"] + a["lanes_per_run"]
+    for s in range(total):
+        m = max(i for i, b in enumerate(begins) if b <= s)
+        mem = members[m]
+        n, pad, k = mem["nbytes"], mem["pad"], s - mem["granule"]
+        dslots = (n + 15) // 16 if n >= 16 else 1
+        pslots = (pad + 15) // 16 if pad >= 16 else 0
+        assert mem["lanes_per_run"] == dslots + pslots
+        src, dst = mem["address"] - BASE, mem["offset"]
+        if k < dslots:
+            if n >= 16:
+                o = n - 16 if k + 1 == dslots else 16 * k
+                out[dst + o:dst + o + 16] = memory[src + o:src + o + 16]
+            else:
+                for piece, at in ((8, 0), (4, n & 8), (2, n & 12), (1, n & 14)):
+                    if n & piece:
+                        out[dst + at:dst + at + piece] = memory[src + at:src + at + piece]
+            if k + 1 == dslots and 0 < pad < 16:
+                for piece, at in ((8, 0), (4, pad & 8), (2, pad & 12), (1, pad & 14)):
+                    if pad & piece:
+                        out[dst + n + at:dst + n + at + piece] = 0
+        else:
+            j = k - dslots
+            o = n + (pad - 16 if j + 1 == pslots else 16 * j)
+            out[dst + o:dst + o + 16] = 0
+
+
+@pytest.mark.parametrize("align", [1, 2, 16, 256, 4096])
+def test_short_tensors_share_group_tiles(pkg, orc, align):
+    """Bundles of many short tensors: the planner packs consecutive ones into group tiles
+    (mode 6).  The records moved slot by slot must give the oracle's payload, the tile count
+    must follow the payload rather than the tensor count, and long tensors in between keep
+    their own segments."""
+    rng = np.random.default_rng(100 + align)
+    memory = rng.integers(0, 256, size=1 << 22, dtype=np.uint8)
+    views, chunks, at = [], [], 64
+    for i in range(1500):
+        np_dt, dl_dt = DTYPES[i % 3]
+        item = np.dtype(np_dt).itemsize
+        if i % 97 == 50:
+            nbytes = int(rng.integers(600, 5000)) // item * item       # a long tensor between the short ones
+        elif i % 41 == 7:
+            nbytes = 0
+        else:
+            nbytes = max(item, int(np.exp(rng.uniform(np.log(1), np.log(512)))) // item * item)
+        at += int(rng.integers(0, 5)) * item
+        views.append(pkg.TensorView(data=BASE + at, device_type=10, device_id=0, dtype=dl_dt,
+                                    shape=(nbytes // item,), strides=None))
+        chunks.append(memory[at:at + nbytes])
+        at += nbytes
+    plan = pkg.BundlePlan.create(views, align=align)
+    segs = plan.segments()
+    if align == 4096:
+        # gaps of up to 4095 zero bytes per tensor would be most of a tile: no groups
+        assert {s["mode"] for s in segs} == {0}
+        assert np.array_equal(interpret(segs, memory, plan.payload_bytes), orc.pack(chunks, align))
+        return
+    assert {s["mode"] for s in segs} == {0, 6}
+    # the records as plain copies
+    assert np.array_equal(interpret(segs, memory, plan.payload_bytes), orc.pack(chunks, align))
+    # and the group tiles slot by slot
+    out = np.full(plan.payload_bytes, 0xEE, np.uint8)
+    group, tiles = [], 0
+    for s in segs + [None]:
+        if s is not None and s["mode"] == 6 and not (s["tiles"] == 1 and group):
+            group.append(s)
+            tiles += s["tiles"]
+            continue
+        if group:
+            assert len(group) >= 2
+            move_group_slots(group, memory, out)
+            group = []
+        if s is None:
+            break
+        if s["mode"] == 6:
+            group.append(s)
+            tiles += 1
+        else:
+            a = s["address"] - BASE
+            out[s["offset"]:s["offset"] + s["run_bytes"]] = memory[a:a + s["run_bytes"]]
+            out[s["offset"] + s["run_bytes"]:s["offset"] + s["run_bytes"] + s["pad"]] = 0
+            tiles += s["tiles"]
+    assert np.array_equal(out, orc.pack(chunks, align))
+    info = plan.launch_info()
+    assert tiles == info["tiles"]
+    short = sum(1 for s in segs if s["mode"] == 6)
+    assert short > 1300
+    if align <= 16:
+        assert info["tiles"] < 1500 // 4       # far fewer wavefronts than tensors
+    # switched off, every tensor gets a segment of its own
+    pkg.tune(group_bytes=0)
+    try:
+        plain = pkg.BundlePlan.create(views, align=align)
+        assert {s["mode"] for s in plain.segments()} == {0}
+        assert plain.launch_info()["tiles"] >= 1400
+    finally:
+        pkg.tune(group_bytes=512)
