@@ -28,7 +28,6 @@ AXR_ERR_MISMATCH = -9
 AXR_ERR_NO_DEVICE = -10
 AXR_ERR_BUSY = -11
 AXR_ERR_CANCELED = -12
-AXR_ERR_CANCELED = -12
 
 # ucx_memory_type_t numbering (ucx_context/ucx_context_def.h:27-39)
 MEM_HOST = 0
@@ -277,6 +276,7 @@ PROTOTYPES = {
     "axr_am_recv_buffer_async": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
     "axr_am_recv_buffer_iov": (C.c_int, [_vp, C.c_uint64, C.c_int, C.POINTER(Buffer), _sz, _vp]),
     "axr_am_message_release": (C.c_int, [_vp, C.c_uint64]),
+    "axr_am_message_info": (C.c_int, [_vp, C.c_uint64, _u64p, _u64p, _intp]),
     "axr_am_pending": (C.c_int, [_vp, C.POINTER(_sz)]),
     "axr_transfer_create": (C.c_int, [_vp, _sz, C.c_int, C.c_int, _vpp]),
     "axr_transfer_submit": (C.c_int, [_vp, _vp, C.c_int64, _vp, C.c_int64]),

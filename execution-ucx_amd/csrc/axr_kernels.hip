@@ -128,8 +128,19 @@ __device__ __forceinline__ void wave_copy(gcbytes src, gbytes dst, uint64_t left
   }
 }
 
+// Zero bytes of an alignment gap: 16-byte stores, the last one covering the gap's final 16
+// bytes (one store instruction for a gap of up to 1 KiB); gaps under 16 bytes bytewise.
 __device__ __forceinline__ void wave_zero(gbytes dst, uint32_t n, uint32_t lane) {
-  for (uint32_t i = lane; i < n; i += kWaveLanes) dst[i] = 0;
+  if (n < kVecBytes) {
+    if (lane < n) dst[lane] = 0;
+    return;
+  }
+  const uint32_t slots = (n + kVecBytes - 1) / kVecBytes;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (uint32_t j = lane; j < slots; j += kWaveLanes) {
+    const uint32_t o = j * kVecBytes;
+    store16<false>(dst + (o + kVecBytes <= n ? o : n - kVecBytes), zero);
+  }
 }
 
 typedef const AXR_CONST Seg* seg_table;

@@ -519,6 +519,21 @@ int axr_am_message_release(axr_am_context_t* ctx, uint64_t key) {
   return guarded([&] { return am_message_release_body(ctx, key); });
 }
 
+static int am_message_info_body(axr_am_context_t* ctx, uint64_t key, uint64_t* data_length, uint64_t* conn_id,
+                                int* is_rndv) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_message_info: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto it = ctx->parked.find(key);
+  if (it == ctx->parked.end()) return fail(AXR_ERR_NO_MESSAGE, "no message with this key");
+  if (data_length) *data_length = it->second->data_length;
+  if (conn_id) *conn_id = it->second->conn_id;
+  if (is_rndv) *is_rndv = it->second->rndv ? 1 : 0;
+  return AXR_OK;
+}
+int axr_am_message_info(axr_am_context_t* ctx, uint64_t key, uint64_t* data_length, uint64_t* conn_id, int* is_rndv) {
+  return guarded([&] { return am_message_info_body(ctx, key, data_length, conn_id, is_rndv); });
+}
+
 static int am_pending_body(axr_am_context_t* ctx, size_t* count) {
   if (!ctx || !count) return fail(AXR_ERR_INVALID, "axr_am_pending: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);

@@ -559,6 +559,13 @@ AXR_API int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_
 /* Drop a message's host copies (and, for an unfetched rendezvous, complete the
  * sender's request as cancelled). */
 AXR_API int axr_am_message_release(axr_am_context_t* ctx, uint64_t key);
+/* What axr_am_recv_header said about a message that is still parked (a rendezvous whose
+ * payload has not been fetched, an eager message not yet released): its payload length,
+ * the reply connection and whether it is a rendezvous.  Any result may be NULL.  Unknown
+ * key -> AXR_ERR_NO_MESSAGE.  The receive-buffer operation of the reference learns the
+ * length the same way, from the parked descriptor (ucx_am_context.hpp:1568-1621). */
+AXR_API int axr_am_message_info(axr_am_context_t* ctx, uint64_t key, uint64_t* data_length,
+                                uint64_t* conn_id, int* is_rndv);
 /* Messages queued and not yet taken by axr_am_recv_header. */
 AXR_API int axr_am_pending(axr_am_context_t* ctx, size_t* count);
 

@@ -53,6 +53,24 @@ def test_receive_adapters_against_the_reference_classes(gpu):
     assert "adapters_selftest ok" in out.stdout
 
 
+@pytest.mark.gpu
+def test_am_bundle_surface_against_the_reference_classes(gpu):
+    """oracle/_ref/am_surface_selftest (tests/cpp/am_surface_selftest.cpp): connection_send /
+    connection_recv / connection_recv_header / connection_recv_buffer of
+    host/loopback_am_context.hpp with the reference's real UcxBuffer, UcxHeader, UcxAmData,
+    UcxAmIovec and UcxBufferVec.  The host bundle of 64 fp32 tensors and a device bundle go
+    PackTensors -> connection_send -> connection_recv_header -> ReceiveBufferFor ->
+    connection_recv_buffer -> UnpackTensors with the payload compared against the oracle's
+    pack; then the reference's edge rules, its iov and divide-by-two known answers, and
+    cancellation."""
+    exe = os.path.join(ROOT, "oracle", "_ref", "am_surface_selftest")
+    assert os.path.exists(exe), "oracle/_ref/am_surface_selftest is missing: run __graft_entry__.build() " \
+                                "where the reference tree is mounted"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=180)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "am_surface_selftest ok" in out.stdout
+
+
 def test_planner_and_header_codec_under_sanitizers(tmp_path):
     """tests/cpp/plan_fuzz.cpp against a planner compiled with AddressSanitizer and
     UBSan (host code only; the kernels' object file is linked as built): random tensor

@@ -113,9 +113,9 @@ def test_small_bundle_and_limits(pkg, orc, gpu):
     assert lib.axr_pack_noalloc(plan._h, buf.data_ptr(), n - 1, None) == capi.AXR_ERR_LENGTH
     plan.close()
     # tables beyond the static area: refused with a clear error, nothing launched
-    arena = torch.zeros(40000 * 16, dtype=torch.uint8, device=gpu)
+    arena = torch.zeros(100000 * 16, dtype=torch.uint8, device=gpu)
     views = [pkg.TensorView(data=arena.data_ptr() + 16 * i, device_type=10, device_id=0, dtype=(1, 8, 1),
-                            shape=(16,), strides=None) for i in range(40000)]
+                            shape=(16,), strides=None) for i in range(100000)]
     plan = pkg.BundlePlan.create(views, align=1)
     assert plan.launch_info()["table_bytes"] > (1 << 20)
     out = torch.full((plan.payload_bytes,), POISON, dtype=torch.uint8, device=gpu)
