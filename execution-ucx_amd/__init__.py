@@ -5,7 +5,7 @@ header and scatters a received buffer back, with hand-written HIP kernels for
 gfx950 behind a C ABI (``include/axon_rocm.h``).  The HIP library is required:
 nothing here computes on the CPU.
 """
-from . import _capi
+from . import _capi, streams
 from ._capi import (AxonRocmError, HeaderError, LengthError, MismatchError, NoDeviceError,
                     NoMessageError, NotImplementedForEager, UnsupportedMemoryError)
 from .bundle import (BundlePlan, DLDataType, DLDevice, PackedBundle, TensorMeta, bundle_to_host, pack_bundle,

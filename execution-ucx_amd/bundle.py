@@ -16,7 +16,7 @@ import ctypes as C
 from dataclasses import dataclass
 from typing import Any, Callable, List, NamedTuple, Optional, Sequence, Tuple
 
-from . import _capi
+from . import _capi, streams
 from .dlpack import DLPackExport, TensorArray, TensorView
 from .memory import DevicePool, PoolBuffer
 
@@ -57,6 +57,11 @@ class TensorMeta:
     nbytes: int = 0
 
 
+def _dlpack_stream(stream) -> Optional[int]:
+    """``stream`` as the DLPack protocol spells it, or None when the caller named none."""
+    return None if stream is None else streams.dlpack_stream_argument(_stream_handle(stream))
+
+
 def _stream_handle(stream) -> Optional[int]:
     if stream is None:
         return None
@@ -78,12 +83,15 @@ class BundlePlan:
 
     # ---- construction
     @classmethod
-    def create(cls, tensors: Sequence[Any], align: int = 1) -> "BundlePlan":
+    def create(cls, tensors: Sequence[Any], align: int = 1, stream=None) -> "BundlePlan":
         """Sender side: ``tensors`` are DLPack producers (or TensorViews), laid
-        out in argument order.  ``align=1`` is the reference's tight layout."""
+        out in argument order.  ``align=1`` is the reference's tight layout.
+        ``stream``: the stream the plan will be packed on, when it is known already; producers
+        other than torch tensors are then told through ``__dlpack__(stream=...)``."""
         lib = _capi.load()
         # descriptors may be prepared once and reused per call
-        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
+        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(
+            tensors, stream=_dlpack_stream(stream))
         h = C.c_void_p()
         _capi.check(lib.axr_plan_create(arr.pointer(), arr.count, align, 0, C.byref(h)))
         return cls(h.value, keepalive=arr)     # the array holds the producers' capsules
@@ -106,8 +114,9 @@ class BundlePlan:
         _capi.check(lib.axr_plan_from_header_bind(buf, len(buf), arr.pointer(), arr.count, C.byref(h)))
         return cls(h.value, keepalive=arr)
 
-    def bind(self, tensors: Sequence[Any]) -> "BundlePlan":
-        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
+    def bind(self, tensors: Sequence[Any], stream=None) -> "BundlePlan":
+        arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(
+            tensors, stream=_dlpack_stream(stream))
         _capi.check(self._lib.axr_plan_bind(self._h, arr.pointer(), arr.count))
         self._keep = arr
         return self
@@ -183,11 +192,24 @@ class BundlePlan:
         _capi.check(self._lib.axr_plan_prepare(self._h, _stream_handle(stream)))
         return self
 
-    def pack(self, payload: int, payload_bytes: int, stream=None) -> None:
-        _capi.check(self._lib.axr_pack(self._h, payload, payload_bytes, _stream_handle(stream)))
+    def pack(self, payload: int, payload_bytes: int, stream=None, order: bool = True) -> None:
+        """Gather on ``stream``.  ``order``: when ``stream`` is not the stream the tensor
+        framework is enqueueing on, the kernel is ordered behind what that stream holds now
+        (the tensors' producers), with an event and no host wait."""
+        handle = _stream_handle(stream)
+        if order:
+            streams.order_behind_producers(handle)
+        _capi.check(self._lib.axr_pack(self._h, payload, payload_bytes, handle))
 
-    def unpack(self, payload: int, payload_bytes: int, stream=None) -> None:
-        _capi.check(self._lib.axr_unpack(self._h, payload, payload_bytes, _stream_handle(stream)))
+    def unpack(self, payload: int, payload_bytes: int, stream=None, order: bool = True) -> None:
+        """Scatter on ``stream``, ordered behind the framework's stream like ``pack`` (the
+        destinations may still be written there).  What the framework enqueues afterwards
+        sees the data once ``streams.make_visible_to_producers(stream)`` has been called
+        (``unpack_bundle`` does) or the stream has been synchronised."""
+        handle = _stream_handle(stream)
+        if order:
+            streams.order_behind_producers(handle)
+        _capi.check(self._lib.axr_unpack(self._h, payload, payload_bytes, handle))
 
     def split(self, payload: int, payload_bytes: int) -> List[Tuple[int, int]]:
         n = self.num_tensors
@@ -253,8 +275,10 @@ class PackedBundle:
 
 def pack_bundle(tensors: Sequence[Any], align: int = 256, pool: Optional[DevicePool] = None,
                 stream=None) -> PackedBundle:
-    """Gather ``tensors`` into one pool buffer on ``stream`` (asynchronous)."""
-    plan = BundlePlan.create(tensors, align=align)
+    """Gather ``tensors`` into one pool buffer on ``stream`` (asynchronous).  The kernel is
+    ordered behind the stream that produced the tensors; no synchronisation is needed between
+    producing them and this call."""
+    plan = BundlePlan.create(tensors, align=align, stream=stream)
     pool = pool or DevicePool.default()
     nbytes = plan.payload_bytes
     buf = pool.alloc(max(nbytes, 1), 256)
@@ -273,6 +297,10 @@ def unpack_bundle(header: bytes, payload: Any, payload_bytes: Optional[int] = No
     header's offsets and each piece is returned as a DLPack producer over the
     payload memory (``from_dlpack_fn`` converts them, e.g. ``torch.from_dlpack``),
     typed and shaped from the header.
+
+    The scatter is ordered behind the tensor framework's stream (the destinations may still
+    be written there), and that stream is made to wait for the scatter, so the framework's
+    next kernels see the data without a host synchronisation.
     """
     if isinstance(payload, PoolBuffer):
         ptr, size = payload.data, payload.size
@@ -282,8 +310,9 @@ def unpack_bundle(header: bytes, payload: Any, payload_bytes: Optional[int] = No
         size = payload_bytes
     plan = BundlePlan.from_header(header)
     if out is not None:
-        plan.bind(out)
+        plan.bind(out, stream=stream)
         plan.unpack(ptr, size, stream)
+        streams.make_visible_to_producers(_stream_handle(stream))
         return plan
     pieces = plan.split(ptr, size)
     metas = plan.metas()

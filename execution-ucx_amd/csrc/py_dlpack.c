@@ -5,7 +5,7 @@
  * else.  The result is a ready array of axr_tensor_t (layout-identical to
  * DLTensor) for axr_plan_create / axr_plan_bind.
  *
- * describe(sequence[, fast_type, fast_export, device_id])
+ * describe(sequence[, fast_type, fast_export, device_id, stream])
  *     -> (descs: bytearray, dims: bytearray, owners: list)
  *   descs   n * sizeof(axr_tensor_t); shape/strides point into `dims`
  *   dims    the copied shapes and strides (int64)
@@ -13,6 +13,12 @@
  *           producers' deleters
  * Every element must provide `__dlpack__()` or be a capsule named "dltensor"
  * or "dltensor_versioned"; describe() returns None when it meets anything else.
+ * With `stream` (an int, the DLPack protocol's value for the stream the consumer
+ * will read on), producers that are not `fast_type` tensors are asked with
+ * `__dlpack__(stream=stream)`, their half of the protocol's stream handshake; a
+ * producer that refuses the argument (host memory, an older protocol) is asked
+ * again without it.  `fast_type` tensors are ordered by the caller, once per
+ * bundle.
  *
  * Objects whose type is exactly `fast_type` are exported with
  * `fast_export(obj)` instead, when `obj.requires_grad` is False, `obj.is_conj()` is
@@ -51,6 +57,24 @@ static const axr_tensor_t* tensor_of_capsule(PyObject* capsule) {
 static PyObject* str_requires_grad;
 static PyObject* str_is_conj;
 static PyObject* str_dlpack;
+static PyObject* str_stream;
+
+/* method(stream=stream), or method() when the producer does not take the argument. */
+static PyObject* call_dlpack(PyObject* method, PyObject* stream) {
+  if (stream && stream != Py_None) {
+    PyObject* empty = PyTuple_New(0);
+    PyObject* kwargs = PyDict_New();
+    PyObject* capsule = NULL;
+    if (empty && kwargs && PyDict_SetItem(kwargs, str_stream, stream) == 0)
+      capsule = PyObject_Call(method, empty, kwargs);
+    Py_XDECREF(empty);
+    Py_XDECREF(kwargs);
+    if (capsule) return capsule;
+    if (PyErr_ExceptionMatches(PyExc_MemoryError) || PyErr_ExceptionMatches(PyExc_KeyboardInterrupt)) return NULL;
+    PyErr_Clear();
+  }
+  return PyObject_CallNoArgs(method);
+}
 
 /* 1 when obj.requires_grad is False (Tensor.__dlpack__ refuses tensors that require grad). */
 static int no_grad(PyObject* obj) {
@@ -105,7 +129,8 @@ static PyObject* describe(PyObject* self, PyObject* args) {
   PyObject* fast_type = Py_None;
   PyObject* fast_export = Py_None;
   long device_id = -1;
-  if (!PyArg_ParseTuple(args, "O|OOl", &arg, &fast_type, &fast_export, &device_id)) return NULL;
+  PyObject* stream = Py_None;
+  if (!PyArg_ParseTuple(args, "O|OOlO", &arg, &fast_type, &fast_export, &device_id, &stream)) return NULL;
   if (fast_type == Py_None || fast_export == Py_None) fast_type = NULL;
   PyObject* seq = PySequence_Fast(arg, "describe() needs a sequence of DLPack producers");
   if (!seq) return NULL;
@@ -136,7 +161,9 @@ static PyObject* describe(PyObject* self, PyObject* args) {
           Py_INCREF(result);
           goto done;
         }
-        capsule = PyObject_CallNoArgs(method);
+        /* tensors of the fast type that took this route are ordered by the caller as well */
+        const int framework_tensor = fast_type && PyObject_IsInstance(obj, fast_type) == 1;
+        capsule = call_dlpack(method, framework_tensor ? Py_None : stream);
         Py_DECREF(method);
       }
       if (!capsule) goto done;
@@ -191,7 +218,7 @@ done:
 
 static PyMethodDef methods[] = {
     {"describe", describe, METH_VARARGS,
-     "describe(sequence[, fast_type, fast_export, device_id]) -> "
+     "describe(sequence[, fast_type, fast_export, device_id, stream]) -> "
      "(descs bytearray, dims bytearray, owners list)"},
     {NULL, NULL, 0, NULL}};
 
@@ -203,7 +230,8 @@ PyMODINIT_FUNC PyInit__axr_dlpack(void) {
   str_requires_grad = PyUnicode_InternFromString("requires_grad");
   str_is_conj = PyUnicode_InternFromString("is_conj");
   str_dlpack = PyUnicode_InternFromString("__dlpack__");
-  if (!str_requires_grad || !str_is_conj || !str_dlpack) return NULL;
+  str_stream = PyUnicode_InternFromString("stream");
+  if (!str_requires_grad || !str_is_conj || !str_dlpack || !str_stream) return NULL;
   PyObject* m = PyModule_Create(&module);
   if (m) PyModule_AddIntConstant(m, "TENSOR_BYTES", (long)sizeof(axr_tensor_t));
   return m;

@@ -128,13 +128,32 @@ class NotDLPackError(TypeError, RuntimeError):
     this is both."""
 
 
-def extract(obj: Any) -> TensorView:
-    """Describe ``obj`` (anything with ``__dlpack__``, or a capsule)."""
+def _is_framework_tensor(obj: Any) -> bool:
+    import sys
+    torch = sys.modules.get("torch")
+    return torch is not None and isinstance(obj, torch.Tensor)
+
+
+def extract(obj: Any, stream: Optional[int] = None) -> TensorView:
+    """Describe ``obj`` (anything with ``__dlpack__``, or a capsule).  ``stream`` is the DLPack
+    protocol's value for the stream the consumer will read on (``streams.dlpack_stream_argument``):
+    a producer other than a torch tensor is asked with ``__dlpack__(stream=stream)`` so that it
+    orders its work before that stream (torch tensors are ordered once per bundle by
+    ``streams.order_behind_producers``); one that refuses the argument is asked without it."""
     if isinstance(obj, TensorView):
         return obj
     capsule = obj
     if hasattr(obj, "__dlpack__"):
-        capsule = obj.__dlpack__()
+        capsule = None
+        if stream is not None and not _is_framework_tensor(obj):
+            try:
+                capsule = obj.__dlpack__(stream=stream)
+            except (MemoryError, KeyboardInterrupt):
+                raise
+            except Exception:  # noqa: BLE001 - host producers and older protocols refuse the argument
+                capsule = None
+        if capsule is None:
+            capsule = obj.__dlpack__()
     if _py.PyCapsule_IsValid(capsule, _NAME):
         ptr = _py.PyCapsule_GetPointer(capsule, _NAME)
         managed = C.cast(ptr, C.POINTER(_ManagedTensor)).contents
@@ -150,8 +169,8 @@ def extract(obj: Any) -> TensorView:
     )
 
 
-def extract_many(objs: Sequence[Any]) -> List[TensorView]:
-    return [extract(o) for o in objs]
+def extract_many(objs: Sequence[Any], stream: Optional[int] = None) -> List[TensorView]:
+    return [extract(o, stream) for o in objs]
 
 
 class TensorArray:
@@ -189,8 +208,10 @@ class TensorArray:
         return C.cast(self.array, C.POINTER(_capi.Tensor))
 
     @classmethod
-    def from_objects(cls, objs: Sequence[Any]) -> "TensorArray":
-        """Descriptors of DLPack producers (or ``TensorView``s)."""
+    def from_objects(cls, objs: Sequence[Any], stream: Optional[int] = None) -> "TensorArray":
+        """Descriptors of DLPack producers (or ``TensorView``s).  ``stream``: the DLPack protocol's
+        value for the stream the bundle's kernels will run on, handed to producers other than
+        torch tensors (see ``extract``)."""
         native = _native()
         exporter = _torch_exporter()
         described = None
@@ -199,9 +220,12 @@ class TensorArray:
             if direct is not None:
                 described = direct.describe(objs, exporter[2])
         if described is None and native is not None:
-            described = native.describe(objs, *exporter)
+            if stream is None:
+                described = native.describe(objs, *exporter)
+            else:
+                described = native.describe(objs, *(exporter or (None, None, -1)), stream)
         if described is None:   # no helper, or something that is not a DLPack producer
-            return cls(extract_many(objs))
+            return cls(extract_many(objs, stream))
         descs, dims, owners = described
         self = cls.__new__(cls)
         n = len(owners)

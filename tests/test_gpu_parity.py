@@ -33,8 +33,9 @@ def run_pack(pkg, tensors, align, gpu, base_shift=0):
     plan = pkg.BundlePlan.create(tensors, align=align)
     n = plan.payload_bytes
     buf = device_bytes(n + base_shift + 64, gpu)
+    # on the stream that produced the tensors: ordered by the stream itself, and the copy to
+    # the host below waits for it
     plan.pack(buf.data_ptr() + base_shift, n, torch.cuda.current_stream().cuda_stream)
-    torch.cuda.synchronize()
     host = buf.cpu().numpy()
     # nothing outside [shift, shift + n) may be written
     assert (host[:base_shift] == POISON).all() and (host[base_shift + n:] == POISON).all()

@@ -52,7 +52,6 @@ def test_two_calls_in_a_row_match_axr_pack(pkg, orc, gpu, align):
     small = make_bundle(gpu, rng, 300, strided_every=5)
     stream = C.c_void_p()
     capi.check(lib.axr_stream_create(C.byref(stream)))
-    torch.cuda.synchronize()          # the inputs were produced on torch's stream
     plans, bufs = [], []
     try:
         for tensors in (big, small):
@@ -64,8 +63,9 @@ def test_two_calls_in_a_row_match_axr_pack(pkg, orc, gpu, align):
             buf = torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu)
             plans.append(plan)
             bufs.append(buf)
-        torch.cuda.synchronize()
-        # two calls back to back, no wait in between
+        # the inputs and the poisoned buffers were produced on torch's stream: the launch stream
+        # is ordered behind it with an event (no host wait), then two calls back to back
+        assert pkg.streams.order_behind_producers(stream.value)
         for plan, buf in zip(plans, bufs):
             capi.check(lib.axr_pack_noalloc(plan._h, buf.data_ptr(), plan.payload_bytes, stream))
         capi.check(lib.axr_stream_synchronize(stream))
