@@ -275,11 +275,14 @@ PROTOTYPES = {
     "axr_am_recv_buffer": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
     "axr_am_recv_buffer_async": (C.c_int, [_vp, C.c_uint64, C.c_int, _vp, _sz, _vp]),
     "axr_am_recv_buffer_iov": (C.c_int, [_vp, C.c_uint64, C.c_int, C.POINTER(Buffer), _sz, _vp]),
+    "axr_am_recv_buffer_borrow": (C.c_int, [_vp, C.c_uint64, _vpp, C.POINTER(_sz), _intp]),
+    "axr_am_borrow_release": (C.c_int, [_vp, C.c_uint64, _vp]),
     "axr_am_message_release": (C.c_int, [_vp, C.c_uint64]),
     "axr_am_message_info": (C.c_int, [_vp, C.c_uint64, _u64p, _u64p, _intp]),
     "axr_am_pending": (C.c_int, [_vp, C.POINTER(_sz)]),
     "axr_transfer_create": (C.c_int, [_vp, _sz, C.c_int, C.c_int, _vpp]),
     "axr_transfer_submit": (C.c_int, [_vp, _vp, C.c_int64, _vp, C.c_int64]),
+    "axr_transfer_set_zero_copy": (C.c_int, [_vp, C.c_int]),
     "axr_transfer_finish": (C.c_int, [_vp]),
     "axr_transfer_destroy": (C.c_int, [_vp]),
     "axr_divide_by_two": (C.c_int, [_vp, _sz, _vp]),

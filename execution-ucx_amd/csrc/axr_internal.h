@@ -242,6 +242,10 @@ struct Tunables {
   // tensor gets its own wavefronts.
   std::atomic<int64_t> group_bytes{512};
   std::atomic<int64_t> group_slots{kGroupMaxSlots};   // lane slots per group tile: 64 or 128
+  // Failure injection for tests of the streamed transfer's error handling: N > 0 makes the
+  // N-th chunk submitted from now on fail after its send has been queued, as if the message
+  // that arrived did not match the receiver's plan (and counts down to 0 = off).
+  std::atomic<int64_t> transfer_fail_after_send{0};
   std::atomic<int64_t> inline_tables{16384};  // bundles of up to this many tiles whose tables fit the kernel
                                   // arguments are launched without a table upload; 0: never
 };

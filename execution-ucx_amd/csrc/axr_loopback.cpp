@@ -83,6 +83,7 @@ struct axr_am_context {
   std::mutex mu;
   std::deque<std::unique_ptr<Message>> arrived;          // not yet seen by recv_header
   std::map<uint64_t, std::unique_ptr<Message>> parked;   // handed out, awaiting fetch/release
+  std::map<uint64_t, std::unique_ptr<Message>> borrowed; // payload lent to the receiver, awaiting release
   std::map<uint64_t, axr_am_context*> endpoints;         // conn id -> peer
   std::map<uint64_t, std::shared_ptr<Request>> requests;
   // Sends that have started and not completed (rendezvous sends whose payload has not been
@@ -228,6 +229,7 @@ static int am_context_destroy_body(axr_am_context_t* ctx) {
     std::lock_guard<std::mutex> lock(ctx->mu);
     for (auto& m : ctx->arrived) m->request->done.store(-1);
     for (auto& kv : ctx->parked) kv.second->request->done.store(-1);
+    for (auto& kv : ctx->borrowed) kv.second->request->done.store(1);   // the receiver is gone: nothing reads on
     for (auto& w : ctx->waiting) w.message->request->done.store(-1);
   }
   delete ctx;
@@ -473,6 +475,61 @@ int axr_am_recv_buffer_iov(axr_am_context_t* ctx,
                            void* stream) {
   return guarded([&] { return am_recv_buffer_iov_body(ctx, key, dst_type, buffer_vec, buffer_count,
                  stream); });
+}
+
+static int am_recv_buffer_borrow_body(axr_am_context_t* ctx, uint64_t key, void** data, size_t* bytes,
+                                      int* memory_type) {
+  if (!ctx || !data || !bytes) return fail(AXR_ERR_INVALID, "axr_am_recv_buffer_borrow: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto it = ctx->parked.find(key);
+  if (it == ctx->parked.end()) return fail(AXR_ERR_NO_MESSAGE, "no message with this key");
+  Message* m = it->second.get();
+  if (!m->rndv) return fail(AXR_ERR_NOT_IMPLEMENTED, "message was eager: its data came with the header");
+  if (m->pieces.size() != 1)
+    return fail(AXR_ERR_UNSUPPORTED, "only a contiguous payload can be borrowed: fetch an iov message with a copy");
+  {
+    Request* r = m->request.get();
+    std::lock_guard<std::mutex> rl(r->mu);
+    if (r->done.load() == -1) {
+      ctx->parked.erase(it);
+      return fail(AXR_ERR_CANCELED, "the sender cancelled this message");
+    }
+    r->claimed = true;
+  }
+  *data = const_cast<void*>(m->pieces[0].data);
+  *bytes = m->pieces[0].size;
+  if (memory_type) *memory_type = m->buffer_type;
+  ctx->borrowed[key] = std::move(it->second);
+  ctx->parked.erase(it);
+  return AXR_OK;
+}
+int axr_am_recv_buffer_borrow(axr_am_context_t* ctx, uint64_t key, void** data, size_t* bytes, int* memory_type) {
+  return guarded([&] { return am_recv_buffer_borrow_body(ctx, key, data, bytes, memory_type); });
+}
+
+static int am_borrow_release_body(axr_am_context_t* ctx, uint64_t key, void* stream) {
+  if (!ctx) return fail(AXR_ERR_INVALID, "axr_am_borrow_release: null context");
+  std::unique_ptr<Message> m;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto it = ctx->borrowed.find(key);
+    if (it == ctx->borrowed.end()) return fail(AXR_ERR_NO_MESSAGE, "no borrowed message with this key");
+    m = std::move(it->second);
+    ctx->borrowed.erase(it);
+  }
+  if (host_type(m->buffer_type)) {   // host readers have read by the time they say so
+    m->request->done.store(1);
+    return AXR_OK;
+  }
+  // completion of the send = completion of what the receiver's stream holds now
+  std::lock_guard<std::mutex> lock(m->request->mu);
+  int rc = check_hip(hipEventCreateWithFlags(&m->request->event, hipEventDisableTiming), "hipEventCreate");
+  if (rc == AXR_OK) rc = check_hip(hipEventRecord(m->request->event, static_cast<hipStream_t>(stream)), "hipEventRecord");
+  if (rc != AXR_OK) m->request->done.store(-1);
+  return rc;
+}
+int axr_am_borrow_release(axr_am_context_t* ctx, uint64_t key, void* stream) {
+  return guarded([&] { return am_borrow_release_body(ctx, key, stream); });
 }
 
 static int am_request_cancel_body(axr_am_context_t* ctx, uint64_t request) {

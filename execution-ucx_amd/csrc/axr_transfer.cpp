@@ -11,7 +11,8 @@
 // per chunk.
 //
 // The send goes through the same loopback context calls a caller would make
-// (axr_am_send / axr_am_recv_header / axr_am_recv_buffer_async), which stand for
+// (axr_am_send / axr_am_recv_header / axr_am_recv_buffer_borrow or axr_am_recv_buffer_async),
+// which stand for
 // connection_send (ucx_am_context.hpp:2234-2642) and connection_recv_buffer
 // (ucx_am_context.hpp:1511-1844) of the reference.
 #include <cstring>
@@ -39,6 +40,7 @@ struct axr_transfer {
   axr_am_context_t* server = nullptr;
   uint64_t conn = 0;
   uint64_t submitted = 0;
+  bool zero_copy = true;        // the receiver unpacks out of the sender's slot
   size_t streams = 1;           // lanes i and i + streams share a stream; the first `streams` lanes own them
 };
 
@@ -101,7 +103,7 @@ static int transfer_create_body(axr_pool_t* pool, size_t slot_bytes, int lanes, 
     else if (!rc) rc = axr_stream_create(&lane.stream);
     if (!rc) rc = axr_event_create(&lane.done);
     if (!rc) rc = axr_pool_alloc(pool, slot_bytes, 256, &lane.send_slot, &lane.send_mem_h);
-    if (!rc) rc = axr_pool_alloc(pool, slot_bytes, 256, &lane.recv_slot, nullptr);
+    // (receive slots are only needed by the copying mode and are allocated when it is chosen)
   }
   // rendezvous for every chunk with a payload: the wire copy is stream ordered
   if (!rc) rc = axr_am_context_create("transfer-sender", 1, &t->client);
@@ -143,6 +145,12 @@ static int transfer_submit_body(axr_transfer_t* t, axr_plan_t* send_plan, int64_
   if (rc) return rc;
   ++t->submitted;
 
+  if (!t->zero_copy && !lane.recv_slot) {
+    rc = axr_pool_alloc(t->pool, t->slot_bytes, 256, &lane.recv_slot, nullptr);
+    if (rc) return rc;
+  }
+  uint64_t borrowed_key = 0;
+  void* source = t->zero_copy ? lane.send_slot : lane.recv_slot;
   axr_job_t job;
   std::memset(&job, 0, sizeof(job));
   // The payload side keeps the plans' own cache treatment (cacheable up to the size of the
@@ -155,6 +163,11 @@ static int transfer_submit_body(axr_transfer_t* t, axr_plan_t* send_plan, int64_
   job.tensor_delta = send_delta;
   rc = axr_submit(&job, 1, lane.stream);
   if (rc) return rc;
+  auto give_up = [&](int status) {
+    // the pack is on the lane's stream already: let it finish before the slot is reused
+    (void)axr_stream_synchronize(lane.stream);
+    return status;
+  };
   if (nbytes) {
     axr_am_data_t am;
     std::memset(&am, 0, sizeof(am));
@@ -163,42 +176,95 @@ static int transfer_submit_body(axr_transfer_t* t, axr_plan_t* send_plan, int64_
     am.buffer_type = AXR_MEM_ROCM;
     am.mem_h = lane.send_mem_h;
     rc = axr_am_send(t->client, t->conn, &am, lane.stream, &lane.request);
-    if (rc) return rc;
+    if (rc) return give_up(rc);
     // From here on a failure must not leave the send parked or its message queued: the
     // slot is reused by the chunk after next.
     axr_am_message_t msg;
     rc = axr_am_recv_header(t->server, &msg);
     if (rc) {
       (void)axr_am_request_cancel(t->client, lane.request);
-      return rc;
+      return give_up(rc);
     }
-    // what arrived is what the receiver planned for
-    if (!msg.is_rndv || msg.data_length != nbytes || msg.header.size != recv_header_bytes ||
+    // what arrived is what the receiver planned for (tests can make one chunk fail here)
+    bool injected = false;
+    {
+      std::atomic<int64_t>& countdown = tunables().transfer_fail_after_send;
+      int64_t left = countdown.load();
+      while (left > 0 && !countdown.compare_exchange_weak(left, left - 1)) {
+      }
+      injected = left == 1;
+    }
+    if (injected || !msg.is_rndv || msg.data_length != nbytes || msg.header.size != recv_header_bytes ||
         std::memcmp(msg.header.data, recv_header, recv_header_bytes) != 0) {
       (void)axr_am_message_release(t->server, msg.key);
       (void)axr_am_request_cancel(t->client, lane.request);
-      return fail(AXR_ERR_MISMATCH, "the received message does not match the receiver's plan");
+      return give_up(fail(AXR_ERR_MISMATCH, "the received message does not match the receiver's plan"));
     }
-    rc = axr_am_recv_buffer_async(t->server, msg.key, AXR_MEM_ROCM, lane.recv_slot, t->slot_bytes,
-                                  lane.stream);
+    if (t->zero_copy) {
+      void* lent = nullptr;
+      size_t lent_bytes = 0;
+      rc = axr_am_recv_buffer_borrow(t->server, msg.key, &lent, &lent_bytes, nullptr);
+      if (!rc && (lent != lane.send_slot || lent_bytes != nbytes)) {
+        (void)axr_am_borrow_release(t->server, msg.key, lane.stream);
+        rc = fail(AXR_ERR_MISMATCH, "the borrowed payload is not the chunk that was sent");
+      }
+      if (!rc) {
+        borrowed_key = msg.key;
+        source = lent;
+      }
+    } else {
+      rc = axr_am_recv_buffer_async(t->server, msg.key, AXR_MEM_ROCM, lane.recv_slot, t->slot_bytes,
+                                    lane.stream);
+    }
     if (rc) {
       (void)axr_am_message_release(t->server, msg.key);
       (void)axr_am_request_cancel(t->client, lane.request);
+      // the lane's stream may already hold this chunk's pack: drain it, so that the slot is
+      // quiet before the next chunk on this lane reuses it
+      (void)axr_stream_synchronize(lane.stream);
       return rc;
     }
     lane.in_flight = true;
   }
   job.plan = recv_plan;
   job.unpack = 1;
-  job.payload = lane.recv_slot;
+  job.payload = source;
   job.tensor_delta = recv_delta;
   rc = axr_submit(&job, 1, lane.stream);
-  if (rc) return rc;
-  return axr_event_record(lane.done, lane.stream);
+  // the send completes behind the scatter that reads its slot (also when the scatter was refused:
+  // the lane must come back to a state in which retire() finds a completed send)
+  if (borrowed_key) {
+    const int released = axr_am_borrow_release(t->server, borrowed_key, lane.stream);
+    if (!rc) rc = released;
+  }
+  const int recorded = axr_event_record(lane.done, lane.stream);
+  if (rc || recorded) {
+    // whatever was enqueued runs to its end before the error is reported: the lane's event and
+    // send request are then settled and the next chunk finds the lane idle
+    (void)axr_stream_synchronize(lane.stream);
+    if (lane.in_flight) {
+      int done = 0;
+      (void)axr_am_request_test(t->client, lane.request, &done);
+      lane.in_flight = false;
+    }
+    return rc ? rc : recorded;
+  }
+  return AXR_OK;
 }
 int axr_transfer_submit(axr_transfer_t* transfer, axr_plan_t* send_plan, int64_t send_delta,
                         axr_plan_t* recv_plan, int64_t recv_delta) {
   return guarded([&] { return transfer_submit_body(transfer, send_plan, send_delta, recv_plan, recv_delta); });
+}
+
+static int transfer_set_zero_copy_body(axr_transfer_t* t, int enable) {
+  if (!t) return fail(AXR_ERR_INVALID, "axr_transfer_set_zero_copy: null transfer");
+  for (auto& lane : t->lanes)
+    if (lane.in_flight) return fail(AXR_ERR_BUSY, "axr_transfer_set_zero_copy: chunks are in flight; call axr_transfer_finish first");
+  t->zero_copy = enable != 0;
+  return AXR_OK;
+}
+int axr_transfer_set_zero_copy(axr_transfer_t* transfer, int enable) {
+  return guarded([&] { return transfer_set_zero_copy_body(transfer, enable); });
 }
 
 static int transfer_finish_body(axr_transfer_t* t) {

@@ -259,6 +259,9 @@ class StreamedTransfer {
   void Submit(const BundlePlan& send, int64_t send_delta, const BundlePlan& recv, int64_t recv_delta) {
     Check(axr_transfer_submit(transfer_, send.get(), send_delta, recv.get(), recv_delta), "axr_transfer_submit");
   }
+  // Zero copy (the default): the receiver scatters straight out of the sender's slot, as after a
+  // same-device zero-copy rendezvous; false: every chunk is copied into a receive slot first.
+  void SetZeroCopy(bool enable) { Check(axr_transfer_set_zero_copy(transfer_, enable ? 1 : 0), "axr_transfer_set_zero_copy"); }
   // Returns when every submitted chunk has arrived in its destination tensors.
   void Finish() { Check(axr_transfer_finish(transfer_), "axr_transfer_finish"); }
 

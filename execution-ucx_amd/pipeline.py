@@ -21,13 +21,18 @@ from .memory import DevicePool
 
 
 def _geometry(arr: TensorArray) -> Tuple[int, tuple]:
-    """(address of the first tensor, everything else relative to it)."""
+    """(address of the first tensor, everything else relative to it).  A bundle with host
+    (kDLCPU) tensors cannot be moved to another base by an address delta (their pieces are
+    copied by the host, from the addresses the plan was bound to), so its key also holds the
+    base itself: host chunks at another address plan anew instead of being rebased."""
     n = arr.count
     if n == 0:
         return 0, ()
     a = arr.array
     base = (a[0].data or 0) + a[0].byte_offset
     key = []
+    if any(a[i].device_type == _capi.kDLCPU for i in range(n)):
+        key.append(("host tensors at", base))
     for i in range(n):
         t = a[i]
         nd = t.ndim
@@ -39,8 +44,10 @@ def _geometry(arr: TensorArray) -> Tuple[int, tuple]:
 
 class StreamedTransfer:
     def __init__(self, slot_bytes: int, pool: Optional[DevicePool] = None, streams: int = 2,
-                 align: int = 256, lanes: Optional[int] = None):
-        """``lanes`` slot pairs (default: max(2, streams)) over ``streams`` HIP streams."""
+                 align: int = 256, lanes: Optional[int] = None, zero_copy: bool = True):
+        """``lanes`` slot pairs (default: max(2, streams)) over ``streams`` HIP streams.
+        ``zero_copy``: the receiver unpacks straight out of the sender's slot (a same-device
+        zero-copy rendezvous); False copies every chunk into a receive slot first."""
         self._lib = _capi.load()
         self.pool = pool or DevicePool.default()
         self.align = align
@@ -49,6 +56,8 @@ class StreamedTransfer:
         lanes = max(2, streams) if lanes is None else lanes
         _capi.check(self._lib.axr_transfer_create(self.pool._h, slot_bytes, lanes, streams, C.byref(h)))
         self._h = h.value
+        if not zero_copy:
+            _capi.check(self._lib.axr_transfer_set_zero_copy(self._h, 0))
         self._plans = None            # (src key, dst key, src base, dst base, send plan, recv plan)
         self._keep: List[Any] = []    # descriptor arrays of chunks that may still be in flight
 

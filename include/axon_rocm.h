@@ -452,6 +452,9 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * other in the bundle share wavefronts: up to 64 tensors or 128 sixteen-byte lane slots
  * per wavefront, so that wavefronts and table bytes scale with the payload and not with
  * the tensor count; default 512, at most 1023, 0: every tensor gets wavefronts of its own),
+ * "transfer_fail_after_send" (failure injection for tests: N > 0 makes the N-th chunk that
+ * axr_transfer_submit is given from now on fail with AXR_ERR_MISMATCH after its send has been
+ * queued, as if the message that arrived did not match the receiver's plan; 0, the default: off),
  * "inline_tables" (the first launch of a bundle of at most this many tiles
  * whose tables fit into 3.5 KiB carries the tables inside the kernel arguments:
  * no table block and no upload; a plan that is launched again uploads its
@@ -556,6 +559,23 @@ AXR_API int axr_am_recv_buffer_async(axr_am_context_t* ctx, uint64_t key, int ds
 AXR_API int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,
                                    const axr_buffer_t* buffer_vec, size_t buffer_count,
                                    void* stream);
+/* Zero-copy fetch of a rendezvous payload: instead of copying, the receiver is handed the
+ * sender's buffer (what a same-process rocm_ipc zero-copy rendezvous gives two endpoints
+ * that share a device: UCX maps the sender's registered memory and the "receive" is a
+ * pointer).  Only for a message whose payload is ONE contiguous buffer in memory the
+ * receiver can address (ROCM, ROCM_MANAGED or HOST of the same process); an iov message ->
+ * AXR_ERR_UNSUPPORTED (fetch it with axr_am_recv_buffer*).  Unknown key ->
+ * AXR_ERR_NO_MESSAGE, eager message -> AXR_ERR_NOT_IMPLEMENTED, cancelled by the sender ->
+ * AXR_ERR_CANCELED.  On success the message is claimed (the sender can no longer cancel),
+ * *data / *bytes / *memory_type describe the sender's buffer, and the send stays incomplete
+ * until axr_am_borrow_release: the sender must not touch the buffer before its request
+ * tests complete, exactly as for a copying fetch that is still running. */
+AXR_API int axr_am_recv_buffer_borrow(axr_am_context_t* ctx, uint64_t key, void** data, size_t* bytes,
+                                      int* memory_type);
+/* The receiver has enqueued its last read of a borrowed buffer on `stream`: the sender's
+ * request completes when the work that `stream` holds now has run (no host wait).  Unknown
+ * key -> AXR_ERR_NO_MESSAGE. */
+AXR_API int axr_am_borrow_release(axr_am_context_t* ctx, uint64_t key, void* stream);
 /* Drop a message's host copies (and, for an unfetched rendezvous, complete the
  * sender's request as cancelled). */
 AXR_API int axr_am_message_release(axr_am_context_t* ctx, uint64_t key);
@@ -582,7 +602,8 @@ AXR_API int axr_am_pending(axr_am_context_t* ctx, size_t* count);
  * one chunk ahead; on one GPU, where gather, wire copy and scatter all compete for
  * the same HBM, this is the faster arrangement.  The transport is a loopback context
  * pair inside the object: every chunk with a payload is a rendezvous whose fetch is
- * a stream-ordered device copy from the send slot to the receive slot.
+ * either a borrow of the send slot (the default) or a stream-ordered device copy from
+ * the send slot to a receive slot (axr_transfer_set_zero_copy).
  *
  * The caller keeps ONE sender plan and ONE receiver plan (axr_plan_from_header of
  * the sender's header, bound to the destination tensors) for all chunks of one
@@ -597,6 +618,13 @@ AXR_API int axr_transfer_create(axr_pool_t* pool, size_t slot_bytes, int lanes, 
                                 axr_transfer_t** transfer);
 AXR_API int axr_transfer_submit(axr_transfer_t* transfer, axr_plan_t* send_plan, int64_t send_delta,
                                 axr_plan_t* recv_plan, int64_t recv_delta);
+/* How a chunk crosses the loopback wire.  1 (the default): the receiver borrows the sender's
+ * slot (axr_am_recv_buffer_borrow) and unpacks straight out of it, the send completing after
+ * the unpack: 4P bytes per chunk, what a zero-copy rendezvous between two endpoints on one
+ * device costs.  0: the payload is copied from the send slot to a receive slot first
+ * (axr_am_recv_buffer_async), 6P bytes per chunk, what a transport that stages through its
+ * own buffers costs.  Call between chunks only (AXR_ERR_BUSY while chunks are in flight). */
+AXR_API int axr_transfer_set_zero_copy(axr_transfer_t* transfer, int enable);
 /* Returns when every submitted chunk has arrived in its destination tensors. */
 AXR_API int axr_transfer_finish(axr_transfer_t* transfer);
 /* Finishes, then releases the slots, streams and contexts. */

@@ -703,11 +703,13 @@ def test_c5_pitched_chunk(pkg, orc, gpu):
         assert int(twin[:, :, spec.cols:].view(torch.int16).ne(0).sum()) == 0     # pitch gap untouched
 
 
-def test_c5_streamed_pipeline(pkg, gpu):
+@pytest.mark.parametrize("zero_copy", [True, False])
+def test_c5_streamed_pipeline(pkg, gpu, zero_copy):
     """Double-buffered pack -> loopback send -> unpack over two streams: small
     chunks (eager and rendezvous sizes by the reference's threshold) and the full
     stream of 32 chunks of 256 MiB (8 GiB), all chunks of a stream served by one
-    sender plan and one receiver plan."""
+    sender plan and one receiver plan.  With the receiver borrowing the sender's slot
+    (zero copy) and with a copy into a receive slot."""
     import torch
     from execution_ucx_amd import workloads
     for spec, chunks in ((workloads.pitched_chunk(views=3, rows=4, cols=64), 7),
@@ -718,7 +720,7 @@ def test_c5_streamed_pipeline(pkg, gpu):
         dst = torch.zeros_like(src)
         torch.cuda.synchronize()
         slot = (spec.view_bytes + 255) // 256 * 256 * spec.views
-        st = pkg.StreamedTransfer(slot_bytes=slot, streams=2)
+        st = pkg.StreamedTransfer(slot_bytes=slot, streams=2, zero_copy=zero_copy)
         per_chunk = spec.views * spec.parent_elems * 2
         for k in range(chunks):
             st.submit(workloads.pitched_views(src.data_ptr() + k * per_chunk, spec),
@@ -732,6 +734,43 @@ def test_c5_streamed_pipeline(pkg, gpu):
         assert pkg.DevicePool.default().stats()["live_blocks"] == 0
         del src, dst, s16, d16
         torch.cuda.empty_cache()
+
+
+def test_streamed_host_chunks_plan_anew(pkg, gpu):
+    """Chunks of host (numpy) tensors of one geometry at different addresses: a bundle with
+    host tensors cannot be rebased by an address delta, so every chunk at a new base gets
+    fresh plans (and the result is right from the second chunk on)."""
+    import torch
+    rng = np.random.default_rng(21)
+    chunks = 4
+    srcs = [[rng.integers(0, 256, size=n, dtype=np.uint8) for n in (70000, 33, 4096)] for _ in range(chunks)]
+    outs = [[np.zeros_like(a) for a in c] for c in srcs]
+    st = pkg.StreamedTransfer(slot_bytes=1 << 20, streams=2)
+    plans_seen = set()
+    for c, o in zip(srcs, outs):
+        st.submit(c, o)
+        plans_seen.add(id(st._plans[4]))
+    st.finish()
+    for c, o in zip(srcs, outs):
+        for a, b in zip(c, o):
+            assert np.array_equal(a, b)
+    assert len(plans_seen) == chunks                     # no plan was moved by a delta
+    # the same chunk again reuses its plans (same base: delta 0)
+    st.submit(srcs[-1], outs[-1])
+    assert id(st._plans[4]) in plans_seen
+    st.finish()
+    st.close()
+    # device chunks of one geometry still share one pair of plans
+    dev = torch.from_numpy(rng.integers(0, 256, size=(3, 5000), dtype=np.uint8)).to(gpu)
+    back = torch.zeros_like(dev)
+    st = pkg.StreamedTransfer(slot_bytes=1 << 20, streams=1)
+    ids = set()
+    for k in range(3):
+        st.submit([dev[k, :3000], dev[k, 3000:]], [back[k, :3000], back[k, 3000:]])
+        ids.add(id(st._plans[4]))
+    st.finish()
+    assert len(ids) == 1 and torch.equal(dev, back)
+    st.close()
 
 
 def test_streamed_transfer_through_the_c_abi(pkg, orc, gpu):
@@ -749,13 +788,14 @@ def test_streamed_transfer_through_the_c_abi(pkg, orc, gpu):
                                         dtype=np.int16)).to(gpu).view(torch.bfloat16)
     send = pkg.BundlePlan.create(workloads.pitched_views(src.data_ptr(), spec), align=256)
     slot = send.payload_bytes
-    for lanes, streams in ((1, 1), (2, 2), (2, 1), (3, 2)):
+    for lanes, streams, zero_copy in ((1, 1, 1), (2, 2, 1), (2, 1, 0), (3, 2, 0), (2, 2, 0), (3, 2, 1)):
         dst = torch.zeros_like(src)
         recv = pkg.BundlePlan.from_header(send.header).bind(workloads.pitched_views(dst.data_ptr(), spec))
         torch.cuda.synchronize()
         t = C.c_void_p()
         assert lib.axr_transfer_create(None, slot, lanes, lanes + 1, C.byref(t)) == capi.AXR_ERR_INVALID
         capi.check(lib.axr_transfer_create(None, slot, lanes, streams, C.byref(t)))
+        capi.check(lib.axr_transfer_set_zero_copy(t, zero_copy))
         # chunks in a scrambled order: deltas need not grow
         order = [int(k) for k in rng.permutation(chunks)]
         for k in order:
@@ -771,6 +811,26 @@ def test_streamed_transfer_through_the_c_abi(pkg, orc, gpu):
         bigplan = pkg.BundlePlan.create([big], align=256)
         bigrecv = pkg.BundlePlan.from_header(bigplan.header).bind([torch.zeros_like(big)])
         assert lib.axr_transfer_submit(t, bigplan._h, 0, bigrecv._h, 0) == capi.AXR_ERR_LENGTH
+        # a chunk that fails after its send was queued (injected: the message "does not match"):
+        # the send is withdrawn, the lane comes back idle, and good chunks follow on every lane
+        dst.zero_()
+        torch.cuda.synchronize()
+        capi.check(lib.axr_transfer_submit(t, send._h, 0, recv._h, 0))
+        pkg.tune(transfer_fail_after_send=1)
+        assert lib.axr_transfer_submit(t, send._h, per_chunk, recv._h, per_chunk) == capi.AXR_ERR_MISMATCH
+        assert b"does not match" in lib.axr_last_error()
+        for k in range(2, 2 + 2 * lanes):
+            capi.check(lib.axr_transfer_submit(t, send._h, k * per_chunk, recv._h, k * per_chunk))
+        capi.check(lib.axr_transfer_finish(t))
+        d16 = dst.view(torch.int16)
+        moved = [0] + list(range(2, 2 + 2 * lanes))
+        assert torch.equal(d16[moved][..., :spec.cols], s16[moved][..., :spec.cols])
+        assert int(d16[1].ne(0).sum()) == 0                       # the failed chunk moved nothing
+        # the mode cannot change under chunks in flight
+        capi.check(lib.axr_transfer_submit(t, send._h, 0, recv._h, 0))
+        assert lib.axr_transfer_set_zero_copy(t, 1 - zero_copy) == capi.AXR_ERR_BUSY
+        capi.check(lib.axr_transfer_finish(t))
+        capi.check(lib.axr_transfer_set_zero_copy(t, zero_copy))
         # another geometry through the same transfer (smaller than a slot)
         a = torch.from_numpy(rng.integers(0, 256, size=5000, dtype=np.uint8)).to(gpu)
         b = torch.zeros_like(a)
