@@ -277,6 +277,11 @@ uint64_t stream_launch_mark();
 void stream_note_drained(void* stream, uint64_t mark);
 bool stream_drained(void* stream, uint64_t mark);
 void stream_forget(void* stream);   // the stream is being destroyed
+// A kernel that writes device-visible HOST memory has been enqueued on `stream`: the next
+// axr_stream_synchronize of that stream must be the runtime's wait (which makes such writes
+// visible to the CPU), not the polled one.  take: true once per note, then forgotten.
+void stream_note_host_writes(void* stream);
+bool stream_take_host_writes(void* stream);
 int fail_nothrow(int status, const char* message) noexcept;
 
 // Every extern "C" entry point runs its body through this: no C++ exception

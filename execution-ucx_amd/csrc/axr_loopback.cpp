@@ -80,6 +80,12 @@ std::set<const void*> g_contexts;
 struct axr_am_context {
   std::string name;
   size_t zcopy_thresh = 4096;
+  // Held from the decision "this message goes out now" until it lies in the peer's queue, in
+  // deliver() and in progress(): with several sending threads the order in which messages
+  // reach the peer is then the order in which that decision was taken, and a message that
+  // progress() has just taken off the waiting queue cannot be overtaken by a newer send.
+  // Taken before `mu`, never while `mu` is held.
+  std::mutex send_mu;
   std::mutex mu;
   std::deque<std::unique_ptr<Message>> arrived;          // not yet seen by recv_header
   std::map<uint64_t, std::unique_ptr<Message>> parked;   // handed out, awaiting fetch/release
@@ -138,7 +144,8 @@ int hand_over(axr_am_context* peer, std::unique_ptr<Message> m) {
 }
 
 // Forgets completed sends and starts waiting ones while there is room, in order.
-void progress(axr_am_context* ctx) {
+// ctx->send_mu is held by the caller.
+void progress_locked(axr_am_context* ctx) {
   for (;;) {
     axr_am_context* peer = nullptr;
     std::unique_ptr<Message> m;
@@ -172,8 +179,14 @@ void progress(axr_am_context* ctx) {
   }
 }
 
+void progress(axr_am_context* ctx) {
+  std::lock_guard<std::mutex> order(ctx->send_mu);
+  progress_locked(ctx);
+}
+
 int deliver(axr_am_context* ctx, uint64_t conn_id, std::unique_ptr<Message> m, uint64_t* request) {
-  progress(ctx);
+  std::lock_guard<std::mutex> order(ctx->send_mu);
+  progress_locked(ctx);
   axr_am_context* peer = nullptr;
   bool wait = false;
   {

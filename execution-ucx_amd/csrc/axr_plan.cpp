@@ -182,6 +182,7 @@ struct axr_plan {
   std::vector<uint8_t> group_blocks; // kGroupBlockBytes per group tile: GroupHead, then Member records
   std::vector<uint32_t> member_tensor;   // kGroupMaxMembers tensor indices per block (inspection)
   bool groups_only = false;          // every tile is a group tile: the kernel walks the blocks directly
+  bool pinned_host_tensors = false;  // some tensor lies in device-visible host memory (kDLROCMHost)
   std::vector<HostCopy> host_copies;
   std::vector<uint32_t> host_copy_tensor;
   std::vector<HostChunk> host_chunks;
@@ -353,6 +354,7 @@ void invalidate_tables(axr_plan* p) {
   p->group_blocks.clear();
   p->member_tensor.clear();
   p->groups_only = false;
+  p->pinned_host_tensors = false;
   p->host_copies.clear();
   p->host_copy_tensor.clear();
   p->host_chunks.clear();
@@ -884,11 +886,13 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   }
   Seg* staged = static_cast<Seg*>(p->block.host);
   uint64_t tiles = 0;
+  bool pinned = false;
   const bool receiver = p->receiver;
   const uint64_t align_mask = static_cast<uint64_t>(p->align) - 1;
   for (size_t i = 0; i < n; ++i) {
     const TensorRec& t = p->tensors[i];
     if ((t.device_type != kDLROCM && t.device_type != kDLROCMHost) || t.nbytes > kSegRunMask) return AXR_OK;
+    pinned = pinned || t.device_type == kDLROCMHost;
     if (t.has_strides && t.nbytes && !compact_strides(p->shape_of(t), p->strides_of(t), t.ndim)) return AXR_OK;
     Seg& sg = staged[i];
     sg.ptr = t.address;
@@ -914,6 +918,7 @@ int device_build_tables(axr_plan* p, hipStream_t stream, bool* done) {
   p->wave_seg.clear();
   p->ntiles = static_cast<uint32_t>(tiles);
   p->cfg.lds_per_wave = 0;
+  p->pinned_host_tensors = pinned;
   finish_geometry(p, rows, n);
   p->dims_at = wave_at;
   p->wave_at = wave_at;
@@ -1011,6 +1016,7 @@ int build_tables(axr_plan* p) {
       collapse(t, shape, strides, item, &c);
     }
     int rc;
+    if (t.device_type == kDLROCMHost) p->pinned_host_tensors = true;
     if (t.device_type == kDLROCM || t.device_type == kDLROCMHost) {
       if (c.nd == 0 && b.add_member(static_cast<uint32_t>(i), t.address, t.offset, t.nbytes, pad, &rc)) {
         if (rc) return rc;
@@ -1325,6 +1331,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
                                      static_cast<uint32_t>(p->wave_at), stream);
     if (rc) return rc;
     ++p->launches;
+    if (!pack && p->pinned_host_tensors) stream_note_host_writes(stream);
     // The launch needs nothing of the plan any more, but callers rely on axr_plan_free and
     // axr_plan_bind returning only when the plan's launches are done (they release the
     // payload or the tensors next), so the stream is remembered all the same.
@@ -1344,6 +1351,7 @@ int run(axr_plan* p, bool pack, void* payload, size_t payload_bytes, void* strea
   rc = launch_bundle_kernel(pack, a, cfg, stream);
   if (rc) return rc;
   ++p->launches;
+  if (!pack && p->pinned_host_tensors) stream_note_host_writes(stream);
   // a capturing stream cannot be drained later; the caller keeps the plan alive
   // for as long as the graph can run
   if (!capturing) remember_stream(p, stream);
@@ -1751,6 +1759,18 @@ int axr_unpack(axr_plan_t* plan, const void* payload, size_t payload_bytes, void
   return guarded([&] { return unpack_body(plan, payload, payload_bytes, stream); });
 }
 
+// Who used the static table area of a device last, and an event behind that use.
+struct StaticAreaUse {
+  std::mutex mu;
+  hipEvent_t after_launch = nullptr;   // created at the first use, kept until the process ends
+  hipStream_t last_stream = nullptr;
+  bool used = false;
+};
+static StaticAreaUse& static_area_use(int device) {
+  static StaticAreaUse uses[64];
+  return uses[device >= 0 && device < 64 ? device : 0];
+}
+
 // axr_pack for callers that must not allocate device memory.  The tables ride in the
 // kernel arguments when they fit; otherwise they are copied, on `stream`, into the static
 // table area of the current device and the same kernel as axr_pack reads them there.
@@ -1806,32 +1826,50 @@ static int pack_noalloc_body(axr_plan_t* p, void* payload, size_t payload_bytes,
   rc = static_table_area(&area);
   if (rc) return rc;
   uint8_t* d = static_cast<uint8_t*>(area);
-  // Three copies out of the plan's own (pageable) vectors, ordered on `stream` behind
-  // whatever that stream's previous call still reads from the area.  The vectors live
-  // until the plan is rebound or freed, and both drain the stream first.
-  remember();
-  rc = check_hip(hipMemcpyAsync(d, p->segs.data(), p->segs.size() * sizeof(Seg), hipMemcpyHostToDevice, stream),
-                 "hipMemcpyAsync(segment table -> static area)");
-  if (!rc && !p->dims.empty())
-    rc = check_hip(hipMemcpyAsync(d + p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims),
-                                  hipMemcpyHostToDevice, stream),
-                   "hipMemcpyAsync(dims table -> static area)");
-  if (!rc)
-    rc = check_hip(hipMemcpyAsync(d + p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t),
-                                  hipMemcpyHostToDevice, stream),
-                   "hipMemcpyAsync(tile index -> static area)");
-  if (!rc && !p->group_blocks.empty())
-    rc = check_hip(hipMemcpyAsync(d + p->members_at, p->group_blocks.data(), p->group_blocks.size(),
-                                  hipMemcpyHostToDevice, stream),
-                   "hipMemcpyAsync(member records -> static area)");
+  // Calls on one stream are ordered by the stream.  A call on ANOTHER stream than the area's
+  // last user first waits (on the device, not on the host) for that user's launch: an event,
+  // created once per device, is recorded behind every launch that reads the area.
+  int device = 0;
+  rc = check_hip(hipGetDevice(&device), "hipGetDevice");
   if (rc) return rc;
-  a.segs = reinterpret_cast<const Seg*>(d);
-  a.dims = reinterpret_cast<const Dims*>(d + dims_arg_at(p));
-  a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
-  rc = launch_bundle_kernel(true, a, p->cfg, stream);
-  if (rc) return rc;
-  ++p->launches;
-  return AXR_OK;
+  StaticAreaUse& use = static_area_use(device);
+  std::lock_guard<std::mutex> area_lock(use.mu);
+  if (!use.after_launch) {
+    rc = check_hip(hipEventCreateWithFlags(&use.after_launch, hipEventDisableTiming), "hipEventCreate(static table area)");
+    if (rc) return rc;
+  }
+  if (use.used && use.last_stream != stream) {
+    rc = check_hip(hipStreamWaitEvent(stream, use.after_launch, 0), "hipStreamWaitEvent(static table area)");
+    if (rc) return rc;
+  }
+  // Copies out of the plan's own (pageable) vectors, ordered on `stream`.  The vectors live
+  // until the plan is rebound or freed, and both drain the stream first; the launch mark is
+  // taken once something has been enqueued, also when a later step fails.
+  bool enqueued = false;
+  auto copy = [&](size_t at, const void* src, size_t bytes, const char* what) {
+    if (rc || bytes == 0) return;
+    rc = check_hip(hipMemcpyAsync(d + at, src, bytes, hipMemcpyHostToDevice, stream), what);
+    enqueued = enqueued || rc == AXR_OK;
+  };
+  copy(0, p->segs.data(), p->segs.size() * sizeof(Seg), "hipMemcpyAsync(segment table -> static area)");
+  copy(p->dims_at, p->dims.data(), p->dims.size() * sizeof(Dims), "hipMemcpyAsync(dims table -> static area)");
+  copy(p->wave_at, p->wave_seg.data(), p->wave_seg.size() * sizeof(uint32_t), "hipMemcpyAsync(tile index -> static area)");
+  copy(p->members_at, p->group_blocks.data(), p->group_blocks.size(), "hipMemcpyAsync(group blocks -> static area)");
+  if (!rc) {
+    a.segs = reinterpret_cast<const Seg*>(d);
+    a.dims = reinterpret_cast<const Dims*>(d + dims_arg_at(p));
+    a.wave_seg = reinterpret_cast<const uint32_t*>(d + p->wave_at);
+    rc = launch_bundle_kernel(true, a, p->cfg, stream);
+    if (!rc) ++p->launches;
+  }
+  if (enqueued) {
+    remember();
+    use.used = true;
+    use.last_stream = stream;
+    const int recorded = check_hip(hipEventRecord(use.after_launch, stream), "hipEventRecord(static table area)");
+    if (!rc) rc = recorded;
+  }
+  return rc;
 }
 int axr_pack_noalloc(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream) {
   return guarded([&] { return pack_noalloc_body(plan, payload, payload_bytes, stream); });
@@ -1945,6 +1983,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     for (size_t k = i; k < end; ++k) {
       axr_plan* p = jobs[k].plan;
       ++p->launches;
+      if (jobs[k].unpack && p->pinned_host_tensors) stream_note_host_writes(stream);
       if (!capturing) remember_stream(p, stream);
     }
     i = end;

@@ -248,6 +248,7 @@ namespace {
 std::atomic<uint64_t> g_launch_mark{0};
 std::mutex g_drained_mutex;
 std::unordered_map<void*, uint64_t> g_drained;   // stream -> highest mark seen drained
+std::unordered_set<void*> g_host_writes;         // streams whose queued kernels write host memory
 }  // namespace
 uint64_t stream_mark_launch() { return g_launch_mark.fetch_add(1, std::memory_order_seq_cst) + 1; }
 uint64_t stream_launch_mark() { return g_launch_mark.load(std::memory_order_seq_cst); }
@@ -264,6 +265,15 @@ bool stream_drained(void* stream, uint64_t mark) {
 void stream_forget(void* stream) {
   std::lock_guard<std::mutex> lock(g_drained_mutex);
   g_drained.erase(stream);
+  g_host_writes.erase(stream);
+}
+void stream_note_host_writes(void* stream) {
+  std::lock_guard<std::mutex> lock(g_drained_mutex);
+  g_host_writes.insert(stream);
+}
+bool stream_take_host_writes(void* stream) {
+  std::lock_guard<std::mutex> lock(g_drained_mutex);
+  return g_host_writes.erase(stream) != 0;
 }
 }  // namespace axr
 
@@ -712,7 +722,11 @@ bool spin_until_stream_end(hipStream_t stream, int64_t budget_us) {
 
 static int stream_synchronize_body(void* stream) {
   const uint64_t reached = stream_launch_mark();
-  const int64_t budget = tunables().spin_wait_us;
+  // A kernel's writes to host memory become visible to the CPU with the completion the runtime
+  // waits for, which the polled wait returns ahead of: a stream that has scattered into
+  // device-visible host tensors since its last wait takes the runtime's wait.
+  const bool host_writes = stream_take_host_writes(stream);
+  const int64_t budget = host_writes ? 0 : tunables().spin_wait_us.load();
   if (!(budget > 0 && spin_until_stream_end(static_cast<hipStream_t>(stream), budget))) {
     int rc = check_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "hipStreamSynchronize");
     if (rc) return rc;

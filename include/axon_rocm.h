@@ -353,13 +353,18 @@ AXR_API int axr_submit(const axr_job_t* jobs, size_t n, void* stream);
  * bundle carries its tables inside the kernel arguments (as axr_pack's first launch
  * does); a larger one has them copied on `stream` into a table area that is part of
  * the library's device code: 1 MiB per GPU, held until the process ends (about
- * 25,000 contiguous tensors; AXR_ERR_LENGTH beyond that).  Every call on one GPU
- * shares that GPU's area: calls on ONE stream are ordered and may follow each other
- * without a wait; calls that overlap on two streams of one GPU race for it and must
- * be ordered by the caller.  Bundles with kDLCPU tensors (pinned staging) and,
- * under stream capture, bundles whose tables exceed the kernel arguments are
- * refused with AXR_ERR_UNSUPPORTED.  The plan must stay alive until the stream has
- * run the call (axr_plan_free and axr_plan_bind wait for it). */
+ * 25,000 contiguous tensors, or 50,000 short ones that share wavefronts;
+ * AXR_ERR_LENGTH beyond that).  Every call on one GPU shares that GPU's area: calls
+ * on ONE stream are ordered by the stream and may follow each other without a wait; a
+ * call on another stream than the area's last user is made to wait, on the device, for
+ * that user's launch (an event created once per GPU and recorded behind every launch
+ * that reads the area), so calls on two streams are serialised, not refused.  The table
+ * copies read the plan's pageable host memory with hipMemcpyAsync; the library allocates
+ * nothing for them, the HIP runtime may stage them through buffers of its own.
+ * Bundles with kDLCPU tensors (pinned staging) and, under stream capture, bundles whose
+ * tables exceed the kernel arguments are refused with AXR_ERR_UNSUPPORTED.  The plan
+ * must stay alive until the stream has run the call (axr_plan_free and axr_plan_bind
+ * wait for it). */
 AXR_API int axr_pack_noalloc(axr_plan_t* plan, void* payload, size_t payload_bytes, void* stream);
 
 /* Launch geometry of a plan's kernel, for profiling reports. */

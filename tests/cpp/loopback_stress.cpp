@@ -186,6 +186,76 @@ int main() {
   stop_churn.store(true);
   threads.back().join();
   if (int rc = axr_am_context_destroy(server)) die("destroy server", rc);
+
+  // Second phase: several threads send on ONE context (one connection each) while another
+  // thread keeps calling axr_am_progress on it.  Every send is a rendezvous and nobody fetches
+  // at first, so the context fills up (256 in flight) and the rest waits; then the receiver
+  // drains.  Every sender's messages must arrive in the order that sender sent them: a message
+  // that progress has just taken off the waiting queue must not be overtaken by a newer send.
+  {
+    axr_am_context_t *shared = nullptr, *sink = nullptr;
+    if (int rc = axr_am_context_create("shared", 1, &shared)) die("create shared", rc);
+    if (int rc = axr_am_context_create("sink", 1, &sink)) die("create sink", rc);
+    constexpr int kThreads = 3, kEach = 300;
+    std::atomic<bool> stop_progress{false};
+    std::atomic<int> sent{0};
+    std::vector<std::vector<uint64_t>> requests(kThreads, std::vector<uint64_t>(kEach));
+    static uint8_t payload[64];
+    std::vector<std::thread> phase;
+    for (int s = 0; s < kThreads; ++s) {
+      phase.emplace_back([s, shared, sink, &requests, &sent] {
+        uint64_t conn = 0;
+        if (int rc = axr_am_connect(shared, sink, &conn)) die("connect shared", rc);
+        for (int q = 0; q < kEach; ++q) {
+          Tag tag{static_cast<uint32_t>(s), static_cast<uint32_t>(q), sizeof(payload), 0};
+          axr_am_data_t d;
+          std::memset(&d, 0, sizeof(d));
+          d.header.data = &tag;
+          d.header.size = sizeof(tag);
+          d.buffer.data = payload;
+          d.buffer.size = sizeof(payload);
+          d.buffer_type = AXR_MEM_HOST;
+          if (int rc = axr_am_send(shared, conn, &d, nullptr, &requests[s][q])) die("send (shared)", rc);
+          sent.fetch_add(1);
+        }
+      });
+    }
+    phase.emplace_back([shared, &stop_progress] {
+      while (!stop_progress.load()) {
+        if (int rc = axr_am_progress(shared, nullptr, nullptr)) die("progress (shared)", rc);
+      }
+    });
+    std::vector<uint32_t> next(kThreads, 0);
+    int got = 0;
+    uint8_t into[64];
+    while (got < kThreads * kEach) {
+      axr_am_message_t m;
+      const int rc = axr_am_recv_header(sink, &m);
+      if (rc == AXR_ERR_NO_MESSAGE) {
+        std::this_thread::yield();
+        continue;
+      }
+      if (rc) die("recv_header (sink)", rc);
+      Tag tag;
+      std::memcpy(&tag, m.header.data, sizeof(tag));
+      if (tag.sender >= static_cast<uint32_t>(kThreads) || tag.seq != next[tag.sender]++)
+        die("order per sending thread on a shared context", -1);
+      if (int rc2 = axr_am_recv_buffer(sink, m.key, AXR_MEM_HOST, into, sizeof(into), nullptr)) die("recv_buffer (sink)", rc2);
+      ++got;
+    }
+    for (size_t i = 0; i < static_cast<size_t>(kThreads); ++i) phase[i].join();
+    stop_progress.store(true);
+    phase.back().join();
+    for (int s = 0; s < kThreads; ++s)
+      for (int q = 0; q < kEach; ++q) {
+        int done = 0;
+        if (int rc = axr_am_request_test(shared, requests[s][q], &done)) die("request_test (shared)", rc);
+        if (done != 1) die("a send on the shared context did not complete", done);
+      }
+    if (int rc = axr_am_context_destroy(shared)) die("destroy shared", rc);
+    if (int rc = axr_am_context_destroy(sink)) die("destroy sink", rc);
+    received.fetch_add(got);
+  }
   std::printf("loopback_stress ok %d\n", received.load());
   return 0;
 }

@@ -1531,6 +1531,26 @@ def test_polled_stream_wait(pkg, orc, gpu):
                     host.copy_(buf)                            # a blocking copy on another stream: no extra wait for ours
                     plan.close()
                     assert np.array_equal(host.numpy(), want), (budget, len(tensors))
+        # A scatter into pinned host tensors: the kernel writes host memory, which the runtime's
+        # wait makes visible and the polled wait does not promise to; the stream's next wait is
+        # therefore the runtime's, whatever the budget, and the CPU reads the data at once.
+        pkg.tune(spin_wait_us=200)
+        plan = pkg.BundlePlan.create(small, align=256)
+        buf = device_bytes(plan.payload_bytes, gpu)
+        torch.cuda.synchronize()
+        plan.pack(buf.data_ptr(), plan.payload_bytes, stream.value)
+        pinned = [torch.zeros(t.numel(), dtype=torch.uint8).pin_memory() for t in small]
+        rplan = pkg.BundlePlan.from_header(plan.header).bind(pinned)
+        assert {s["mode"] for s in rplan.segments()} <= {0, 6}        # device segments: the kernel writes them
+        for _ in range(5):
+            for t in pinned:
+                t.zero_()
+            rplan.unpack(buf.data_ptr(), plan.payload_bytes, stream.value)
+            check(lib.axr_stream_synchronize(stream))
+            for t, src in zip(pinned, small):
+                assert np.array_equal(t.numpy(), src.cpu().numpy())
+        rplan.close()
+        plan.close()
     finally:
         pkg.tune(spin_wait_us=0)
         check(lib.axr_stream_destroy(stream))

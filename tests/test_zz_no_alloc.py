@@ -88,6 +88,25 @@ def test_two_calls_in_a_row_match_axr_pack(pkg, orc, gpu, align):
         capi.check(lib.axr_stream_synchronize(stream))
         n = plans[0].payload_bytes
         assert np.array_equal(bufs[0].cpu().numpy()[:n], orc.pack(host_chunks(big), align))
+        # calls on TWO streams share the one table area: the second stream is made to wait for
+        # the first one's launch on the device, so alternating calls without any host wait
+        # still give each bundle its own tables
+        other = C.c_void_p()
+        capi.check(lib.axr_stream_create(C.byref(other)))
+        for buf in bufs:
+            buf.fill_(POISON)
+        assert pkg.streams.order_behind_producers(stream.value)
+        assert pkg.streams.order_behind_producers(other.value)
+        for _ in range(4):
+            capi.check(lib.axr_pack_noalloc(plans[0]._h, bufs[0].data_ptr(), plans[0].payload_bytes, stream))
+            capi.check(lib.axr_pack_noalloc(plans[1]._h, bufs[1].data_ptr(), plans[1].payload_bytes, other))
+        capi.check(lib.axr_stream_synchronize(stream))
+        capi.check(lib.axr_stream_synchronize(other))
+        for tensors, plan, buf in zip((big, small), plans, bufs):
+            n = plan.payload_bytes
+            got = buf.cpu().numpy()
+            assert np.array_equal(got[:n], orc.pack(host_chunks(tensors), align)) and (got[n:] == POISON).all()
+        capi.check(lib.axr_stream_destroy(other))
     finally:
         for plan in plans:
             plan.close()
