@@ -193,6 +193,12 @@ class AmMessage(C.Structure):
                 ("eager_data", Buffer)]
 
 
+class UcxProbe(C.Structure):
+    _fields_ = [("available", C.c_int), ("version_major", C.c_uint), ("version_minor", C.c_uint),
+                ("version_release", C.c_uint), ("have_symbol", C.c_int * 6), ("library", C.c_char * 256),
+                ("message", C.c_char * 512)]
+
+
 REGISTER_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p))
 UNREGISTER_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)
 
@@ -280,6 +286,9 @@ PROTOTYPES = {
     "axr_am_message_release": (C.c_int, [_vp, C.c_uint64]),
     "axr_am_message_info": (C.c_int, [_vp, C.c_uint64, _u64p, _u64p, _intp]),
     "axr_am_pending": (C.c_int, [_vp, C.POINTER(_sz)]),
+    "axr_ucx_probe": (C.c_int, [C.POINTER(UcxProbe)]),
+    "axr_ucx_symbol_name": (C.c_char_p, [C.c_int]),
+    "axr_am_context_create_ucx": (C.c_int, [C.c_char_p, _vpp]),
     "axr_transfer_create": (C.c_int, [_vp, _sz, C.c_int, C.c_int, _vpp]),
     "axr_transfer_submit": (C.c_int, [_vp, _vp, C.c_int64, _vp, C.c_int64]),
     "axr_transfer_set_zero_copy": (C.c_int, [_vp, C.c_int]),

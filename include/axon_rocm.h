@@ -594,6 +594,31 @@ AXR_API int axr_am_message_info(axr_am_context_t* ctx, uint64_t key, uint64_t* d
 /* Messages queued and not yet taken by axr_am_recv_header. */
 AXR_API int axr_am_pending(axr_am_context_t* ctx, size_t* count);
 
+/* ------------------------------------------------------------- UCX, probed */
+
+/* What a real UCX backend needs from the machine, found at run time: the reference links
+ * OpenUCX at build time (ucp_init / ucp_worker_create, ucx_am_context.cpp:694-749; ucp_mem_map,
+ * :1128-1147; ucp_am_send_nbx and ucp_am_recv_data_nbx, ucx_connection.cpp:353-453;
+ * ucp_worker_progress, ucx_am_context.cpp:218-296).  This library looks for libucp.so.0
+ * (or the file named by the environment variable AXR_UCX_LIBRARY) with dlopen, resolves those
+ * entry points and reads the version.  It calls nothing else: the parameter structures of the
+ * UCX calls come from ucp.h, which this build was made without. */
+#define AXR_UCX_SYMBOLS 6
+typedef struct axr_ucx_probe {
+  int available;                      /* 1: the library loaded and every entry point is there */
+  unsigned version_major, version_minor, version_release;   /* ucp_get_version, 0 when unknown */
+  int have_symbol[AXR_UCX_SYMBOLS];   /* in the order of axr_ucx_symbol_name */
+  char library[256];                  /* the name dlopen accepted, "" when none */
+  char message[512];                  /* one line for a log */
+} axr_ucx_probe_t;
+/* Probes once per process; later calls return the first result. */
+AXR_API int axr_ucx_probe(axr_ucx_probe_t* probe);
+AXR_API const char* axr_ucx_symbol_name(int index);
+/* The UCX-backed counterpart of axr_am_context_create.  Always AXR_ERR_UNSUPPORTED in this
+ * build, with a message that says which of the two things is missing: the UCX library on
+ * this machine, or (when it is there) the UCX headers at build time.  *ctx is NULL. */
+AXR_API int axr_am_context_create_ucx(const char* name, axr_am_context_t** ctx);
+
 /* ------------------------------------------------------- streamed transfers */
 
 /* A large payload moved in chunks: pack -> connection_send -> connection_recv_buffer
@@ -648,6 +673,14 @@ AXR_API int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mi
  * a packed buffer equals the sum of its tensors' checksums taken with
  * start = offset[i]. */
 AXR_API int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum);
+/* --------------------------------------------------------------- calibration */
+
+/* The two entry points below are NOT part of the drop-in surface: nothing of the reference
+ * corresponds to them and no caller of the bundle path needs them.  They are the yardsticks
+ * the measurements are read against (what a plain copy, and a plain gather of equal rows,
+ * reach on the same device), kept in the library so that they run with the same compiler
+ * flags, streams and timing harness as the kernels they calibrate. */
+
 /* Plain device copy kernel (16 B per lane, grid-stride); calibration
  * reference for profiler counters and bandwidth. */
 AXR_API int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream);

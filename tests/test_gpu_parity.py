@@ -1540,7 +1540,9 @@ def test_polled_stream_wait(pkg, orc, gpu):
         torch.cuda.synchronize()
         plan.pack(buf.data_ptr(), plan.payload_bytes, stream.value)
         pinned = [torch.zeros(t.numel(), dtype=torch.uint8).pin_memory() for t in small]
-        rplan = pkg.BundlePlan.from_header(plan.header).bind(pinned)
+        views = [pkg.TensorView(data=p.data_ptr(), device_type=11, device_id=0, dtype=(1, 8, 1),
+                                shape=(p.numel(),), strides=None, owner=p) for p in pinned]
+        rplan = pkg.BundlePlan.from_header(plan.header).bind(views)
         assert {s["mode"] for s in rplan.segments()} <= {0, 6}        # device segments: the kernel writes them
         for _ in range(5):
             for t in pinned:

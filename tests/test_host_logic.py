@@ -781,3 +781,74 @@ def test_header_whose_sizes_wrap_64_bits_is_refused(pkg):
     h += struct.pack("<QQiiiBBHQq", 0, 1, 10, 0, 1, 1, 8, 1, 0, 1)
     with pytest.raises(pkg.AxonRocmError):
         pkg.BundlePlan.from_header(h)
+
+
+def _probe_in_subprocess(env_library=None):
+    """axr_ucx_probe and axr_am_context_create_ucx in a fresh process (the probe runs once per
+    process), optionally with AXR_UCX_LIBRARY naming the library to load."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import ctypes as C, json, sys\n"
+        f"sys.path.insert(0, {root!r})\n"
+        "import __graft_entry__ as e\n"
+        "pkg = e.load_package(); capi = pkg._capi; lib = capi.load()\n"
+        "p = capi.UcxProbe(); assert lib.axr_ucx_probe(C.byref(p)) == 0\n"
+        "ctx = C.c_void_p(1)\n"
+        "rc = lib.axr_am_context_create_ucx(b'x', C.byref(ctx))\n"
+        "print(json.dumps({'available': p.available, 'version': [p.version_major, p.version_minor, p.version_release],\n"
+        "  'have': list(p.have_symbol), 'library': p.library.decode(), 'message': p.message.decode(),\n"
+        "  'names': [lib.axr_ucx_symbol_name(i).decode() for i in range(6)],\n"
+        "  'rc': rc, 'ctx': ctx.value, 'error': lib.axr_last_error().decode()}))\n")
+    env = dict(os.environ)
+    env.pop("AXR_UCX_LIBRARY", None)
+    if env_library is not None:
+        env["AXR_UCX_LIBRARY"] = env_library
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
+    assert out.returncode == 0, out.stderr[-2000:]
+    return json.loads(out.stdout.strip().splitlines()[-1])
+
+
+def test_ucx_backend_is_probed_and_refused_clearly(pkg, tmp_path):
+    """No UCX on this image: the probe says so, and the UCX-backed context is refused with
+    AXR_ERR_UNSUPPORTED and a message that names the library and the loopback alternative.
+    With a library that exports the entry points (a stand-in built here: the probe only looks
+    symbols up and asks for the version) the refusal names the other missing piece, the UCX
+    headers at build time.  Nothing beyond this probe exists of a UCX backend."""
+    import shutil
+    import subprocess
+    capi = pkg._capi
+    r = _probe_in_subprocess()
+    assert r["names"] == ["ucp_init_version", "ucp_worker_create", "ucp_mem_map", "ucp_am_send_nbx",
+                          "ucp_am_recv_data_nbx", "ucp_worker_progress"]
+    if not r["available"]:                       # the image as it is
+        assert r["library"] == "" and r["have"] == [0] * 6
+        assert "libucp.so.0" in r["message"]
+        assert r["rc"] == capi.AXR_ERR_UNSUPPORTED and r["ctx"] is None
+        assert "libucp.so.0" in r["error"] and "axr_am_context_create" in r["error"]
+    # a named library that does not exist is the only one tried
+    r = _probe_in_subprocess(str(tmp_path / "nowhere" / "libucp.so.0"))
+    assert not r["available"] and "nowhere" in r["message"] and r["rc"] == capi.AXR_ERR_UNSUPPORTED
+    gcc = shutil.which("gcc")
+    if not gcc:
+        pytest.skip("no C compiler for the stand-in library")
+    src = tmp_path / "standin.c"
+    src.write_text(
+        "void ucp_get_version(unsigned* a, unsigned* b, unsigned* c) { *a = 1; *b = 20; *c = 0; }\n"
+        + "".join(f"int {n}(void) {{ return -1; }}\n" for n in
+                  ("ucp_init_version", "ucp_worker_create", "ucp_mem_map", "ucp_am_send_nbx", "ucp_worker_progress")))
+    partial = tmp_path / "libucp_partial.so"
+    subprocess.run([gcc, "-shared", "-fPIC", str(src), "-o", str(partial)], check=True)
+    r = _probe_in_subprocess(str(partial))
+    assert not r["available"] and r["version"] == [1, 20, 0]
+    assert r["have"] == [1, 1, 1, 1, 0, 1] and "ucp_am_recv_data_nbx" in r["message"]
+    src.write_text(src.read_text() + "int ucp_am_recv_data_nbx(void) { return -1; }\n")
+    whole = tmp_path / "libucp_whole.so"
+    subprocess.run([gcc, "-shared", "-fPIC", str(src), "-o", str(whole)], check=True)
+    r = _probe_in_subprocess(str(whole))
+    assert r["available"] == 1 and r["have"] == [1] * 6 and r["library"] == str(whole)
+    assert r["rc"] == capi.AXR_ERR_UNSUPPORTED and r["ctx"] is None
+    assert "ucp.h" in r["error"] and "UCX 1.20.0" in r["error"]

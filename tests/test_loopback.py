@@ -540,3 +540,17 @@ def test_memory_policy_with_tracked_numpy_arrays(pkg, gpu):
         bundle.payload.release()
     client.close()
     server.close()
+
+
+@pytest.mark.gpu
+def test_the_pytorch_rocm_example_runs(gpu):
+    """examples/pytorch_rocm_example.py: the reference's torch example (custom memory policy,
+    a + b) and its divide-by-two round trip known answer, on the GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, os.path.join(root, "examples", "pytorch_rocm_example.py")],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "pytorch_rocm_example ok" in out.stdout and "all elements == 3.0" in out.stdout
