@@ -16,6 +16,7 @@ from .dlpack import DLPackExport, TensorView, extract, extract_many
 from .loopback import AmMessage, LoopbackAmContext
 from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager
 from .pipeline import StreamedTransfer
+from .runtime import AxonRuntime
 from .transfer import (classify_argument, flatten_arguments, recv_arguments, recv_tensors, regroup,
                        send_arguments, send_tensors)
 

@@ -852,3 +852,63 @@ def test_ucx_backend_is_probed_and_refused_clearly(pkg, tmp_path):
     assert r["available"] == 1 and r["have"] == [1] * 6 and r["library"] == str(whole)
     assert r["rc"] == capi.AXR_ERR_UNSUPPORTED and r["ctx"] is None
     assert "ucp.h" in r["error"] and "UCX 1.20.0" in r["error"]
+
+
+def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
+    """The AxonRuntime-shaped entry (axon/python/src/bindings_runtime.cpp:700-830, 910-1016):
+    registration rules, in-process addresses, and a call whose arguments and result are plain
+    values only (no tensor, so no payload and no GPU work: the record travels as an eager
+    header-only message)."""
+    import asyncio
+    rt = pkg.runtime
+    with pytest.raises(ValueError):
+        pkg.AxonRuntime("")
+    server = pkg.AxonRuntime("cpu_server", device=pkg.cpu())
+    with pytest.raises(RuntimeError, match="not been started"):
+        server.get_local_address()
+    server.start()
+    assert server.register_function(lambda a, b="x": f"{a}:{b}", function_name="join") == 1
+    assert server.register_function(len, 7) == 7 and server.register_function(abs) == 2
+    with pytest.raises(RuntimeError, match="already registered"):
+        server.register_function(len, 9)               # name "len" taken
+    with pytest.raises(RuntimeError, match="already registered"):
+        server.register_function(max, 7)
+    with pytest.raises(TypeError):
+        server.register_function(3)
+    import json
+    assert json.loads(server.get_local_signatures()) == {"join": 1, "len": 7, "abs": 2}
+    client = pkg.AxonRuntime("cpu_client", device=pkg.cpu())
+    client.start_client()
+    assert server.get_local_address() != client.get_local_address()
+    assert server.get_local_address().startswith(b"axr-loopback\0cpu_server\0")
+
+    async def body():
+        with pytest.raises(RuntimeError, match="no worker at this address"):
+            await client.connect_endpoint_async(b"axr-loopback\0cpu_server\0" + bytes(16), "cpu_server")
+        await client.connect_endpoint_async(server.get_local_address(), "cpu_server")
+        kw = dict(worker_name="cpu_server", session_id=3, workflow_id=1)
+        assert await client.invoke(5, "y", function="join", **kw) == "5:y"
+        assert await client.invoke(-2.5, function=2, **kw) == 2.5
+        assert await client.invoke(None, function="join", **kw) == "None:x"
+        with pytest.raises(RuntimeError, match="not registered"):
+            await client.invoke(1, function="nobody", **kw)
+        with pytest.raises(RuntimeError, match="TypeError"):
+            await client.invoke(1, function=7, **kw)      # len(1) fails in the handler
+        with pytest.raises(RuntimeError, match="not serving"):
+            await server.connect_endpoint_async(client.get_local_address(), "cpu_client")
+            await server.invoke(1, worker_name="cpu_client", session_id=0, function=1)
+        with pytest.raises(TypeError):
+            await client.invoke(object(), function="join", **kw)
+    asyncio.run(body())
+    # the record framing
+    rec, rest = rt._unframe(rt._frame({"a": 1}, b"tail"))
+    assert rec == {"a": 1} and rest == b"tail"
+    with pytest.raises(RuntimeError):
+        rt._unframe(b"nope")
+    targs, slots = rt._split_arguments([1, [], "s", None, [[]]])
+    assert slots == [{"v": 1}, "t", {"v": "s"}, {"v": None}, "t"] and targs == [[], [[]]]
+    assert rt._merge_arguments(slots, ["A", "B"]) == [1, "A", "s", None, "B"]
+    client.stop()
+    server.stop()
+    with pytest.raises(RuntimeError, match="not been started"):
+        asyncio.run(client.invoke(1, worker_name="cpu_server", session_id=0, function=1))
