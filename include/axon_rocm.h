@@ -564,7 +564,8 @@ AXR_API int axr_am_recv_buffer_async(axr_am_context_t* ctx, uint64_t key, int ds
 AXR_API int axr_am_recv_buffer_iov(axr_am_context_t* ctx, uint64_t key, int dst_type,
                                    const axr_buffer_t* buffer_vec, size_t buffer_count,
                                    void* stream);
-/* Zero-copy fetch of a rendezvous payload: instead of copying, the receiver is handed the
+/* Zero-copy fetch of a rendezvous payload (in place of the ucp_am_recv_data_nbx of
+ * ucx_connection.cpp:376-399, which copies into the receiver's buffer): the receiver is handed the
  * sender's buffer (what a same-process rocm_ipc zero-copy rendezvous gives two endpoints
  * that share a device: UCX maps the sender's registered memory and the "receive" is a
  * pointer).  Only for a message whose payload is ONE contiguous buffer in memory the
@@ -579,7 +580,9 @@ AXR_API int axr_am_recv_buffer_borrow(axr_am_context_t* ctx, uint64_t key, void*
                                       int* memory_type);
 /* The receiver has enqueued its last read of a borrowed buffer on `stream`: the sender's
  * request completes when the work that `stream` holds now has run (no host wait).  Unknown
- * key -> AXR_ERR_NO_MESSAGE. */
+ * key -> AXR_ERR_NO_MESSAGE.  A receiving context that is destroyed with borrows not yet
+ * released completes those sends at once: drain whatever still reads the borrowed buffers
+ * before destroying the context. */
 AXR_API int axr_am_borrow_release(axr_am_context_t* ctx, uint64_t key, void* stream);
 /* Drop a message's host copies (and, for an unfetched rendezvous, complete the
  * sender's request as cancelled). */
