@@ -790,15 +790,20 @@ __device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* 
   typedef uint16_t __attribute__((aligned(1))) loose16;
   constexpr uint32_t R = kGroupMaxSlots / kWaveLanes;
   static_assert(R == 2, "two masks per group head");
-  uint32_t my_lo = 0, my_hi = 0, my_off_pad = 0, my_nb = 0;
-  if (lane < kGroupMaxMembers) {   // (records past the group's last member are zero)
-    const AXR_CONST Member* recs = reinterpret_cast<const AXR_CONST Member*>(head + 1);
-    const u32x4 r = *reinterpret_cast<const AXR_CONST u32x4*>(recs + lane);
-    my_lo = r.x;
-    my_hi = r.y;
-    my_off_pad = r.z;
-    my_nb = r.w;
+  {
+    // the block's address is the same in every lane: say so, and the head arrives by scalar load
+    const uint64_t a = reinterpret_cast<uint64_t>(head);
+    head = reinterpret_cast<const AXR_CONST GroupHead*>(
+        static_cast<uint64_t>(uniform(static_cast<uint32_t>(a))) |
+        static_cast<uint64_t>(uniform(static_cast<uint32_t>(a >> 32))) << 32);
   }
+  // Lane l holds member l % 16's record (only lanes 0..15 are ever asked for theirs).  Every lane
+  // loads, so that no branch stands between this load and the loads of the head: a load under a
+  // lane mask is waited for inside its branch, which put two memory round trips in a row here.
+  const AXR_CONST Member* recs = reinterpret_cast<const AXR_CONST Member*>(head + 1);
+  const u32x4 rec = *reinterpret_cast<const AXR_CONST u32x4*>(recs + (lane & (kGroupMaxMembers - 1u)));
+  asm volatile("" ::: "memory");   // the record load is issued before the head's loads are waited for
+  const uint32_t my_lo = rec.x, my_hi = rec.y, my_off_pad = rec.z, my_nb = rec.w;
   // member of slot s: the number of members that begin at or before s, minus one
   const uint64_t mask0 = head->starts[0], mask1 = head->starts[1];
   gbytes pay = payload + head->off;
