@@ -14,13 +14,15 @@ arguments of plain types (None, bool, int, float, str) travel in the request rec
 What it is not: the RPC runtime.  There is no dispatcher, no hybrid logical clock, no
 session or workflow bookkeeping, no thread pool and no network: peers are runtimes of the
 same process, found by the address ``get_local_address`` returns, and a request is served
-inside the ``invoke`` that sent it (handlers may be coroutines; they are awaited there).
+inside the ``invoke`` that sent it (handlers may be coroutines; they are awaited there; a
+serving runtime takes one request at a time, concurrent calls to it queue up).
 ``thread_pool_size``, ``timeout`` and ``lifecycle_policy`` are accepted and kept, nothing
 acts on them.  A handler's exception reaches the caller as ``RuntimeError``, an unknown
 function or worker likewise, as the reference reports them on the future.
 """
 from __future__ import annotations
 
+import asyncio
 import contextlib
 import inspect
 import json
@@ -112,7 +114,8 @@ class AxonRuntime:
         self._next_function_id = 1
         self._next_request_id = 1
         self._serving = False
-        self._pending_reply = None
+        self._serve_locks: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()   # one per event loop
+        self._stash: Dict[int, tuple] = {}      # replies taken off the queue by another call, by request id
 
     # ------------------------------------------------------------------ lifecycle
     def _activate(self):
@@ -140,6 +143,7 @@ class AxonRuntime:
         with _workers_mu:
             _workers.pop(self._address, None)
         self._peers.clear()
+        self._stash.clear()
         self._serving = False
         if self._ctx is not None:
             self._ctx.close()
@@ -249,8 +253,16 @@ class AxonRuntime:
             raise
         return _merge_arguments(record["slots"], regroup(structure, tensors))
 
-    async def _serve_one(self, back: int) -> None:
-        """Receive one request, run its function, send the reply on ``back``."""
+    def _serve_lock(self) -> asyncio.Lock:
+        loop = asyncio.get_running_loop()
+        lock = self._serve_locks.get(loop)
+        if lock is None:
+            lock = self._serve_locks[loop] = asyncio.Lock()
+        return lock
+
+    async def _serve_one(self, back: int):
+        """Receive one request, run its function, send the reply on ``back``; returns the
+        reply's send (request handle, bundle) for the caller to finish."""
         msg, record, rest = self._take()
         reply = {"kind": "reply", "id": record.get("id")}
         fn = self._lookup(record.get("function"))
@@ -265,9 +277,9 @@ class AxonRuntime:
                 if inspect.isawaitable(result):
                     result = await result
                 values = list(result) if isinstance(result, tuple) else [result]
-                self._pending_reply = self._send(back, dict(reply, tuple=isinstance(result, tuple)), values)
+                return self._send(back, dict(reply, tuple=isinstance(result, tuple)), values)
         except Exception as e:  # noqa: BLE001  (a handler's failure is the caller's RuntimeError)
-            self._pending_reply = self._send(back, dict(reply, kind="error", error=f"{type(e).__name__}: {e}"), [])
+            return self._send(back, dict(reply, kind="error", error=f"{type(e).__name__}: {e}"), [])
 
     def _lookup(self, function: Any) -> Optional[_Function]:
         if isinstance(function, int) and not isinstance(function, bool):
@@ -301,21 +313,31 @@ class AxonRuntime:
         request_id, self._next_request_id = self._next_request_id, self._next_request_id + 1
         record = {"kind": "request", "id": request_id, "function": function, "session": int(session_id),
                   "workflow": int(workflow_id)}
-        with self._activate():
-            sent = self._send(conn, record, list(args))
-        await peer._serve_one(back)
+        # one request at a time per serving runtime: the request is sent, served and answered
+        # under the server's lock, so the message the server takes is this one
+        async with peer._serve_lock():
+            with self._activate():
+                sent = self._send(conn, record, list(args))
+            pending = await peer._serve_one(back)
         try:
             with self._activate():
-                msg, reply, rest = self._take()
+                msg, reply, rest = self._take_reply(request_id)
                 failed = reply.get("kind") == "error"
                 self._finish(sent, tolerate_failure=failed)     # a refused request was never fetched
                 values = self._open(msg, reply, rest, memory_policy, from_dlpack_fn)
         finally:
-            pending, peer._pending_reply = peer._pending_reply, None
-            if pending is not None:
-                peer._finish(pending, tolerate_failure=True)
+            peer._finish(pending, tolerate_failure=True)
         if failed:
             raise RuntimeError(reply.get("error", "remote error"))
-        if reply.get("id") != request_id:
-            raise RuntimeError("reply does not belong to this request")
         return tuple(values) if reply.get("tuple") else values[0]
+
+    def _take_reply(self, request_id: int):
+        """The reply to ``request_id``: replies to other calls of this runtime that are still
+        suspended (calls to several servers run concurrently) are set aside for them."""
+        while True:
+            if request_id in self._stash:
+                return self._stash.pop(request_id)
+            msg, record, rest = self._take()
+            if record.get("id") == request_id:
+                return msg, record, rest
+            self._stash[record.get("id")] = (msg, record, rest)

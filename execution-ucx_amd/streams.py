@@ -22,13 +22,18 @@ from __future__ import annotations
 
 import ctypes as C
 import sys
+import threading
 from typing import Optional
 
 from . import _capi
 
 # (device, direction) -> event handle.  An event may be recorded again while an earlier wait
 # on it is still queued: a wait captures the record that was current when it was enqueued.
+# Record and wait are enqueued as a pair under a lock: the producer's stream is per thread
+# (torch's current stream is thread-local), and another thread's record between the two
+# would make this thread wait for the wrong stream.
 _events = {}
+_pair_lock = threading.Lock()
 
 
 def _event(device: int, direction: int) -> int:
@@ -57,9 +62,10 @@ def producer_stream() -> Optional[tuple]:
 
 def _order(later: Optional[int], earlier: Optional[int], device: int, direction: int) -> None:
     lib = _capi.load()
-    ev = _event(device, direction)
-    _capi.check(lib.axr_event_record(ev, earlier or None))
-    _capi.check(lib.axr_stream_wait_event(later or None, ev))
+    with _pair_lock:
+        ev = _event(device, direction)
+        _capi.check(lib.axr_event_record(ev, earlier or None))
+        _capi.check(lib.axr_stream_wait_event(later or None, ev))
 
 
 def order_behind_producers(stream: Optional[int]) -> bool:

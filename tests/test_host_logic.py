@@ -912,3 +912,42 @@ def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
     server.stop()
     with pytest.raises(RuntimeError, match="not been started"):
         asyncio.run(client.invoke(1, worker_name="cpu_server", session_id=0, function=1))
+
+
+def test_runtime_concurrent_calls_keep_their_replies(pkg):
+    """Calls that overlap in one event loop: two clients on one server (served one at a time)
+    and one client on two servers whose handlers finish in the opposite order."""
+    import asyncio
+    order = []
+
+    async def slow(tag, delay):
+        order.append(("in", tag))
+        await asyncio.sleep(delay)
+        order.append(("out", tag))
+        return f"done {tag}"
+
+    async def body():
+        s1, s2 = pkg.AxonRuntime("srv1", device=pkg.cpu()), pkg.AxonRuntime("srv2", device=pkg.cpu())
+        c1, c2 = pkg.AxonRuntime("cli1", device=pkg.cpu()), pkg.AxonRuntime("cli2", device=pkg.cpu())
+        for s in (s1, s2):
+            s.start()
+            s.register_function(slow, 1)
+        for c in (c1, c2):
+            c.start_client()
+            await c.connect_endpoint_async(s1.get_local_address(), "srv1")
+            await c.connect_endpoint_async(s2.get_local_address(), "srv2")
+        kw = dict(session_id=0, function=1)
+        # two clients, one server: the second request waits for the first reply
+        r = await asyncio.gather(c1.invoke("a", 0.05, worker_name="srv1", **kw),
+                                 c2.invoke("b", 0.0, worker_name="srv1", **kw))
+        assert r == ["done a", "done b"]
+        assert order == [("in", "a"), ("out", "a"), ("in", "b"), ("out", "b")]
+        order.clear()
+        # one client, two servers: the slower server's reply arrives second, each call gets its own
+        r = await asyncio.gather(c1.invoke("x", 0.05, worker_name="srv1", **kw),
+                                 c1.invoke("y", 0.0, worker_name="srv2", **kw))
+        assert r == ["done x", "done y"]
+        assert order == [("in", "x"), ("in", "y"), ("out", "y"), ("out", "x")]
+        for rt in (c1, c2, s1, s2):
+            rt.stop()
+    asyncio.run(body())
