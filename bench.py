@@ -987,6 +987,10 @@ def small_segments(h, tensors=65536, lo=8, hi=512, copies=4, steps=400):
         r["pack_bytes_moved_vs_plain_copy"] = round(r["pack_only"]["GBps_bytes_moved"] /
                                                     out["plain_copy_same_bytes"]["GBps_2n"], 3)
         r["unpack_vs_plain_copy"] = round(r["unpack_only"]["GBps_2P"] / out["plain_copy_same_bytes"]["GBps_2n"], 3)
+    # a bundle seen for the first time: plan -> pack -> sync -> header decode + bind -> unpack -> sync
+    # (the group tables are built on the host; nothing is reused between repetitions)
+    fresh = end_to_end_us(h, spec, steps=10)
+    out["fresh_bundle"] = {k: round(v, 2) for k, v in fresh.items()}
     return out
 
 
