@@ -274,9 +274,10 @@ class AxonRuntime:
             with self._activate():
                 args = self._open(msg, record, rest, fn.memory_policy, fn.from_dlpack_fn)
                 result = fn.callable(*args)
-                if inspect.isawaitable(result):
-                    result = await result
-                values = list(result) if isinstance(result, tuple) else [result]
+            if inspect.isawaitable(result):     # awaited outside the activation: the device that is
+                result = await result           # current on this thread is not held across a suspension
+            values = list(result) if isinstance(result, tuple) else [result]
+            with self._activate():
                 return self._send(back, dict(reply, tuple=isinstance(result, tuple)), values)
         except Exception as e:  # noqa: BLE001  (a handler's failure is the caller's RuntimeError)
             return self._send(back, dict(reply, kind="error", error=f"{type(e).__name__}: {e}"), [])
