@@ -180,3 +180,41 @@ def test_grouped_plans_in_submit_with_deltas_and_without_allocation(pkg, orc, gp
     capi.check(lib.axr_pack_noalloc(plan_a._h, out.data_ptr(), n, None))
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy()[:n], orc.pack(chunks_a, 16))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_mixtures_of_short_long_strided_and_empty_tensors(pkg, orc, gpu, seed):
+    """Group tiles next to ordinary and strided segments in random order: short (1-1099 B),
+    long (1.1-40 KB), pitched 2-D views and empty tensors at odd offsets, a random alignment
+    and a shifted payload base; pack against the oracle, unpack into fresh tensors."""
+    import torch
+    rng = np.random.default_rng(10_000 + seed)
+    tensors, chunks = [], []
+    for k in rng.integers(0, 10, size=int(rng.integers(50, 400))):
+        if k < 8:
+            nb = int(rng.integers(1, 1100)) if k < 6 else int(rng.integers(1100, 40000))
+            raw = torch.from_numpy(rng.integers(0, 256, size=nb + 32, dtype=np.uint8)).to(gpu)
+            o = int(rng.integers(0, 32))
+            t = raw[o:o + nb]
+        elif k == 8:
+            rows, cols, pitch = int(rng.integers(1, 20)), int(rng.integers(1, 3000)), 3100
+            raw = torch.from_numpy(rng.integers(0, 256, size=rows * pitch, dtype=np.uint8)).to(gpu)
+            t = raw.reshape(rows, pitch)[:, :cols]
+        else:
+            t = torch.empty(0, dtype=torch.uint8, device=gpu)
+        tensors.append(t)
+        chunks.append(t.contiguous().reshape(-1).cpu().numpy())
+    align = int(rng.choice([1, 2, 16, 64, 256, 1024]))
+    shift = int(rng.integers(0, 16))
+    got, plan, buf = pack_checked(pkg, tensors, align, gpu, shift=shift)
+    assert np.array_equal(got, orc.pack(chunks, align))
+    outs = [torch.full_like(t, 0xEE) if t.is_contiguous() else
+            torch.full((t.shape[0], 3100), 0xEE, dtype=torch.uint8, device=gpu)[:, :t.shape[1]] for t in tensors]
+    rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+    torch.cuda.synchronize()
+    rplan.unpack(buf.data_ptr() + shift, plan.payload_bytes)
+    torch.cuda.synchronize()
+    for o, c in zip(outs, chunks):
+        assert np.array_equal(o.contiguous().reshape(-1).cpu().numpy(), c)
+    rplan.close()
+    plan.close()
