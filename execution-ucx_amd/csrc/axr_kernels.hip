@@ -807,7 +807,6 @@ __device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* 
   // member of slot s: the number of members that begin at or before s, minus one
   const uint64_t mask0 = head->starts[0], mask1 = head->starts[1];
   gbytes pay = payload + head->off;
-  const uint32_t slots = head->slots;
   uint32_t m[R];
   {
     const uint32_t lo0 = static_cast<uint32_t>(mask0), hi0 = static_cast<uint32_t>(mask0 >> 32);
@@ -828,8 +827,15 @@ __device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* 
     f_off_pad[r] = lane_value(from, my_off_pad);
     f_nb[r] = lane_value(from, my_nb);
   }
+  // What slot s of a member does, without branches.  With k16 = 16 * (s - first slot of the
+  // member) and nd = the bytes its data slots span (n rounded up to 16, at least 16):
+  //   k16 < nd           a data slot: bytes [min(k16, n - 16), +16) of a member of 16 bytes or
+  //                      more (the last slot overlaps its neighbour), the pieces of a shorter one;
+  //   nd <= k16 < nd + pad, pad >= 16   (pack) a zero slot: gap bytes [min(k16 - nd, pad - 16), +16);
+  //   anything else      nothing - which covers the slots past the group's last one: they map to
+  //                      the last member with k16 beyond its data and zero slots.
   gbytes ten[R], pp[R];
-  uint32_t kind[R];      // 0 nothing, 1 sixteen data bytes, 2 sixteen zero bytes (pack)
+  bool data16[R], zero16[R];
   uint32_t small_n[R];   // a member shorter than 16 bytes: its length, in the lane of its only data slot
   uint32_t small_pad[R]; // a gap shorter than 16 bytes, in the lane of the member's last data slot
   gbytes gap_at[R], small_pp[R];
@@ -838,34 +844,23 @@ __device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* 
     const uint32_t s = r * kWaveLanes + lane;
     const uint64_t ptr = (static_cast<uint64_t>(f_hi[r]) << 32 | f_lo[r]) + delta;
     const uint32_t off_pad = f_off_pad[r], nb = f_nb[r];
-    const uint32_t n = nb & 0xffffu, k = s - (nb >> 16);
+    const uint32_t n = nb & 0xffffu, k16 = (s - (nb >> 16)) << 4;
     const uint32_t rel = off_pad & ((1u << kMemberOffBits) - 1u), pad = off_pad >> kMemberOffBits;
-    const uint32_t dslots = group_data_slots(n), pslots = group_pad_slots(pad);
-    const bool live = s < slots;
+    const bool big = n >= kVecBytes;
+    const uint32_t nd = big ? (n + kVecBytes - 1u) & ~(kVecBytes - 1u) : kVecBytes;
+    const bool is_data = k16 < nd;
+    const uint32_t zb = k16 - nd;
+    data16[r] = is_data && big;
+    zero16[r] = PACK && pad >= kVecBytes && zb < pad;
+    small_n[r] = (is_data && !big) ? n : 0u;
+    small_pad[r] = (PACK && k16 + kVecBytes == nd && pad < kVecBytes) ? pad : 0u;
+    const uint32_t o = data16[r] ? (k16 < n - kVecBytes ? k16 : n - kVecBytes) : 0u;
+    const uint32_t oz = zero16[r] ? n + (zb < pad - kVecBytes ? zb : pad - kVecBytes) : o;
     gbytes t0 = as_global(ptr), p0 = pay + rel;
-    kind[r] = 0;
-    small_n[r] = 0;
-    small_pad[r] = 0;
-    ten[r] = t0;
-    pp[r] = p0;
-    gap_at[r] = p0;
+    ten[r] = t0 + o;
+    pp[r] = p0 + oz;
     small_pp[r] = p0;
-    if (live && k < dslots) {
-      if (n >= kVecBytes) {
-        const uint32_t o = (k + 1u == dslots) ? n - kVecBytes : k * kVecBytes;
-        ten[r] = t0 + o;
-        pp[r] = p0 + o;
-        kind[r] = 1;
-      } else {
-        small_n[r] = n;
-      }
-      if (PACK && k + 1u == dslots && pad && pad < kVecBytes) small_pad[r] = pad;
-    } else if (PACK && live && k < dslots + pslots) {
-      const uint32_t j = k - dslots;
-      pp[r] = p0 + n + ((j + 1u == pslots) ? pad - kVecBytes : j * kVecBytes);
-      kind[r] = 2;
-    }
-    if (PACK && small_pad[r]) gap_at[r] = p0 + n;   // where the short gap begins (payload side)
+    gap_at[r] = p0 + n;   // where a short gap begins (payload side)
   }
   // Ordinary (cacheable) accesses on both sides whatever the launch's hints: short tensors
   // share their 128-byte lines with their neighbours, and a line marked as streaming is fetched
@@ -884,7 +879,7 @@ __device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* 
 #pragma unroll
   for (uint32_t r = 0; r < R; ++r) {
     v[r] = u32x4{0u, 0u, 0u, 0u};
-    if (kind[r] == 1) v[r] = load16<false>(PACK ? ten[r] : pp[r]);
+    if (data16[r]) v[r] = load16<false>(PACK ? ten[r] : pp[r]);
   }
   if (wave_has_small) {
 #pragma unroll
@@ -905,8 +900,8 @@ __device__ __attribute__((noinline)) void group_tile(const AXR_CONST GroupHead* 
   for (uint32_t r = 0; r < R; ++r) asm volatile("" : "+v"(v[r])::"memory");
 #pragma unroll
   for (uint32_t r = 0; r < R; ++r) {
-    if (kind[r] == 1) store16<false>(PACK ? pp[r] : ten[r], v[r]);
-    else if (kind[r] == 2) store16<false>(pp[r], v[r]);
+    if (data16[r]) store16<false>(PACK ? pp[r] : ten[r], v[r]);
+    else if (PACK && zero16[r]) store16<false>(pp[r], v[r]);
   }
   if (wave_has_small) {
 #pragma unroll
