@@ -779,6 +779,20 @@ struct Builder {
 
 int build_tables(axr_plan* p);
 
+// A payload that streams to and from memory (larger than payload_cache_bytes, so written and
+// read with non-temporal accesses) moves fastest in tiles of 1 KiB, one load and one store per
+// lane, in workgroups of a single wavefront: the 1 GiB cache-block gather 6.02 -> 6.29 TB/s
+// (pack 6.26 -> 6.51, unpack 5.80 -> 6.09), 1 GiB of pitched rows of 4-64 KiB 6.24-6.40 ->
+// 6.59-6.61, the 405 MB layer bundle 6.43 -> 6.52.  Either change alone is slower than the
+// 2 KiB tiles in workgroups of two wavefronts it replaces, and payloads that stay in the
+// last-level cache lose 7-24 % with it (48 MB mixed bundle, 256 MiB chunk of pitched rows).
+// Up to max_tiles tiles, i.e. 1 GiB.
+bool streams_in_small_tiles(const axr_plan* p) {
+  const Tunables& tn = tunables();
+  return p->payload_bytes > static_cast<uint64_t>(tn.payload_cache_bytes) &&
+         (p->payload_bytes >> 10) <= static_cast<uint64_t>(tn.max_tiles);
+}
+
 // Launch geometry of a bundle of p->ntiles tiles in nseg segments: one tile per wave until
 // the grid would exceed max_waves, workgroup size, cache hints, and the size of the blocks of
 // the tile-block index (about one segment each, a power of two up to 256 tiles: a bundle of
@@ -788,7 +802,8 @@ void finish_geometry(axr_plan* p, uint32_t rows, size_t nseg, bool may_be_direct
   uint64_t tpw = (p->ntiles + static_cast<uint64_t>(tn.max_waves) - 1) /
                  static_cast<uint64_t>(tn.max_waves);
   if (tpw == 0) tpw = 1;
-  p->cfg.threads = tn.threads ? static_cast<uint32_t>(tn.threads) : (p->ntiles < 65536 ? 256u : 128u);
+  p->cfg.threads = tn.threads ? static_cast<uint32_t>(tn.threads)
+                              : (rows == 1 && tn.tile_rows == 0 ? kWaveLanes : (p->ntiles < 65536 ? 256u : 128u));
   p->cfg.elements = false;
   for (const Dims& dm : p->dims) p->cfg.elements = p->cfg.elements || dm.mode != kModeRunTiles;
   if (p->cfg.elements) p->cfg.threads = std::min(p->cfg.threads, kMaxElementThreads);
@@ -826,6 +841,7 @@ uint32_t rows_for_compact_bundle(const axr_plan* p) {
   const Tunables& tn = tunables();
   uint32_t rows = static_cast<uint32_t>(tn.tile_rows);
   if (rows) return rows;
+  if (streams_in_small_tiles(p)) return 1;
   rows = 2;
   while (rows < kMaxTileRows &&
          p->payload_bytes / (static_cast<uint64_t>(rows) * kRowBytes) > static_cast<uint64_t>(tn.max_tiles))
@@ -990,6 +1006,21 @@ int build_tables(axr_plan* p) {
     if (uniform_runs && common_run >= 2 * kRowBytes && common_run <= kMaxTileRows * kRowBytes &&
         p->payload_bytes <= static_cast<uint64_t>(tn.payload_cache_bytes)) {
       while (rows < kMaxTileRows && rows * kRowBytes < common_run) rows *= 2;
+    }
+    if (streams_in_small_tiles(p)) {
+      // only for bundles of compact tensors and strided views that move as run tiles
+      bool run_tiles_only = true;
+      for (const TensorRec& t : p->tensors) {
+        if (t.nbytes == 0 || !t.has_strides) continue;
+        const uint64_t item = (static_cast<uint64_t>(t.bits) + 7) / 8;
+        Collapsed c;
+        collapse(t, p->shape_of(t), p->strides_of(t), item, &c);
+        if (c.nd != 0 && c.run_bytes < static_cast<uint64_t>(tn.gather_run_bytes)) {
+          run_tiles_only = false;
+          break;
+        }
+      }
+      if (run_tiles_only) rows = 1;
     }
     while (rows < kMaxTileRows &&
            p->payload_bytes / (static_cast<uint64_t>(rows) * kRowBytes) >
