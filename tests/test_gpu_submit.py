@@ -397,3 +397,51 @@ def test_many_small_bundles_in_one_call(pkg, orc, gpu):
     finally:
         for p in plans + rplans:
             p.close()
+
+
+@pytest.mark.parametrize("device_tables", [1, 0])
+def test_streaming_geometry_for_payloads_beyond_the_cache(pkg, gpu, device_tables):
+    """A payload between 256 MiB and 1 GiB moves in 1 KiB tiles, one wavefront per workgroup
+    (tables built on the device and on the host).  6000 contiguous tensors of odd lengths around
+    64 KiB at odd addresses, tight layout: the packed bytes are the tensors' concatenation,
+    compared on the device, and an unpack into fresh memory gives the tensors back with the
+    bytes between them untouched."""
+    import torch
+    rng = np.random.default_rng(12)
+    sizes = rng.integers(50_000, 80_000, size=6000)
+    gaps = rng.integers(0, 100, size=6000)
+    total = int(sizes.sum() + gaps.sum()) + 64
+    g = torch.Generator(device=gpu)
+    g.manual_seed(7)
+    arena = torch.randint(0, 256, (total,), dtype=torch.uint8, device=gpu, generator=g)
+    views, at = [], 3
+    for n, gap in zip(sizes, gaps):
+        at += int(gap)
+        views.append(arena[at:at + int(n)])
+        at += int(n)
+    before = C.c_int64()
+    pkg._capi.check(pkg._capi.load().axr_tune_get(b"device_tables", C.byref(before)))
+    pkg.tune(device_tables=device_tables)
+    try:
+        plan = pkg.BundlePlan.create(views, align=1)
+        n = plan.payload_bytes
+        assert (256 << 20) < n <= (1 << 30) and n == int(sizes.sum())
+        buf = torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu)
+        plan.pack(buf.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+        info = plan.launch_info()
+        assert info["tile_bytes"] == 1024 and info["threads_per_workgroup"] == 64
+        assert torch.equal(buf[:n], torch.cat(views)) and bool((buf[n:] == POISON).all())
+        out_arena = torch.full_like(arena, POISON)
+        outs = [out_arena[v.data_ptr() - arena.data_ptr():][:v.numel()] for v in views]
+        rplan = pkg.BundlePlan.from_header(plan.header).bind(outs)
+        rplan.unpack(buf.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+        assert rplan.launch_info()["tile_bytes"] == 1024
+        mask = torch.zeros(total, dtype=torch.bool, device=gpu)
+        for v in views:
+            o = v.data_ptr() - arena.data_ptr()
+            mask[o:o + v.numel()] = True
+        assert torch.equal(out_arena[mask], arena[mask]) and bool((out_arena[~mask] == POISON).all())
+        rplan.close()
+        plan.close()
+    finally:
+        pkg.tune(device_tables=before.value)
