@@ -1087,7 +1087,14 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   // jobs reads one entry beyond its own)
   uint32_t j = 0;
   const uint32_t count = jt->count;
-  for (uint32_t k = 1; k < count && wg >= jt->job[k].wg_begin; ++k) j = k;
+  uint32_t local_wg;
+  if (jt->interleaved) {   // jobs of equal grids take the workgroups in turn
+    j = wg % count;
+    local_wg = wg / count;
+  } else {
+    for (uint32_t k = 1; k < count && wg >= jt->job[k].wg_begin; ++k) j = k;
+    local_wg = wg - jt->job[j].wg_begin;
+  }
   const AXR_CONST JobDesc* d = &jt->job[j];
   KernelArgs a;
   a.ntiles = d->ntiles;
@@ -1099,7 +1106,7 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   dims_table dims = reinterpret_cast<dims_table>(d->dims);
   const AXR_CONST uint32_t* wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(d->wave_seg);
   gbytes payload = reinterpret_cast<gbytes>(d->payload);
-  const uint32_t local = wg - d->wg_begin;
+  const uint32_t local = local_wg;
   if (d->unpack) {   // workgroup-uniform
     bundle_body<false, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, jt->lds_per_wave,
                                                  jt->nt_bits);

@@ -2016,6 +2016,12 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
       cfg.lds_per_wave = std::max(cfg.lds_per_wave, p->cfg.lds_per_wave);
     }
     table.count = static_cast<uint32_t>(end - i);
+    const int64_t interleave = tunables().submit_interleave;
+    if (interleave > 0 || (interleave < 0 && (cfg.nontemporal & 2u) != 0)) {
+      bool equal = true;
+      for (size_t k = i; k < end; ++k) equal = equal && jobs[k].plan->cfg.workgroups == first->cfg.workgroups;
+      table.interleaved = equal ? 1u : 0u;
+    }
     table.lds_per_wave = cfg.lds_per_wave;
     table.nt_bits = cfg.nontemporal;
     cfg.workgroups = wg;

@@ -497,6 +497,8 @@ static int tune_set_body(const char* key, int64_t value) {
   } else if (k == "transfer_fail_after_send") {
     if (value < 0) return fail(AXR_ERR_INVALID, "transfer_fail_after_send must not be negative");
     t.transfer_fail_after_send = value;
+  } else if (k == "submit_interleave") {
+    t.submit_interleave = value;
   } else if (k == "group_slots") {
     if (value != 64 && value != 128) return fail(AXR_ERR_INVALID, "group_slots must be 64 or 128");
     t.group_slots = value;
@@ -540,6 +542,7 @@ static int tune_get_body(const char* key, int64_t* value) {
   else if (k == "device_tables") *value = t.device_tables;
   else if (k == "group_bytes") *value = t.group_bytes;
   else if (k == "group_slots") *value = t.group_slots;
+  else if (k == "submit_interleave") *value = t.submit_interleave;
   else if (k == "transfer_fail_after_send") *value = t.transfer_fail_after_send;
   else return fail(AXR_ERR_INVALID, "unknown tunable: " + k);
   return AXR_OK;

@@ -421,8 +421,13 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
                               size_t* count);
 
 /* Tuning knobs (process-wide, read when a plan builds its device tables):
- * "tile_rows" (KiB per wavefront tile: 0 auto, 1, 2, 4, 8, 16), "max_tiles",
- * "max_waves", "threads" (workgroup size), "nontemporal" (-1 auto, or bit 0
+ * "tile_rows" (KiB per wavefront tile: 1, 2, 4, 8, 16, or 0 = automatic: 2; a whole run of up
+ * to 16 KiB for bundles of strided views of one run length whose payload stays in the
+ * last-level cache; 1 for payloads of compact tensors and long strided runs between
+ * payload_cache_bytes and max_tiles KiB, which stream to and from memory), "max_tiles",
+ * "max_waves", "threads" (workgroup size; 0 = automatic: 256 below 65,536 tiles, 128 above, 64
+ * with the automatic 1 KiB tiles and for short strided rows that are no multiple of 16
+ * bytes), "nontemporal" (-1 auto, or bit 0
  * tensor side / bit 1 payload side), "payload_cache_bytes", "gather_run_bytes",
  * "xcd_remap" (each accelerator die walks one contiguous share of the tiles: 1 always,
  * 0 never, -1 (default) for bundles made mostly of transposed views whose rows do not
@@ -454,9 +459,12 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * "loopback_copy_kernel" (1, default: the loopback context moves a device payload
  * to device memory with the library's copy kernel; 0: with hipMemcpyAsync),
  * "group_bytes" (contiguous device tensors of at most this many bytes that follow each
- * other in the bundle share wavefronts: up to 64 tensors or 128 sixteen-byte lane slots
+ * other in the bundle share wavefronts: up to 16 tensors or 128 sixteen-byte lane slots
  * per wavefront, so that wavefronts and table bytes scale with the payload and not with
  * the tensor count; default 512, at most 1023, 0: every tensor gets wavefronts of its own),
+ * "submit_interleave" (jobs of one axr_submit launch whose grids are equal take the
+ * workgroups in turn instead of one range each: 1 always, 0 never, -1, the default, when the
+ * payloads stream; read at every axr_submit),
  * "transfer_fail_after_send" (failure injection for tests: N > 0 makes the N-th chunk that
  * axr_transfer_submit is given from now on fail with AXR_ERR_MISMATCH after its send has been
  * queued, as if the message that arrived did not match the receiver's plan; 0, the default: off),
