@@ -165,7 +165,7 @@ struct JobDesc {              // 64 bytes
 static_assert(sizeof(JobDesc) == 64, "JobDesc layout");
 struct alignas(16) JobTable {
   uint32_t count, lds_per_wave, nt_bits;
-  uint32_t interleaved;       // 1: job = workgroup % count, local workgroup = workgroup / count (equal grids)
+  uint32_t interleaved;       // 1: two jobs of equal grids, job = workgroup & 1, local workgroup = workgroup >> 1
   JobDesc job[kMaxJobs];
 };
 
@@ -243,12 +243,12 @@ struct Tunables {
   // tensor gets its own wavefronts.
   std::atomic<int64_t> group_bytes{512};
   std::atomic<int64_t> group_slots{kGroupMaxSlots};   // lane slots per group tile: 64 or 128
-  // Jobs of one axr_submit launch whose grids are equal take the workgroups in turn (job = workgroup
-  // % jobs) instead of one range each: 1 always, 0 never, -1 when the payloads stream.  With a pack
-  // and an unpack in one launch the memory then sees reads and writes of both throughout: the
+  // The two jobs of an axr_submit launch whose grids are equal and whose payloads stream take the
+  // workgroups in turn (even / odd) instead of one range each (1, the default; 0: never).  With a
+  // pack and an unpack in one launch the memory then sees reads and writes of both throughout: the
   // 405 MB layer bundle 6.50 -> 6.65 TB/s.  Payloads kept in the last-level cache are better off
-  // with the pack's range first (48 MB mixed bundle: 6.18 against 6.11 TB/s).
-  std::atomic<int64_t> submit_interleave{-1};
+  // with the pack's range first (48 MB mixed bundle: 6.18 against 6.11 TB/s) and never interleave.
+  std::atomic<int64_t> submit_interleave{1};
   // Failure injection for tests of the streamed transfer's error handling: N > 0 makes the
   // N-th chunk submitted from now on fail after its send has been queued, as if the message
   // that arrived did not match the receiver's plan (and counts down to 0 = off).

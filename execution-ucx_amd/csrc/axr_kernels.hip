@@ -1087,13 +1087,16 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   // jobs reads one entry beyond its own)
   uint32_t j = 0;
   const uint32_t count = jt->count;
-  uint32_t local_wg;
-  if (jt->interleaved) {   // jobs of equal grids take the workgroups in turn
-    j = wg % count;
-    local_wg = wg / count;
-  } else {
-    for (uint32_t k = 1; k < count && wg >= jt->job[k].wg_begin; ++k) j = k;
-    local_wg = wg - jt->job[j].wg_begin;
+  for (uint32_t k = 1; k < count && wg >= jt->job[k].wg_begin; ++k) j = k;
+  uint32_t local_wg = wg - jt->job[j].wg_begin;
+  if constexpr (NTP) {
+    // Streaming payloads only (these instantiations): two jobs of equal grids take the
+    // workgroups in turn.  Kept out of the other instantiations, where the extra test cost the
+    // 48 MB bundle 0.7 % per launch.
+    if (jt->interleaved) {
+      j = wg & 1u;
+      local_wg = wg >> 1;
+    }
   }
   const AXR_CONST JobDesc* d = &jt->job[j];
   KernelArgs a;

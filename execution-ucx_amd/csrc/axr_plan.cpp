@@ -2017,10 +2017,9 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     }
     table.count = static_cast<uint32_t>(end - i);
     const int64_t interleave = tunables().submit_interleave;
-    if (interleave > 0 || (interleave < 0 && (cfg.nontemporal & 2u) != 0)) {
-      bool equal = true;
-      for (size_t k = i; k < end; ++k) equal = equal && jobs[k].plan->cfg.workgroups == first->cfg.workgroups;
-      table.interleaved = equal ? 1u : 0u;
+    if (interleave != 0 && (cfg.nontemporal & 2u) != 0) {   // the streaming instantiations carry the code
+      // (two jobs: a shift and a mask in the kernel)
+      table.interleaved = (end - i == 2 && jobs[i + 1].plan->cfg.workgroups == first->cfg.workgroups) ? 1u : 0u;
     }
     table.lds_per_wave = cfg.lds_per_wave;
     table.nt_bits = cfg.nontemporal;

@@ -448,42 +448,42 @@ def test_streaming_geometry_for_payloads_beyond_the_cache(pkg, gpu, device_table
 
 
 @pytest.mark.parametrize("interleave", [1, 0])
-def test_jobs_of_equal_grids_take_workgroups_in_turn(pkg, orc, gpu, interleave):
-    """Three bundles of one geometry (the same sizes at other addresses) in one launch: the
-    pack of two and the unpack of a third, with the jobs' workgroups interleaved
-    ("submit_interleave", what a launch of streaming payloads does by itself) and in one
-    range each; the same bytes either way."""
+def test_two_jobs_of_equal_grids_take_workgroups_in_turn(pkg, orc, gpu, interleave):
+    """Two bundles of one geometry (the same sizes at other addresses) in one launch: the pack
+    of one and the unpack of the other, payloads streaming, with the jobs' workgroups
+    interleaved ("submit_interleave", the default for such a launch) and in one range each;
+    the same bytes either way."""
     import torch
     lib, capi = pkg._capi.load(), pkg._capi
     rng = np.random.default_rng(77)
     sizes = [int(x) for x in np.exp(rng.uniform(np.log(16), np.log(90000), size=500))]
     sets = []
-    for _ in range(3):
+    for _ in range(2):
         sets.append([torch.from_numpy(rng.integers(0, 256, size=n, dtype=np.uint8)).to(gpu) for n in sizes])
     plans = [pkg.BundlePlan.create(s, align=256) for s in sets]
     n = plans[0].payload_bytes
     assert len({p.launch_info()["workgroups"] for p in plans}) == 1
-    bufs = [torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu) for _ in range(3)]
-    wants = [orc.pack([chunk_of(t) for t in s], 256) for s in sets]
-    # the third bundle's payload is packed first, on its own, and unpacked inside the joint launch
-    plans[2].pack(bufs[2].data_ptr(), n)
-    outs = [torch.zeros_like(t) for t in sets[2]]
-    rplan = pkg.BundlePlan.from_header(plans[2].header).bind(outs)
+    bufs = [torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu) for _ in range(2)]
+    want = orc.pack([chunk_of(t) for t in sets[0]], 256)
+    # the second bundle's payload is packed first, on its own, and unpacked inside the joint launch
+    plans[1].pack(bufs[1].data_ptr(), n)
+    outs = [torch.zeros_like(t) for t in sets[1]]
+    rplan = pkg.BundlePlan.from_header(plans[1].header).bind(outs)
     torch.cuda.synchronize()
     before = C.c_int64()
     capi.check(lib.axr_tune_get(b"submit_interleave", C.byref(before)))
     pkg.tune(submit_interleave=interleave)
     try:
-        arr = job_array(capi, [(plans[0], 0, bufs[0].data_ptr(), n, 0), (rplan, 1, bufs[2].data_ptr(), n, 0),
-                               (plans[1], 0, bufs[1].data_ptr(), n, 0)])
-        capi.check(lib.axr_submit(arr, 3, None))
+        arr = job_array(capi, [(plans[0], 0, bufs[0].data_ptr(), n, 0), (rplan, 1, bufs[1].data_ptr(), n, 0)])
+        for k in range(2):          # interleaving is for payloads that stream: ask for that treatment
+            arr[k].flags = capi.JOB_PAYLOAD_STREAMING
+        capi.check(lib.axr_submit(arr, 2, None))
         torch.cuda.synchronize()
     finally:
         pkg.tune(submit_interleave=before.value)
-    for k in (0, 1):
-        got = bufs[k].cpu().numpy()
-        assert np.array_equal(got[:n], wants[k]) and (got[n:] == POISON).all()
-    for o, t in zip(outs, sets[2]):
+    got = bufs[0].cpu().numpy()
+    assert np.array_equal(got[:n], want) and (got[n:] == POISON).all()
+    for o, t in zip(outs, sets[1]):
         assert torch.equal(o, t)
     for p in plans + [rplan]:
         p.close()
