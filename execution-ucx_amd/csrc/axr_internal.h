@@ -166,6 +166,10 @@ static_assert(sizeof(JobDesc) == 64, "JobDesc layout");
 struct alignas(16) JobTable {
   uint32_t count, lds_per_wave, nt_bits;
   uint32_t interleaved;       // 1: two jobs of equal grids, job = workgroup & 1, local workgroup = workgroup >> 1
+  // first workgroup of every job once more, side by side (0xffffffff past the last job): a workgroup
+  // finds its job by comparing with all of them after ONE scalar load, instead of walking the
+  // descriptors with a dependent load per step
+  uint32_t begins[kMaxJobs];
   JobDesc job[kMaxJobs];
 };
 

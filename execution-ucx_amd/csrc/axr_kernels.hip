@@ -1083,22 +1083,21 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   const AXR_CONST JobTable* jt =
       (const AXR_CONST JobTable*)__builtin_amdgcn_kernarg_segment_ptr();
   const uint32_t wg = blockIdx.x;
-  // the job whose workgroup range holds this workgroup (the ranges ascend; a launch of two
-  // jobs reads one entry beyond its own)
+  // the job whose workgroup range holds this workgroup: the ranges ascend, so it is the number of
+  // ranges that begin at or below this workgroup (entries past the last job hold 0xffffffff)
   uint32_t j = 0;
-  const uint32_t count = jt->count;
-  for (uint32_t k = 1; k < count && wg >= jt->job[k].wg_begin; ++k) j = k;
-  uint32_t local_wg = wg - jt->job[j].wg_begin;
+#pragma unroll
+  for (uint32_t k = 1; k < kMaxJobs; ++k) j += wg >= jt->begins[k] ? 1u : 0u;
+  bool in_turn = false;
   if constexpr (NTP) {
     // Streaming payloads only (these instantiations): two jobs of equal grids take the
     // workgroups in turn.  Kept out of the other instantiations, where the extra test cost the
     // 48 MB bundle 0.7 % per launch.
-    if (jt->interleaved) {
-      j = wg & 1u;
-      local_wg = wg >> 1;
-    }
+    in_turn = jt->interleaved != 0;
+    if (in_turn) j = wg & 1u;
   }
   const AXR_CONST JobDesc* d = &jt->job[j];
+  const uint32_t local_wg = in_turn ? wg >> 1 : wg - d->wg_begin;
   KernelArgs a;
   a.ntiles = d->ntiles;
   a.tiles_per_wave = d->tiles_per_wave;
