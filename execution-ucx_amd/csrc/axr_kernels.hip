@@ -950,7 +950,12 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
     // contiguous share of the index space so neighbouring tiles share an L2
     wg = (wg % kXcds) * a.xcd_remap + wg / kXcds;
   }
-  const uint32_t wave = uniform(wg * (blockDim.x >> 6) + (threadIdx.x >> 6));
+  // wavefronts per workgroup travel in bits 8-15 of the hint argument, which is preloaded into
+  // a scalar register: blockDim would be a load from the hidden kernel arguments in front of
+  // everything else
+  const uint32_t waves_per_wg = nt_bits >> 8;
+  nt_bits &= 3u;
+  const uint32_t wave = uniform(wg * waves_per_wg + (threadIdx.x >> 6));
   uint32_t t = wave * a.tiles_per_wave;
   if (t >= a.ntiles) return;
   const uint32_t t_end =
@@ -1354,11 +1359,16 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const uint8_t* src_arg
   wave_copy<2, NT, NT>(src, dst, bytes - off, lane, lane * kVecBytes);
 }
 
+// The cache hints (bits 0-1) and the wavefronts per workgroup (bits 8-15) in one argument.
+uint32_t hint_argument(const LaunchConfig& cfg) {
+  return (cfg.nontemporal & 3u) | (cfg.threads / kWaveLanes) << 8;
+}
+
 template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
   const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * (cfg.threads / kWaveLanes) : 0u;
-#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave, cfg.nontemporal, args.tensor_delta
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave, hint_argument(cfg), args.tensor_delta
 #define AXR_LAUNCH(NTT, NTP, EL) \
   hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, lds_bytes, stream, AXR_ARGS)
   // cfg.elements: strided tensors with short runs or transpositions are present
@@ -1489,7 +1499,7 @@ int launch_bundle_kernel_inline(bool pack, const KernelArgs& args, const LaunchC
 #define AXR_INLINE_LAUNCH(PACK, EL)                                                              \
   hipLaunchKernelGGL((bundle_kernel_inline<PACK, EL>), grid, block, lds_bytes, s, args.payload,   \
                      args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift,            \
-                     cfg.lds_per_wave, cfg.nontemporal, dims_at, wave_at, tables)
+                     cfg.lds_per_wave, hint_argument(cfg), dims_at, wave_at, tables)
   if (pack) {
     if (cfg.elements) AXR_INLINE_LAUNCH(true, true); else AXR_INLINE_LAUNCH(true, false);
   } else {

@@ -2023,7 +2023,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
       table.interleaved = (end - i == 2 && jobs[i + 1].plan->cfg.workgroups == first->cfg.workgroups) ? 1u : 0u;
     }
     table.lds_per_wave = cfg.lds_per_wave;
-    table.nt_bits = cfg.nontemporal;
+    table.nt_bits = (cfg.nontemporal & 3u) | (cfg.threads / kWaveLanes) << 8;   // hints, wavefronts per workgroup
     cfg.workgroups = wg;
     if (cfg.lds_per_wave) {
       // every plan sized its workgroups for its own LDS need; the launch uses the largest
