@@ -163,12 +163,14 @@ struct JobDesc {              // 64 bytes
   uint32_t reserved;
 };
 static_assert(sizeof(JobDesc) == 64, "JobDesc layout");
+constexpr uint32_t kNoJobBegin = 0x7fffffffu;        // beyond every workgroup index of a launch
+constexpr uint32_t kJobTableKernargOffset = 64;      // the table follows 14 scalar arguments, 16-byte aligned
 struct alignas(16) JobTable {
   uint32_t count, lds_per_wave, nt_bits;
   uint32_t interleaved;       // 1: two jobs of equal grids, job = workgroup & 1, local workgroup = workgroup >> 1
-  // first workgroup of every job once more, side by side (0xffffffff past the last job): a workgroup
-  // finds its job by comparing with all of them after ONE scalar load, instead of walking the
-  // descriptors with a dependent load per step
+  // first workgroup of every job once more, side by side (kNoJobBegin past the last job): the kernel
+  // gets the first eleven as scalar arguments as well and reads the rest here, instead of walking
+  // the descriptors with a dependent load per step
   uint32_t begins[kMaxJobs];
   JobDesc job[kMaxJobs];
 };

@@ -1081,24 +1081,45 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
 // sender packing bundle k + 1 while the receiver unpacks bundle k; a batch of small
 // bundles).  Halves the per-launch cost of short kernels.  The job table arrives by value
 // and is read in place in the kernarg segment (scalar loads, no private copy).
+// 1 when `wg` lies at or beyond `begin`, by the sign of the difference (both are below 2^31):
+// scalar arithmetic, where a comparison turned into a lane mask and back.
+__device__ __forceinline__ uint32_t at_or_beyond(uint32_t wg, uint32_t begin) {
+  return ((wg - begin) >> 31) ^ 1u;
+}
+
+// The head of the job table arrives as scalar arguments in front of the table: count, LDS per
+// wavefront, hints, the in-turn flag and the first workgroups of jobs 1-10.  Leading scalar
+// arguments are preloaded into scalar registers when a wavefront starts, so a workgroup of a
+// launch of up to eleven jobs finds its job without a single load (first workgroups of jobs
+// that do not exist are kNoJobBegin).
 template <uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_jobs_kernel(
+    uint32_t count, uint32_t lds_per_wave, uint32_t nt_bits, uint32_t interleaved, uint32_t b1, uint32_t b2,
+    uint32_t b3, uint32_t b4, uint32_t b5, uint32_t b6, uint32_t b7, uint32_t b8, uint32_t b9, uint32_t b10,
     JobTable jobs_arg) {
   (void)jobs_arg;
-  const AXR_CONST JobTable* jt =
-      (const AXR_CONST JobTable*)__builtin_amdgcn_kernarg_segment_ptr();
+  static_assert(kJobTableKernargOffset % alignof(JobTable) == 0 && kJobTableKernargOffset >= 14 * 4, "kernarg layout");
+  const AXR_CONST JobTable* jt = (const AXR_CONST JobTable*)((const AXR_CONST uint8_t*)
+      __builtin_amdgcn_kernarg_segment_ptr() + kJobTableKernargOffset);
   const uint32_t wg = blockIdx.x;
   // the job whose workgroup range holds this workgroup: the ranges ascend, so it is the number of
-  // ranges that begin at or below this workgroup (entries past the last job hold 0xffffffff)
-  uint32_t j = 0;
+  // ranges that begin at or below this workgroup
+  uint32_t j = at_or_beyond(wg, b1);
+  if (count > 2) {
+    j += at_or_beyond(wg, b2) + at_or_beyond(wg, b3) + at_or_beyond(wg, b4) + at_or_beyond(wg, b5) +
+         at_or_beyond(wg, b6) + at_or_beyond(wg, b7) + at_or_beyond(wg, b8) + at_or_beyond(wg, b9) +
+         at_or_beyond(wg, b10);
+    if (count > 11) {
 #pragma unroll
-  for (uint32_t k = 1; k < kMaxJobs; ++k) j += wg >= jt->begins[k] ? 1u : 0u;
+      for (uint32_t k = 11; k < kMaxJobs; ++k) j += at_or_beyond(wg, jt->begins[k]);
+    }
+  }
   bool in_turn = false;
   if constexpr (NTP) {
     // Streaming payloads only (these instantiations): two jobs of equal grids take the
     // workgroups in turn.  Kept out of the other instantiations, where the extra test cost the
     // 48 MB bundle 0.7 % per launch.
-    in_turn = jt->interleaved != 0;
+    in_turn = interleaved != 0;
     if (in_turn) j = wg & 1u;
   }
   const AXR_CONST JobDesc* d = &jt->job[j];
@@ -1115,11 +1136,9 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   gbytes payload = reinterpret_cast<gbytes>(d->payload);
   const uint32_t local = local_wg;
   if (d->unpack) {   // workgroup-uniform
-    bundle_body<false, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, jt->lds_per_wave,
-                                                 jt->nt_bits);
+    bundle_body<false, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, lds_per_wave, nt_bits);
   } else {
-    bundle_body<true, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, jt->lds_per_wave,
-                                                jt->nt_bits);
+    bundle_body<true, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, lds_per_wave, nt_bits);
   }
 }
 
@@ -1449,7 +1468,10 @@ int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stre
   const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * waves_per_wg : 0u;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define AXR_JOBS(ROWS, NTT, NTP, EL) \
-  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, jobs)
+  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, jobs.count,         \
+                     jobs.lds_per_wave, jobs.nt_bits, jobs.interleaved, jobs.begins[1], jobs.begins[2],      \
+                     jobs.begins[3], jobs.begins[4], jobs.begins[5], jobs.begins[6], jobs.begins[7],          \
+                     jobs.begins[8], jobs.begins[9], jobs.begins[10], jobs)
 #define AXR_JOBS_NT(ROWS, EL)                                    \
   switch (cfg.nontemporal & 3u) {                                \
     case 0: AXR_JOBS(ROWS, false, false, EL); break;             \

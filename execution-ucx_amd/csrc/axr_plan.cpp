@@ -2016,7 +2016,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
       cfg.lds_per_wave = std::max(cfg.lds_per_wave, p->cfg.lds_per_wave);
     }
     table.count = static_cast<uint32_t>(end - i);
-    for (uint32_t k = 0; k < kMaxJobs; ++k) table.begins[k] = k < table.count ? table.job[k].wg_begin : 0xffffffffu;
+    for (uint32_t k = 0; k < kMaxJobs; ++k) table.begins[k] = k < table.count ? table.job[k].wg_begin : kNoJobBegin;
     const int64_t interleave = tunables().submit_interleave;
     if (interleave != 0 && (cfg.nontemporal & 2u) != 0) {   // the streaming instantiations carry the code
       // (two jobs: a shift and a mask in the kernel)
