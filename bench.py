@@ -1168,7 +1168,9 @@ def main():
         # the reference's own layout (tight concatenation) and a payload that bypasses the
         # last-level cache on both sides
         extras["c2_tight"] = c2_variant(align=1)
-        extras["c2_payload_streaming"] = c2_variant(payload_cache_bytes=0)
+        # same geometry, both sides non-temporal (lowering payload_cache_bytes instead would also
+        # switch the bundle to the tile geometry of payloads that stream)
+        extras["c2_payload_streaming"] = c2_variant(nontemporal=3)
         extras.update({k: round(v, 2) for k, v in end_to_end_us(h, spec).items()})
         extras["fresh_bundle_from_cpp"] = end_to_end_from_cpp()
         del sets

@@ -249,11 +249,12 @@ struct Tunables {
   // tensor gets its own wavefronts.
   std::atomic<int64_t> group_bytes{512};
   std::atomic<int64_t> group_slots{kGroupMaxSlots};   // lane slots per group tile: 64 or 128
-  // The two jobs of an axr_submit launch whose grids are equal and whose payloads stream take the
-  // workgroups in turn (even / odd) instead of one range each (1, the default; 0: never).  With a
-  // pack and an unpack in one launch the memory then sees reads and writes of both throughout: the
-  // 405 MB layer bundle 6.50 -> 6.65 TB/s.  Payloads kept in the last-level cache are better off
-  // with the pack's range first (48 MB mixed bundle: 6.18 against 6.11 TB/s) and never interleave.
+  // The two jobs of an axr_submit launch whose grids are equal and whose payloads are larger than
+  // payload_cache_bytes take the workgroups in turn (even / odd) instead of one range each (1, the
+  // default; 0: never; 2: also smaller payloads that were asked to stream).  With a pack and an
+  // unpack in one launch the memory then sees reads and writes of both throughout: the 405 MB
+  // layer bundle 6.50 -> 6.65 TB/s.  Smaller payloads are better off with the pack's range first,
+  // cached (48 MB mixed bundle: 6.18 against 6.11 TB/s) or streaming (5.78 against 5.51).
   std::atomic<int64_t> submit_interleave{1};
   // Failure injection for tests of the streamed transfer's error handling: N > 0 makes the
   // N-th chunk submitted from now on fail after its send has been queued, as if the message

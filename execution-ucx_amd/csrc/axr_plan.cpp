@@ -2018,9 +2018,11 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     table.count = static_cast<uint32_t>(end - i);
     for (uint32_t k = 0; k < kMaxJobs; ++k) table.begins[k] = k < table.count ? table.job[k].wg_begin : kNoJobBegin;
     const int64_t interleave = tunables().submit_interleave;
-    if (interleave != 0 && (cfg.nontemporal & 2u) != 0) {   // the streaming instantiations carry the code
-      // (two jobs: a shift and a mask in the kernel)
-      table.interleaved = (end - i == 2 && jobs[i + 1].plan->cfg.workgroups == first->cfg.workgroups) ? 1u : 0u;
+    if (interleave != 0 && (cfg.nontemporal & 2u) != 0 && end - i == 2 &&   // the streaming instantiations carry the code
+        jobs[i + 1].plan->cfg.workgroups == first->cfg.workgroups) {
+      const uint64_t cache = static_cast<uint64_t>(tunables().payload_cache_bytes);
+      const bool beyond_cache = first->payload_bytes > cache && jobs[i + 1].plan->payload_bytes > cache;
+      table.interleaved = (beyond_cache || interleave > 1) ? 1u : 0u;
     }
     table.lds_per_wave = cfg.lds_per_wave;
     table.nt_bits = (cfg.nontemporal & 3u) | (cfg.threads / kWaveLanes) << 8;   // hints, wavefronts per workgroup

@@ -463,8 +463,8 @@ AXR_API int axr_plan_segments(axr_plan_t* plan, axr_segment_info_t* out, size_t 
  * per wavefront, so that wavefronts and table bytes scale with the payload and not with
  * the tensor count; default 512, at most 1023, 0: every tensor gets wavefronts of its own),
  * "submit_interleave" (1, the default: the two jobs of an axr_submit launch of two jobs with equal
- * grids and streaming payloads take the workgroups in turn instead of one range each; 0: never;
- * read at every axr_submit),
+ * grids and payloads larger than payload_cache_bytes take the workgroups in turn instead of one
+ * range each; 2: also smaller payloads that stream; 0: never; read at every axr_submit),
  * "transfer_fail_after_send" (failure injection for tests: N > 0 makes the N-th chunk that
  * axr_transfer_submit is given from now on fail with AXR_ERR_MISMATCH after its send has been
  * queued, as if the message that arrived did not match the receiver's plan; 0, the default: off),

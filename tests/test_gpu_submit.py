@@ -447,12 +447,12 @@ def test_streaming_geometry_for_payloads_beyond_the_cache(pkg, gpu, device_table
         pkg.tune(device_tables=before.value)
 
 
-@pytest.mark.parametrize("interleave", [1, 0])
+@pytest.mark.parametrize("interleave", [2, 0])
 def test_two_jobs_of_equal_grids_take_workgroups_in_turn(pkg, orc, gpu, interleave):
     """Two bundles of one geometry (the same sizes at other addresses) in one launch: the pack
     of one and the unpack of the other, payloads streaming, with the jobs' workgroups
-    interleaved ("submit_interleave", the default for such a launch) and in one range each;
-    the same bytes either way."""
+    interleaved ("submit_interleave" = 2; by default only payloads beyond the cache size do
+    that) and in one range each; the same bytes either way."""
     import torch
     lib, capi = pkg._capi.load(), pkg._capi
     rng = np.random.default_rng(77)
