@@ -1087,31 +1087,35 @@ __device__ __forceinline__ uint32_t at_or_beyond(uint32_t wg, uint32_t begin) {
   return ((wg - begin) >> 31) ^ 1u;
 }
 
-// The head of the job table arrives as scalar arguments in front of the table: count, LDS per
-// wavefront, hints, the in-turn flag and the first workgroups of jobs 1-10.  Leading scalar
-// arguments are preloaded into scalar registers when a wavefront starts, so a workgroup of a
-// launch of up to eleven jobs finds its job without a single load (first workgroups of jobs
-// that do not exist are kNoJobBegin).
+// What a wavefront needs before its first table read arrives as scalar arguments in front of
+// the job table: leading scalar arguments are preloaded into scalar registers when a wavefront
+// starts, a struct passed by value is not.  `head` = job count (bits 0-7), the in-turn flag (bit
+// 8), the directions of jobs 0 and 1 (bits 9, 10: 1 = unpack) and their tile-block shifts (bits
+// 16-23, 24-31); then the first workgroups of jobs 1-3 and, for jobs 0 and 1, the address of the
+// tile-block index, the tile count and the tiles per wavefront.  A workgroup of a launch of one
+// or two jobs (a pack and an unpack handed over together) finds its job and issues its first
+// table read without a load in front of it; the rest of its job's descriptor (table and payload
+// addresses, the address delta) is read from the table at the same time.  Launches of more jobs
+// read the descriptor first (first workgroups of jobs that do not exist are kNoJobBegin).
 template <uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_jobs_kernel(
-    uint32_t count, uint32_t lds_per_wave, uint32_t nt_bits, uint32_t interleaved, uint32_t b1, uint32_t b2,
-    uint32_t b3, uint32_t b4, uint32_t b5, uint32_t b6, uint32_t b7, uint32_t b8, uint32_t b9, uint32_t b10,
+    uint32_t head, uint32_t lds_per_wave, uint32_t nt_bits, uint32_t b1, uint64_t index0, uint32_t ntiles0,
+    uint32_t per_wave0, uint64_t index1, uint32_t ntiles1, uint32_t per_wave1, uint32_t b2, uint32_t b3,
     JobTable jobs_arg) {
   (void)jobs_arg;
   static_assert(kJobTableKernargOffset % alignof(JobTable) == 0 && kJobTableKernargOffset >= 14 * 4, "kernarg layout");
   const AXR_CONST JobTable* jt = (const AXR_CONST JobTable*)((const AXR_CONST uint8_t*)
       __builtin_amdgcn_kernarg_segment_ptr() + kJobTableKernargOffset);
   const uint32_t wg = blockIdx.x;
+  const uint32_t count = head & 0xffu;
   // the job whose workgroup range holds this workgroup: the ranges ascend, so it is the number of
   // ranges that begin at or below this workgroup
   uint32_t j = at_or_beyond(wg, b1);
   if (count > 2) {
-    j += at_or_beyond(wg, b2) + at_or_beyond(wg, b3) + at_or_beyond(wg, b4) + at_or_beyond(wg, b5) +
-         at_or_beyond(wg, b6) + at_or_beyond(wg, b7) + at_or_beyond(wg, b8) + at_or_beyond(wg, b9) +
-         at_or_beyond(wg, b10);
-    if (count > 11) {
+    j += at_or_beyond(wg, b2) + at_or_beyond(wg, b3);
+    if (count > 4) {
 #pragma unroll
-      for (uint32_t k = 11; k < kMaxJobs; ++k) j += at_or_beyond(wg, jt->begins[k]);
+      for (uint32_t k = 4; k < kMaxJobs; ++k) j += at_or_beyond(wg, jt->begins[k]);
     }
   }
   bool in_turn = false;
@@ -1119,23 +1123,42 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
     // Streaming payloads only (these instantiations): two jobs of equal grids take the
     // workgroups in turn.  Kept out of the other instantiations, where the extra test cost the
     // 48 MB bundle 0.7 % per launch.
-    in_turn = interleaved != 0;
+    in_turn = (head & 0x100u) != 0;
     if (in_turn) j = wg & 1u;
   }
   const AXR_CONST JobDesc* d = &jt->job[j];
-  const uint32_t local_wg = in_turn ? wg >> 1 : wg - d->wg_begin;
   KernelArgs a;
-  a.ntiles = d->ntiles;
-  a.tiles_per_wave = d->tiles_per_wave;
   a.xcd_remap = 0;
-  a.seg_shift = d->seg_shift;
+  const AXR_CONST uint32_t* wave_seg;
+  uint32_t begin, unpack;
+  if (j < 2) {   // from the preloaded arguments (uniform)
+    wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(j ? index1 : index0);
+    a.ntiles = j ? ntiles1 : ntiles0;
+    a.tiles_per_wave = j ? per_wave1 : per_wave0;
+    a.seg_shift = (head >> (16u + 8u * j)) & 0xffu;
+    unpack = (head >> (9u + j)) & 1u;
+    begin = j ? b1 : 0u;
+  } else {
+    wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(d->wave_seg);
+    a.ntiles = d->ntiles;
+    a.tiles_per_wave = d->tiles_per_wave;
+    a.seg_shift = d->seg_shift;
+    unpack = d->unpack;
+    begin = d->wg_begin;
+    // consumed here, so that these loads are waited for inside this arm and not where the arms
+    // meet (scalar loads return out of order: a wait there would cover the loads issued below)
+    asm volatile("" : "+s"(begin), "+s"(unpack), "+s"(a.ntiles), "+s"(a.tiles_per_wave), "+s"(a.seg_shift));
+    asm volatile("" : "+s"(wave_seg));
+  }
+  // The rest of the descriptor is asked for here, behind the branch: loads issued in front of it
+  // would be waited for where the two arms meet, ahead of the first table read.
+  asm volatile("" ::: "memory");
   a.tensor_delta = d->tensor_delta;
   seg_table segs = reinterpret_cast<seg_table>(d->segs);
   dims_table dims = reinterpret_cast<dims_table>(d->dims);
-  const AXR_CONST uint32_t* wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(d->wave_seg);
   gbytes payload = reinterpret_cast<gbytes>(d->payload);
-  const uint32_t local = local_wg;
-  if (d->unpack) {   // workgroup-uniform
+  const uint32_t local = in_turn ? wg >> 1 : wg - begin;
+  if (unpack) {   // workgroup-uniform
     bundle_body<false, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, lds_per_wave, nt_bits);
   } else {
     bundle_body<true, ROWS, NTT, NTP, ELEMENTS>(segs, dims, wave_seg, payload, a, local, lds_per_wave, nt_bits);
@@ -1467,11 +1490,17 @@ int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stre
   const dim3 grid(cfg.workgroups), block(cfg.threads);
   const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * waves_per_wg : 0u;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  for (uint32_t k = 0; k < 2 && k < jobs.count; ++k)
+    if (jobs.job[k].seg_shift > 0xffu) return fail(AXR_ERR_INVALID, "tile-block shift does not fit the job head");
+  // count, in-turn flag, directions and tile-block shifts of jobs 0 and 1 (see the kernel)
+  const uint32_t head = (jobs.count & 0xffu) | (jobs.interleaved ? 0x100u : 0u) |
+                        (jobs.job[0].unpack ? 0x200u : 0u) | (jobs.count > 1 && jobs.job[1].unpack ? 0x400u : 0u) |
+                        (jobs.job[0].seg_shift & 0xffu) << 16 | (jobs.count > 1 ? jobs.job[1].seg_shift & 0xffu : 0u) << 24;
 #define AXR_JOBS(ROWS, NTT, NTP, EL) \
-  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, jobs.count,         \
-                     jobs.lds_per_wave, jobs.nt_bits, jobs.interleaved, jobs.begins[1], jobs.begins[2],      \
-                     jobs.begins[3], jobs.begins[4], jobs.begins[5], jobs.begins[6], jobs.begins[7],          \
-                     jobs.begins[8], jobs.begins[9], jobs.begins[10], jobs)
+  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, head,               \
+                     jobs.lds_per_wave, jobs.nt_bits, jobs.begins[1], jobs.job[0].wave_seg, jobs.job[0].ntiles, \
+                     jobs.job[0].tiles_per_wave, jobs.job[1].wave_seg, jobs.job[1].ntiles,                     \
+                     jobs.job[1].tiles_per_wave, jobs.begins[2], jobs.begins[3], jobs)
 #define AXR_JOBS_NT(ROWS, EL)                                    \
   switch (cfg.nontemporal & 3u) {                                \
     case 0: AXR_JOBS(ROWS, false, false, EL); break;             \
