@@ -242,6 +242,45 @@ def run_sets_two_streams(h: Harness, sets, steps, warmup):
     return times[len(times) // 2]
 
 
+def run_sets_one_direction_two_streams(h: Harness, sets, steps, warmup, unpack):
+    """Only the packs (or only the unpacks) of the rotating sets, alternating between two
+    streams: a sender (or a receiver) with several independent bundles in flight, whose launches
+    need no order among themselves.  Host clock around a synchronisation of both streams;
+    returns milliseconds.  The payloads must hold packed data before the unpacks are timed."""
+    lib, check = h.lib, h.capi.check
+    second = C.c_void_p()
+    check(lib.axr_stream_create(C.byref(second)))
+    streams = (h.stream, second.value)
+    n = len(sets)
+    calls = [((s.up if unpack else s.pp), s.ptr, s.nbytes) for s in sets]
+    fn = lib.axr_unpack if unpack else lib.axr_pack
+
+    def step(i):
+        plan, ptr, nb = calls[i % n]
+        rc = fn(plan, ptr, nb, streams[i % 2])
+        if rc:
+            check(rc)
+
+    def drain():
+        for stream in streams:
+            check(lib.axr_stream_synchronize(stream))
+
+    for i in range(warmup):
+        step(i)
+    drain()
+    times, total = [], 0.0
+    while total < h.MIN_TIMED_MS and len(times) < h.MAX_BATCHES:
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        drain()
+        times.append((time.perf_counter() - t0) * 1e3)
+        total += times[-1]
+    check(lib.axr_stream_destroy(second))
+    times.sort()
+    return times[len(times) // 2]
+
+
 def tensor_byte_mask(h, spec):
     """Boolean device tensor over the arena: True for bytes that belong to a tensor."""
     import numpy as np
@@ -1158,6 +1197,14 @@ def main():
         # not `value`: bundles in flight on two streams hide the gap between dependent launches
         ms2 = run_sets_two_streams(h, sets, args.steps, args.warmup)
         extras["c2_two_streams_GBps"] = round(rate(P, ms2, args.steps), 1)
+        # a sender or a receiver alone, its independent bundles alternating between two streams (2P per launch)
+        both = {}
+        for name, unpack in (("pack", False), ("unpack", True)):
+            ms = run_sets_one_direction_two_streams(h, sets, args.steps, args.warmup, unpack)
+            gbps = 2.0 * P * args.steps / (ms * 1e-3) / 1e9
+            both[name + "_only"] = {"GBps_2P": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+        extras["c2_one_direction_two_streams"] = both
+        check_sets(h, sets, "the two-stream one-direction steps")
         extras["c2_graph_replay_GBps"] = graph_replay(h, sets, P)
         if len(sets) >= 4 and len(sets) % 2 == 0:
             # not `value`: two bundles each way per launch (four jobs), the fixed cost of a launch paid once
