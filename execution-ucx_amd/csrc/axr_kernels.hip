@@ -1058,15 +1058,20 @@ __device__ __forceinline__ void bundle_body(seg_table segs, dims_table dims,
 template <bool PACK, uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_kernel(
     const Seg* segs_arg, const Dims* dims_arg, const uint32_t* wave_seg_arg, uint8_t* payload_arg,
-    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t seg_shift,
-    uint32_t lds_per_wave, uint32_t nt_bits, int64_t tensor_delta) {
-  // Scalar arguments (not one struct) so that the compiler can preload them
-  // into SGPRs at dispatch instead of fetching the kernarg segment first.
+    uint32_t ntiles, uint32_t tiles_per_wave, uint32_t xcd_remap, uint32_t geometry, int64_t tensor_delta) {
+  // Scalar arguments (not one struct) so that the compiler can preload them into SGPRs at
+  // dispatch instead of fetching the kernarg segment first.  Fourteen dwords are preloaded,
+  // which is why the LDS bytes per wavefront (bits 0-16), the hints with the wavefronts per
+  // workgroup (bits 17-23, the argument bundle_body takes) and the tile-block shift (bits
+  // 24-31) share one of them: the address delta then fits in as well, and no wavefront waits
+  // for a kernel-argument load before it can form its first tensor address.
+  const uint32_t lds_per_wave = geometry & 0x1ffffu;
+  const uint32_t nt_bits = (geometry >> 17 & 3u) | (geometry >> 19 & 0x1fu) << 8;
   KernelArgs a;
   a.ntiles = ntiles;
   a.tiles_per_wave = tiles_per_wave;
   a.xcd_remap = xcd_remap;
-  a.seg_shift = seg_shift;
+  a.seg_shift = geometry >> 24;
   a.tensor_delta = tensor_delta;
   bundle_body<PACK, ROWS, NTT, NTP, ELEMENTS>(
       reinterpret_cast<seg_table>(reinterpret_cast<uintptr_t>(segs_arg)),
@@ -1410,7 +1415,12 @@ template <bool PACK, uint32_t ROWS>
 int launch_rows(const KernelArgs& args, const LaunchConfig& cfg, hipStream_t stream) {
   const dim3 grid(cfg.workgroups), block(cfg.threads);
   const uint32_t lds_bytes = cfg.elements ? cfg.lds_per_wave * (cfg.threads / kWaveLanes) : 0u;
-#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, args.seg_shift, cfg.lds_per_wave, hint_argument(cfg), args.tensor_delta
+  if (cfg.lds_per_wave > 0x1ffffu || args.seg_shift > 0xffu || cfg.threads / kWaveLanes > 0x1fu)
+    return fail(AXR_ERR_INVALID, "launch geometry does not fit the kernel's geometry argument");
+  // LDS bytes per wavefront | hints << 17 | wavefronts per workgroup << 19 | tile-block shift << 24
+  const uint32_t geometry = cfg.lds_per_wave | (cfg.nontemporal & 3u) << 17 |
+                            (cfg.threads / kWaveLanes) << 19 | args.seg_shift << 24;
+#define AXR_ARGS args.segs, args.dims, args.wave_seg, args.payload, args.ntiles, args.tiles_per_wave, args.xcd_remap, geometry, args.tensor_delta
 #define AXR_LAUNCH(NTT, NTP, EL) \
   hipLaunchKernelGGL((bundle_kernel<PACK, ROWS, NTT, NTP, EL>), grid, block, lds_bytes, stream, AXR_ARGS)
   // cfg.elements: strided tensors with short runs or transpositions are present
