@@ -1092,21 +1092,22 @@ __device__ __forceinline__ uint32_t at_or_beyond(uint32_t wg, uint32_t begin) {
   return ((wg - begin) >> 31) ^ 1u;
 }
 
-// What a wavefront needs before its first table read arrives as scalar arguments in front of
+// What a wavefront needs for its first two table reads arrives as scalar arguments in front of
 // the job table: leading scalar arguments are preloaded into scalar registers when a wavefront
-// starts, a struct passed by value is not.  `head` = job count (bits 0-7), the in-turn flag (bit
-// 8), the directions of jobs 0 and 1 (bits 9, 10: 1 = unpack) and their tile-block shifts (bits
-// 16-23, 24-31); then the first workgroups of jobs 1-3 and, for jobs 0 and 1, the address of the
-// tile-block index, the tile count and the tiles per wavefront.  A workgroup of a launch of one
-// or two jobs (a pack and an unpack handed over together) finds its job and issues its first
-// table read without a load in front of it; the rest of its job's descriptor (table and payload
-// addresses, the address delta) is read from the table at the same time.  Launches of more jobs
-// read the descriptor first (first workgroups of jobs that do not exist are kNoJobBegin).
+// starts, a struct passed by value is not (and the kernel-argument segment is slow memory).
+// `head` = job count (bits 0-7), the in-turn flag (bit 8), the directions of jobs 0 and 1 (bits
+// 9, 10: 1 = unpack), "jobs 0 and 1 give every wavefront one tile" (bit 11) and their tile-block
+// shifts (bits 16-23, 24-31); then the hints, the first workgroup of job 1 and, for jobs 0 and 1,
+// the tile count and the addresses of the tile-block index and of the segment records.  A
+// workgroup of a launch of one or two jobs (a pack and an unpack handed over together) finds its
+// job, reads its index entry and its segment record without a kernel-argument load in front of
+// them; the rest of its job's descriptor (payload address, address delta, strided-view table) is
+// read from the table meanwhile.  Launches of more jobs, or of jobs whose wavefronts take several
+// tiles, read the descriptor first (first workgroups of jobs that do not exist are kNoJobBegin).
 template <uint32_t ROWS, bool NTT, bool NTP, bool ELEMENTS>
 __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? kMaxElementThreads : kMaxThreadsPerWorkgroup) void bundle_jobs_kernel(
-    uint32_t head, uint32_t lds_per_wave, uint32_t nt_bits, uint32_t b1, uint64_t index0, uint32_t ntiles0,
-    uint32_t per_wave0, uint64_t index1, uint32_t ntiles1, uint32_t per_wave1, uint32_t b2, uint32_t b3,
-    JobTable jobs_arg) {
+    uint32_t head, uint32_t nt_bits, uint32_t b1, uint32_t ntiles0, uint64_t index0, uint64_t segs0,
+    uint64_t index1, uint64_t segs1, uint32_t ntiles1, uint32_t lds_per_wave, JobTable jobs_arg) {
   (void)jobs_arg;
   static_assert(kJobTableKernargOffset % alignof(JobTable) == 0 && kJobTableKernargOffset >= 14 * 4, "kernarg layout");
   const AXR_CONST JobTable* jt = (const AXR_CONST JobTable*)((const AXR_CONST uint8_t*)
@@ -1117,11 +1118,8 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   // ranges that begin at or below this workgroup
   uint32_t j = at_or_beyond(wg, b1);
   if (count > 2) {
-    j += at_or_beyond(wg, b2) + at_or_beyond(wg, b3);
-    if (count > 4) {
 #pragma unroll
-      for (uint32_t k = 4; k < kMaxJobs; ++k) j += at_or_beyond(wg, jt->begins[k]);
-    }
+    for (uint32_t k = 2; k < kMaxJobs; ++k) j += at_or_beyond(wg, jt->begins[k]);
   }
   bool in_turn = false;
   if constexpr (NTP) {
@@ -1135,16 +1133,19 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
   KernelArgs a;
   a.xcd_remap = 0;
   const AXR_CONST uint32_t* wave_seg;
+  seg_table segs;
   uint32_t begin, unpack;
-  if (j < 2) {   // from the preloaded arguments (uniform)
+  if (j < 2 && (head & 0x800u) != 0) {   // from the preloaded arguments (uniform)
     wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(j ? index1 : index0);
+    segs = reinterpret_cast<seg_table>(j ? segs1 : segs0);
     a.ntiles = j ? ntiles1 : ntiles0;
-    a.tiles_per_wave = j ? per_wave1 : per_wave0;
+    a.tiles_per_wave = 1;
     a.seg_shift = (head >> (16u + 8u * j)) & 0xffu;
     unpack = (head >> (9u + j)) & 1u;
     begin = j ? b1 : 0u;
   } else {
     wave_seg = reinterpret_cast<const AXR_CONST uint32_t*>(d->wave_seg);
+    uint64_t segs_at = d->segs;
     a.ntiles = d->ntiles;
     a.tiles_per_wave = d->tiles_per_wave;
     a.seg_shift = d->seg_shift;
@@ -1153,13 +1154,13 @@ __global__ __attribute__((amdgpu_waves_per_eu(4))) __launch_bounds__(ELEMENTS ? 
     // consumed here, so that these loads are waited for inside this arm and not where the arms
     // meet (scalar loads return out of order: a wait there would cover the loads issued below)
     asm volatile("" : "+s"(begin), "+s"(unpack), "+s"(a.ntiles), "+s"(a.tiles_per_wave), "+s"(a.seg_shift));
-    asm volatile("" : "+s"(wave_seg));
+    asm volatile("" : "+s"(wave_seg), "+s"(segs_at));
+    segs = reinterpret_cast<seg_table>(segs_at);
   }
   // The rest of the descriptor is asked for here, behind the branch: loads issued in front of it
   // would be waited for where the two arms meet, ahead of the first table read.
   asm volatile("" ::: "memory");
   a.tensor_delta = d->tensor_delta;
-  seg_table segs = reinterpret_cast<seg_table>(d->segs);
   dims_table dims = reinterpret_cast<dims_table>(d->dims);
   gbytes payload = reinterpret_cast<gbytes>(d->payload);
   const uint32_t local = in_turn ? wg >> 1 : wg - begin;
@@ -1502,15 +1503,16 @@ int launch_bundle_jobs(const JobTable& jobs, const LaunchConfig& cfg, void* stre
   hipStream_t s = static_cast<hipStream_t>(stream);
   for (uint32_t k = 0; k < 2 && k < jobs.count; ++k)
     if (jobs.job[k].seg_shift > 0xffu) return fail(AXR_ERR_INVALID, "tile-block shift does not fit the job head");
-  // count, in-turn flag, directions and tile-block shifts of jobs 0 and 1 (see the kernel)
+  // count, in-turn flag, directions, one tile per wavefront and tile-block shifts of jobs 0 and 1
+  const bool one_tile_each = jobs.job[0].tiles_per_wave == 1 && (jobs.count < 2 || jobs.job[1].tiles_per_wave == 1);
   const uint32_t head = (jobs.count & 0xffu) | (jobs.interleaved ? 0x100u : 0u) |
                         (jobs.job[0].unpack ? 0x200u : 0u) | (jobs.count > 1 && jobs.job[1].unpack ? 0x400u : 0u) |
+                        (one_tile_each ? 0x800u : 0u) |
                         (jobs.job[0].seg_shift & 0xffu) << 16 | (jobs.count > 1 ? jobs.job[1].seg_shift & 0xffu : 0u) << 24;
 #define AXR_JOBS(ROWS, NTT, NTP, EL) \
-  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, head,               \
-                     jobs.lds_per_wave, jobs.nt_bits, jobs.begins[1], jobs.job[0].wave_seg, jobs.job[0].ntiles, \
-                     jobs.job[0].tiles_per_wave, jobs.job[1].wave_seg, jobs.job[1].ntiles,                     \
-                     jobs.job[1].tiles_per_wave, jobs.begins[2], jobs.begins[3], jobs)
+  hipLaunchKernelGGL((bundle_jobs_kernel<ROWS, NTT, NTP, EL>), grid, block, lds_bytes, s, head, jobs.nt_bits,   \
+                     jobs.begins[1], jobs.job[0].ntiles, jobs.job[0].wave_seg, jobs.job[0].segs,               \
+                     jobs.job[1].wave_seg, jobs.job[1].segs, jobs.job[1].ntiles, jobs.lds_per_wave, jobs)
 #define AXR_JOBS_NT(ROWS, EL)                                    \
   switch (cfg.nontemporal & 3u) {                                \
     case 0: AXR_JOBS(ROWS, false, false, EL); break;             \
