@@ -487,3 +487,38 @@ def test_two_jobs_of_equal_grids_take_workgroups_in_turn(pkg, orc, gpu, interlea
         assert torch.equal(o, t)
     for p in plans + [rplan]:
         p.close()
+
+
+def test_two_jobs_whose_wavefronts_take_several_tiles(pkg, orc, gpu):
+    """A launch of two jobs normally finds what it needs for its first table reads in the
+    preloaded kernel arguments; plans whose wavefronts walk several tiles ("max_waves") read
+    their descriptors instead.  Same bytes."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    rng = np.random.default_rng(78)
+    before = C.c_int64()
+    capi.check(lib.axr_tune_get(b"max_waves", C.byref(before)))
+    pkg.tune(max_waves=96)
+    try:
+        sets = [random_tensors(rng, gpu, 300, strided_every=7) for _ in range(2)]
+        plans = [pkg.BundlePlan.create(s, align=64) for s in sets]
+        bufs = [torch.full((p.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu) for p in plans]
+        plans[1].pack(bufs[1].data_ptr(), plans[1].payload_bytes)
+        info = plans[0].launch_info()
+        assert info["tiles"] > 96 * (info["threads_per_workgroup"] // 64) or info["workgroups"] * (info["threads_per_workgroup"] // 64) < info["tiles"]
+        outs = zeros_like_views(sets[1])
+        rplan = pkg.BundlePlan.from_header(plans[1].header).bind(outs)
+        torch.cuda.synchronize()
+        arr = job_array(capi, [(plans[0], 0, bufs[0].data_ptr(), plans[0].payload_bytes, 0),
+                               (rplan, 1, bufs[1].data_ptr(), plans[1].payload_bytes, 0)])
+        capi.check(lib.axr_submit(arr, 2, None))
+        torch.cuda.synchronize()
+    finally:
+        pkg.tune(max_waves=before.value)
+    n = plans[0].payload_bytes
+    got = bufs[0].cpu().numpy()
+    assert np.array_equal(got[:n], orc.pack([chunk_of(t) for t in sets[0]], 64)) and (got[n:] == POISON).all()
+    for o, t in zip(outs, sets[1]):
+        assert np.array_equal(chunk_of(o), chunk_of(t))      # bytes: the random bit patterns hold NaNs
+    for p in plans + [rplan]:
+        p.close()
