@@ -1990,7 +1990,18 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
     LaunchConfig cfg = first->cfg;
     cfg.nontemporal = effective_nontemporal(first, jobs[i].flags);
     uint32_t wg = 0;
-    for (size_t k = i; k < end; ++k) {
+    // The jobs of a call do not depend on each other, so their order inside the launch is free:
+    // gathers take the first workgroups, scatters follow.  A scatter then mostly runs while the
+    // payload its gather wrote a launch earlier is still in the last-level cache and the new
+    // gather's tensor reads are under way (48 MB mixed bundle: 6.37 against 6.15 TB/s the other
+    // way round).
+    size_t order[kMaxJobs];
+    size_t slots = 0;
+    for (int unpacks = 0; unpacks < 2; ++unpacks)
+      for (size_t k = i; k < end; ++k)
+        if ((jobs[k].unpack != 0) == (unpacks != 0)) order[slots++] = k;
+    for (size_t slot = 0; slot < slots; ++slot) {
+      const size_t k = order[slot];
       const axr_job_t& j = jobs[k];
       axr_plan* p = j.plan;
       if (!p->resident) {
@@ -1998,7 +2009,7 @@ static int submit_body(const axr_job_t* jobs, size_t n, void* stream_) {
         if (rc) return rc;
       }
       const uint8_t* d = static_cast<const uint8_t*>(p->block.device);
-      JobDesc& jd = table.job[k - i];
+      JobDesc& jd = table.job[slot];
       jd.segs = reinterpret_cast<uint64_t>(d);
       jd.dims = reinterpret_cast<uint64_t>(d + dims_arg_at(p));
       jd.wave_seg = reinterpret_cast<uint64_t>(d + p->wave_at);

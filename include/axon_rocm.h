@@ -323,7 +323,8 @@ AXR_API int axr_plan_prepare(axr_plan_t* plan, void* stream);
  * (up to sixteen per launch; a short kernel's fixed cost is paid once), the rest run
  * one after the other, all on `stream`.  The jobs of one call must not depend on
  * each other (no job may read what another one writes) and no plan may appear
- * twice.  `tensor_delta` is added to every bound tensor address of that job: a
+ * twice; inside a shared launch the gathers take the first workgroups whatever
+ * their place in `jobs`.  `tensor_delta` is added to every bound tensor address of that job: a
  * plan bound once serves tensors of the same shapes and strides at another base
  * (the chunks of a streamed transfer) without rebuilding or re-uploading its
  * tables; it must be 0 for bundles with kDLCPU tensors.  Results are those of
