@@ -1378,9 +1378,13 @@ __global__ __launch_bounds__(256) void rows_reference_kernel(uint8_t* strided_ar
 // that fall into each segment, so that the host neither builds the index nor waits for a copy
 // engine.  Tensors without bytes are segments without tiles, which the bundle kernel's walk
 // steps over.
+constexpr uint32_t kUtilityThreads = 256;   // workgroup size of the table expansion and stream copy launches
+
 __global__ __launch_bounds__(256) void expand_tables_kernel(const Seg* staged, uint32_t n, Seg* segs,
                                                             uint32_t* wave_seg, uint32_t seg_shift) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  // (the launch below always uses workgroups of kUtilityThreads: blockDim would be a load from
+  // the hidden kernel arguments in front of the first read)
+  const uint32_t i = blockIdx.x * kUtilityThreads + threadIdx.x;
   if (i > n) return;
   const Seg sg = staged[i];
   segs[i] = sg;
@@ -1399,7 +1403,7 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const uint8_t* src_arg
                                                           uint64_t bytes) {
   constexpr uint32_t kTile = 2 * kRowBytes;
   const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
-  const uint64_t wave = uniform(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+  const uint64_t wave = uniform(blockIdx.x * (kUtilityThreads >> 6) + (threadIdx.x >> 6));
   const uint64_t off = wave * kTile;
   if (off >= bytes) return;
   gcbytes src = reinterpret_cast<gcbytes>(reinterpret_cast<uintptr_t>(src_arg)) + off;
@@ -1609,7 +1613,7 @@ int static_table_area(void** ptr) {
 
 int launch_expand_tables(const Seg* staged, uint32_t n, Seg* segs, uint32_t* wave_seg, uint32_t seg_shift,
                          void* stream) {
-  hipLaunchKernelGGL(expand_tables_kernel, dim3((n + 1 + 255) / 256), dim3(256), 0,
+  hipLaunchKernelGGL(expand_tables_kernel, dim3((n + kUtilityThreads) / kUtilityThreads), dim3(kUtilityThreads), 0,
                      static_cast<hipStream_t>(stream), staged, n, segs, wave_seg, seg_shift);
   return check_hip(hipGetLastError(), "table expansion launch");
 }
@@ -1617,9 +1621,9 @@ int launch_expand_tables(const Seg* staged, uint32_t n, Seg* segs, uint32_t* wav
 int launch_stream_copy(void* dst, const void* src, size_t bytes, bool nontemporal, void* stream) {
   if (bytes == 0) return AXR_OK;
   const uint64_t waves = (static_cast<uint64_t>(bytes) + 2 * kRowBytes - 1) / (2 * kRowBytes);
-  const uint64_t groups = (waves + 3) / 4;
+  const uint64_t groups = (waves + kUtilityThreads / kWaveLanes - 1) / (kUtilityThreads / kWaveLanes);
   if (groups > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "range too long for one copy launch");
-  const dim3 grid(static_cast<uint32_t>(groups)), block(256);
+  const dim3 grid(static_cast<uint32_t>(groups)), block(kUtilityThreads);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (nontemporal) {
     hipLaunchKernelGGL(stream_copy_kernel<true>, grid, block, 0, s, static_cast<const uint8_t*>(src),
