@@ -290,8 +290,10 @@ class AxonRuntime:
     def _finish(self, sent, tolerate_failure: bool = False) -> None:
         request, bundle = sent
         try:
-            if not self._ctx.test(request):
-                raise RuntimeError("the peer did not fetch the payload")
+            if self._ctx is not None and not self._ctx.test(request):
+                # nobody fetched the payload: withdraw the message before its memory goes back
+                self._ctx.cancel(request)
+                raise _capi.AxonRocmError(_capi.AXR_ERR_CANCELED, "the peer did not fetch the payload")
         except _capi.AxonRocmError:
             if not tolerate_failure:
                 raise
@@ -319,7 +321,11 @@ class AxonRuntime:
         async with peer._serve_lock():
             with self._activate():
                 sent = self._send(conn, record, list(args))
-            pending = await peer._serve_one(back)
+            try:
+                pending = await peer._serve_one(back)
+            except BaseException:                   # the server could not even answer (or the call
+                self._finish(sent, tolerate_failure=True)   # was cancelled): the request's bundle
+                raise                                       # goes back to its pool all the same
         try:
             with self._activate():
                 msg, reply, rest = self._take_reply(request_id)

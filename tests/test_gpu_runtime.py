@@ -199,3 +199,36 @@ def test_failures_reach_the_caller_as_runtime_errors(pkg, gpu):
     import gc
     gc.collect()
     assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+
+
+def test_a_call_cancelled_inside_its_handler_gives_its_memory_back(pkg, gpu):
+    """The caller gives up (asyncio.wait_for) while the handler is suspended: the request's
+    payload block returns to the pool and the pair serves the next call."""
+    import torch
+
+    async def never(x):
+        await asyncio.sleep(3600)
+        return x
+
+    async def body():
+        server, client = pair(pkg, "cancel_server", "cancel_client")
+        try:
+            server.register_function(never, 1)
+            server.register_function(lambda x: x * 2, 2, function_name="twice",
+                                     from_dlpack_fn=torch.from_dlpack)
+            await client.connect_endpoint_async(server.get_local_address(), "cancel_server")
+            big = torch.arange(1 << 20, dtype=torch.float32, device=gpu)     # rendezvous
+            with pytest.raises(asyncio.TimeoutError):
+                await asyncio.wait_for(
+                    client.invoke(big, worker_name="cancel_server", session_id=0, function=1), 0.05)
+            out = await client.invoke(big, worker_name="cancel_server", session_id=0, function="twice",
+                                      from_dlpack_fn=torch.from_dlpack)
+            assert torch.equal(out, big * 2)
+            del out
+        finally:
+            client.stop()
+            server.stop()
+    run(body())
+    import gc
+    gc.collect()
+    assert pkg.DevicePool.default().stats()["live_blocks"] == 0
