@@ -410,6 +410,11 @@ class DLPackExport:
         managed.deleter = _managed_deleter
         _live_exports[key] = (managed, shape, self, self._release)
         self._exported = True
+        native = _native()
+        if native is not None and hasattr(native, "new_capsule"):
+            # the C destructor keeps a consumer's pending exception intact when a refused
+            # capsule is dropped; the ctypes one below cannot run under a pending exception
+            return native.new_capsule(C.addressof(managed))
         return _py.PyCapsule_New(C.addressof(managed), _NAME, _capsule_destructor)
 
     def __del__(self):

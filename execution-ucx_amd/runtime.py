@@ -9,7 +9,8 @@ serving runtime receives it through the registered function's memory policy (or 
 converted by ``from_dlpack_fn``), runs the handler, and the result travels back the same
 way into the caller's memory policy.  The policy's own tensor objects are what the handler
 and the caller get (axon/python/src/memory_policy_helpers.cpp:44-140).  Non-tensor
-arguments of plain types (None, bool, int, float, str) travel in the request record.
+arguments (None, bool, int, float, str, and lists of bool / int / float / str or lists of lists of
+bool / int / float, classified and typed as the reference does it) travel in the request record.
 
 What it is not: the RPC runtime.  There is no dispatcher, no hybrid logical clock, no
 session or workflow bookkeeping, no thread pool and no network: peers are runtimes of the
@@ -56,10 +57,79 @@ class _Function:
         self.memory_policy, self.lifecycle_policy, self.from_dlpack_fn = memory_policy, lifecycle_policy, from_dlpack_fn
 
 
-def _is_tensor_argument(arg: Any) -> bool:
-    if _is_tensor(arg):
+def _holds_plain_values(arg: Sequence[Any]) -> bool:
+    """ClassifyArg for a list or tuple (bindings_runtime_helpers.hpp:262-330): True when the
+    reference would send it as a non-tensor parameter, False for a (nested) list of tensors.
+    An empty sequence counts as an empty list of tensors."""
+    if len(arg) == 0 or _is_tensor(arg[0]):
+        return False
+    if not isinstance(arg[0], (list, tuple)):
         return True
-    return isinstance(arg, (list, tuple)) and not isinstance(arg, _PLAIN)
+    for inner in arg:
+        if not isinstance(inner, (list, tuple)):
+            raise TypeError("Heterogeneous sequences are not supported as RPC arguments: expected all "
+                            "elements to be sequences (list/tuple) for List[List[Tensor]]")
+        if len(inner) == 0:
+            continue
+        if _is_tensor(inner[0]):
+            return False
+        if isinstance(inner[0], (bool, int, float, str)):
+            return True
+        raise TypeError("Unsupported element type inside nested sequence: expected a DLPack-compatible "
+                        "tensor, int, float, bool, or str for List[List[T]] argument")
+    return True
+
+
+def _element_cast(first: Any, nested: bool) -> Callable[[Any], Any]:
+    """The element type a list takes from its first element (param_conversion.cpp:381-408; nested
+    lists hold bool, int or float only, :435-446) as a function that admits an element."""
+    def exactly(kind, name):
+        def cast(x):
+            if not isinstance(x, kind):
+                raise RuntimeError(f"list element {x!r} is not {name}")
+            return x
+        return cast
+
+    def as_int(x):
+        if not isinstance(x, int):
+            raise RuntimeError(f"list element {x!r} is not an int")
+        return int(x)
+
+    def as_float(x):
+        if isinstance(x, bool) or not isinstance(x, (int, float)):
+            raise RuntimeError(f"list element {x!r} is not a float")
+        return float(x)
+
+    if isinstance(first, bool):
+        return exactly(bool, "a bool")
+    if isinstance(first, int):
+        return as_int
+    if isinstance(first, float):
+        return as_float
+    if isinstance(first, str) and not nested:
+        return exactly(str, "a str")
+    if nested:
+        raise RuntimeError(f"EncodeNestedListToParamMeta: unsupported element type '{type(first)}'. "
+                           "List[List[...]] only supports int, float, bool elements.")
+    raise RuntimeError("Unsupported list element type for inference")
+
+
+def _plain_sequence(arg: Sequence[Any]) -> List[Any]:
+    """A list or tuple of plain values as the reference's parameter inference admits it
+    (InferParamMeta, param_conversion.cpp:369-409: one element type per list, taken from the
+    first element; EncodeNestedListToParamMeta, :419-457: from the first element of the first
+    inner list that has one).  Arrives as lists."""
+    if isinstance(arg[0], (list, tuple)):
+        first = next((inner[0] for inner in arg if len(inner)), None)
+        if first is None:
+            raise RuntimeError("cannot infer element type from List[List[...]] when all inner lists are empty")
+        cast = _element_cast(first, nested=True)
+        if not all(isinstance(inner, (list, tuple)) for inner in arg):
+            raise TypeError("Heterogeneous sequences are not supported as RPC arguments: expected all "
+                            "elements to be sequences (list/tuple)")
+        return [[cast(x) for x in inner] for inner in arg]
+    cast = _element_cast(arg[0], nested=False)
+    return [cast(x) for x in arg]
 
 
 def _split_arguments(args: Sequence[Any]) -> Tuple[List[Any], List[Any]]:
@@ -69,12 +139,17 @@ def _split_arguments(args: Sequence[Any]) -> Tuple[List[Any], List[Any]]:
     for arg in args:
         if isinstance(arg, _PLAIN):
             slots.append({"v": arg})
-        elif _is_tensor_argument(arg):
+        elif _is_tensor(arg):
             tensor_args.append(arg)
             slots.append("t")
+        elif isinstance(arg, (list, tuple)):
+            if _holds_plain_values(arg):
+                slots.append({"v": _plain_sequence(arg)})
+            else:
+                tensor_args.append(arg)
+                slots.append("t")
         else:
-            raise TypeError(f"unsupported argument type {type(arg).__name__}: a DLPack tensor, a "
-                            "(nested) list of tensors, or None / bool / int / float / str")
+            raise RuntimeError(f"Unsupported type for inference: {type(arg)}")     # param_conversion.cpp:410-414
     return tensor_args, slots
 
 

@@ -66,12 +66,57 @@ def recv_tensors(ctx: LoopbackAmContext,
     return _receive(ctx, msg, msg.header, memory_policy, from_dlpack_fn, stream, pool)
 
 
+def _host_views(plan: BundlePlan, metas: Sequence[TensorMeta], host, from_dlpack_fn) -> List[Any]:
+    """kDLCPU producers over ``host`` (a numpy byte array holding the whole payload), split at
+    the header's offsets; every view keeps the array alive."""
+    from .dlpack import DLPackExport
+    pieces = plan.split(host.ctypes.data if host.size else 0, host.size)
+    out = []
+    for (p, _n), m in zip(pieces, metas):
+        exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLCPU, 0, release=(lambda keep=host: None))
+        out.append(from_dlpack_fn(exp) if from_dlpack_fn else exp)
+    return out
+
+
+def _receive_without_policy(ctx, msg, bundle_header, from_dlpack_fn, stream, pool) -> List[Any]:
+    """Tensors that were in host memory at the sender arrive in host memory (the reference's
+    default receive memory is host, axon/src/axon_worker.cpp:1098-1219, and an eager payload
+    is in host memory when it is delivered, ucx_context/ucx_am_context/ucx_am_context.cpp:864-953),
+    so that ``numpy.from_dlpack`` can take them; device tensors arrive as views of the
+    received device payload."""
+    import numpy as np
+    with BundlePlan.from_header(bundle_header) as plan:
+        metas = plan.metas()
+        on_host = [m.device.device_type == _capi.kDLCPU and m.nbytes > 0 for m in metas]
+        if not any(on_host):
+            payload = _payload_on_device(ctx, msg, pool, stream)
+            return unpack_bundle(bundle_header, payload, payload_bytes=msg.data_length,
+                                 from_dlpack_fn=from_dlpack_fn)
+        everything_on_host = all(h or m.nbytes == 0 for h, m in zip(on_host, metas))
+        if everything_on_host and not msg.is_rndv:        # the bytes are on the host already
+            host = np.frombuffer(msg.eager_data, dtype=np.uint8, count=msg.data_length).copy()
+            return _host_views(plan, metas, host, from_dlpack_fn)
+        payload = _payload_on_device(ctx, msg, pool, stream)
+        try:
+            host = np.empty(msg.data_length, dtype=np.uint8)
+            if msg.data_length:                            # one copy of the whole payload
+                _capi.check(_capi.load().axr_memcpy(_capi.MEM_HOST, host.ctypes.data, ROCM, payload.data,
+                                                    msg.data_length))
+            views = _host_views(plan, metas, host, None)
+            if not everything_on_host:
+                device_views = unpack_bundle(bundle_header, payload, payload_bytes=msg.data_length)
+                views = [h if is_host else d for h, d, is_host in zip(views, device_views, on_host)]
+            return [from_dlpack_fn(v) if from_dlpack_fn else v for v in views]
+        finally:
+            if everything_on_host:
+                payload.release()
+
+
 def _receive(ctx, msg, bundle_header, memory_policy, from_dlpack_fn, stream, pool) -> List[Any]:
     pool = pool or DevicePool.default()
-    payload = _payload_on_device(ctx, msg, pool, stream)
     if memory_policy is None:
-        return unpack_bundle(bundle_header, payload, payload_bytes=msg.data_length,
-                             from_dlpack_fn=from_dlpack_fn)
+        return _receive_without_policy(ctx, msg, bundle_header, from_dlpack_fn, stream, pool)
+    payload = _payload_on_device(ctx, msg, pool, stream)
     metas = BundlePlan.from_header(bundle_header)
     wanted = metas.metas()
     metas.close()

@@ -184,7 +184,7 @@ def test_failures_reach_the_caller_as_runtime_errors(pkg, gpu):
                 await client.invoke(big, worker_name="err_server", session_id=0, function="nobody")
             with pytest.raises(RuntimeError, match="incompatible buffer type"):
                 await client.invoke(big, worker_name="err_server", session_id=0, function="echo")
-            with pytest.raises(TypeError):
+            with pytest.raises(RuntimeError, match="Unsupported type for inference"):
                 await client.invoke({"a": 1}, worker_name="err_server", session_id=0, function=5)
             # and the pair still works afterwards
             server.register_function(lambda x: x, 7, function_name="echo2")
@@ -230,5 +230,144 @@ def test_a_call_cancelled_inside_its_handler_gives_its_memory_back(pkg, gpu):
             server.stop()
     run(body())
     import gc
+    gc.collect()
+    assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+
+
+def test_numpy_arguments_and_results_like_the_reference_suite(pkg, gpu):
+    """axon/python/tests/test_numpy_rpc.py:94-247 with the same functions and values: tensors in,
+    an int out; a tensor out; a list of tensors out; a tuple of an int and tensors out; a tensor,
+    an int and a str in; the eight-argument receive_shards call with nested tensor lists next to
+    lists of str, int and bool."""
+    async def sum_int_func(a, b):
+        return int(np.sum(a + b))
+
+    async def sum_arr_func(a, b, c):
+        return np.array([np.sum(a + b) + np.sum(c)], dtype=np.int64)
+
+    async def list_func(a, b):
+        return [a + b, a * b]
+
+    async def tuple_func(x, y):
+        return (int(np.sum(x) + np.sum(y)), x.copy(), y.copy())
+
+    async def mixed_args_func(a, b, c):
+        return f"{np.sum(a)}_{b}_{c}"
+
+    seen = {}
+
+    async def receive_shards_func(op_name, names, step, sender_rank, payload_groups, counts_groups,
+                                  is_ragged_flags, has_indices_flags):
+        assert isinstance(op_name, str) and isinstance(names, list) and isinstance(payload_groups, list)
+        seen.update(names=names, step=step, rank=sender_rank, counts=counts_groups, ragged=is_ragged_flags,
+                    indices=has_indices_flags, groups=[[np.array(t) for t in g] for g in payload_groups])
+        return 0
+
+    async def body():
+        server, client = pair(pkg, "test_worker", "client_worker")
+        try:
+            for i, fn in enumerate([sum_int_func, sum_arr_func, list_func, tuple_func, mixed_args_func,
+                                    receive_shards_func]):
+                server.register_function(fn, i, from_dlpack_fn=np.from_dlpack)
+            await client.connect_endpoint_async(server.get_local_address(), "test_worker")
+            kw = dict(worker_name="test_worker", session_id=0)
+            a = np.array([1, 2, 3, 4, 5, 6, 7, 8], dtype=np.int64)
+            b = np.array([9, 10, 11, 12, 13, 14, 15, 16], dtype=np.int64)
+            c = np.array([17, 18, 19, 20], dtype=np.int64)
+            result = await client.invoke(a, b, function=0, **kw)
+            assert isinstance(result, int) and result == 136
+            result = await client.invoke(a, b, c, function=1, from_dlpack_fn=np.from_dlpack, **kw)
+            assert isinstance(result, np.ndarray) and result[0] == 210
+            result = await client.invoke(a, b, function=2, from_dlpack_fn=np.from_dlpack, **kw)
+            assert isinstance(result, list) and len(result) == 2
+            assert isinstance(result[0], np.ndarray) and isinstance(result[1], np.ndarray)
+            np.testing.assert_array_equal(result[0], a + b)
+            np.testing.assert_array_equal(result[1], a * b)
+            x, y = np.array([1, 2, 3], dtype=np.int64), np.array([4, 5, 6], dtype=np.int64)
+            result = await client.invoke(x, y, function=3, from_dlpack_fn=np.from_dlpack, **kw)
+            assert isinstance(result, tuple) and len(result) == 3 and result[0] == 21
+            np.testing.assert_array_equal(result[1], x)
+            np.testing.assert_array_equal(result[2], y)
+            result = await client.invoke(x, 100, "hello", function=4, from_dlpack_fn=np.from_dlpack, **kw)
+            assert isinstance(result, str) and result == "6_100_hello"
+            rng = np.random.default_rng(0)
+            groups = [[rng.random((2, 2)), rng.random((3, 3))], [rng.random((4, 4))]]
+            result = await client.invoke("test_op", ["tensor_1", "tensor_2"], 10, 0, groups, [[2, 2], [1]],
+                                         [False, True], [True, False], function=5,
+                                         from_dlpack_fn=np.from_dlpack, **kw)
+            assert result == 0
+            assert seen["names"] == ["tensor_1", "tensor_2"] and seen["step"] == 10 and seen["rank"] == 0
+            assert seen["counts"] == [[2, 2], [1]] and seen["ragged"] == [False, True]
+            assert seen["indices"] == [True, False]
+            assert [len(g) for g in seen["groups"]] == [2, 1]
+            for got_group, want_group in zip(seen["groups"], groups):
+                for got, want in zip(got_group, want_group):
+                    np.testing.assert_array_equal(got, want)
+        finally:
+            client.stop()
+            server.stop()
+    run(body())
+    seen.clear()
+    import gc
+    gc.collect()
+    assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+
+
+def test_a_tensor_the_handler_keeps_outlives_the_call(pkg, gpu):
+    """axon/python/tests/test_numpy_rpc.py:472-583: an input tensor stored beyond the handler
+    stays valid after the call has finished, and is released once the last reference goes."""
+    import gc
+    import weakref
+    kept = {}
+
+    async def store_input_func(a, b):
+        kept["a"] = a
+        return a + b
+
+    async def store_then_release_input_func(a):
+        kept["tmp"] = a
+        kept["ref"] = weakref.ref(a)
+        del a
+        await asyncio.sleep(0)
+        total = int(np.sum(kept["tmp"]))
+        kept["tmp"] = None
+        return total
+
+    async def body():
+        server, client = pair(pkg, "test_lifetime_server", "test_lifetime_client")
+        try:
+            server.register_function(store_input_func, 200, from_dlpack_fn=np.from_dlpack)
+            server.register_function(store_then_release_input_func, 201, from_dlpack_fn=np.from_dlpack)
+            await client.connect_endpoint_async(server.get_local_address(), "test_lifetime_server")
+            kw = dict(worker_name="test_lifetime_server", session_id=0, from_dlpack_fn=np.from_dlpack)
+            a = np.array([1.0, 2.0, 3.0, 4.0], dtype=np.float64)
+            b = np.array([10.0, 20.0, 30.0, 40.0], dtype=np.float64)
+            result = await client.invoke(a, b, function=200, **kw)
+            await asyncio.sleep(0)
+            gc.collect()
+            np.testing.assert_array_equal(kept["a"], a)
+            np.testing.assert_array_equal(result, a + b)
+            # the same with a rendezvous-sized tensor (its memory is a pool block)
+            big = np.arange(1 << 18, dtype=np.float64)
+            result = await client.invoke(big, big, function=200, **kw)
+            await asyncio.sleep(0)
+            gc.collect()
+            np.testing.assert_array_equal(kept["a"], big)
+            np.testing.assert_array_equal(result, big + big)
+            del result
+            kept["a"] = None
+            c = np.array([3.0, 4.0, 5.0, 6.0], dtype=np.float64)
+            assert await client.invoke(c, function=201, **kw) == int(np.sum(c))
+            for _ in range(10):
+                if kept["ref"]() is None:
+                    break
+                gc.collect()
+                await asyncio.sleep(0)
+            assert kept["tmp"] is None and kept["ref"]() is None
+        finally:
+            client.stop()
+            server.stop()
+    run(body())
+    kept.clear()
     gc.collect()
     assert pkg.DevicePool.default().stats()["live_blocks"] == 0

@@ -522,6 +522,14 @@ def test_dlpack_export_single_consume(pkg):
     del capsule, ok
     gc.collect()
     assert released[-1] == 8
+    # a consumer that refuses the capsule (numpy takes host memory only) drops it with its own
+    # exception pending: that exception is what the caller sees, and the memory is released
+    refused = pkg.DLPackExport(0x1000, (4,), (2, 32, 1), 10, 0, release=lambda: released.append(9))
+    with pytest.raises(RuntimeError, match="Unsupported device"):
+        np.from_dlpack(refused)
+    del refused
+    gc.collect()
+    assert released[-1] == 9
 
 
 def test_device_objects(pkg):
@@ -869,6 +877,7 @@ def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
     server.start()
     assert server.register_function(lambda a, b="x": f"{a}:{b}", function_name="join") == 1
     assert server.register_function(len, 7) == 7 and server.register_function(abs) == 2
+    server.register_function(lambda *a: a if len(a) > 1 else a[0], 30, function_name="echo_all")
     with pytest.raises(RuntimeError, match="already registered"):
         server.register_function(len, 9)               # name "len" taken
     with pytest.raises(RuntimeError, match="already registered"):
@@ -876,7 +885,7 @@ def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
     with pytest.raises(TypeError):
         server.register_function(3)
     import json
-    assert json.loads(server.get_local_signatures()) == {"join": 1, "len": 7, "abs": 2}
+    assert json.loads(server.get_local_signatures()) == {"join": 1, "len": 7, "abs": 2, "echo_all": 30}
     client = pkg.AxonRuntime("cpu_client", device=pkg.cpu())
     client.start_client()
     assert server.get_local_address() != client.get_local_address()
@@ -897,17 +906,29 @@ def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
         with pytest.raises(RuntimeError, match="not serving"):
             await server.connect_endpoint_async(client.get_local_address(), "cpu_client")
             await server.invoke(1, worker_name="cpu_client", session_id=0, function=1)
-        with pytest.raises(TypeError):
+        with pytest.raises(RuntimeError, match="Unsupported type for inference"):
             await client.invoke(object(), function="join", **kw)
+        # lists of plain values travel as parameters, typed by their first element
+        # (axon/python/tests/test_numpy_rpc.py:216-247 receive_shards, :399-436 nested bool)
+        names, counts, flags = ["tensor_1", "tensor_2"], [[2, 2], [1]], [False, True]
+        assert await client.invoke(names, counts, flags, function="echo_all", **kw) == (names, counts, flags)
+        nested = await client.invoke([[True, False], [], [False]], function="echo_all", **kw)
+        assert nested == [[True, False], [], [False]] and all(isinstance(x, bool) for row in nested for x in row)
+        assert await client.invoke([1.5, 2], function="echo_all", **kw) == [1.5, 2.0]
     asyncio.run(body())
+    for bad, error in (([[], []], RuntimeError), ([1, "a"], RuntimeError), ([["a"]], RuntimeError),
+                       ([[1], 2], TypeError), ({"a": 1}, RuntimeError), ([object()], RuntimeError),
+                       ([[object()]], TypeError), ([1, 2.5], RuntimeError)):
+        with pytest.raises(error):
+            rt._split_arguments([bad])
     # the record framing
     rec, rest = rt._unframe(rt._frame({"a": 1}, b"tail"))
     assert rec == {"a": 1} and rest == b"tail"
     with pytest.raises(RuntimeError):
         rt._unframe(b"nope")
-    targs, slots = rt._split_arguments([1, [], "s", None, [[]]])
-    assert slots == [{"v": 1}, "t", {"v": "s"}, {"v": None}, "t"] and targs == [[], [[]]]
-    assert rt._merge_arguments(slots, ["A", "B"]) == [1, "A", "s", None, "B"]
+    targs, slots = rt._split_arguments([1, [], "s", None, [1, 2]])
+    assert slots == [{"v": 1}, "t", {"v": "s"}, {"v": None}, {"v": [1, 2]}] and targs == [[]]
+    assert rt._merge_arguments(slots, ["A"]) == [1, "A", "s", None, [1, 2]]
     client.stop()
     server.stop()
     with pytest.raises(RuntimeError, match="not been started"):
