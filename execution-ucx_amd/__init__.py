@@ -10,8 +10,8 @@ from ._capi import (AxonRocmError, HeaderError, LengthError, MismatchError, NoDe
                     NoMessageError, NotImplementedForEager, UnsupportedMemoryError)
 from .bundle import (BundlePlan, DLDataType, DLDevice, PackedBundle, TensorMeta, bundle_to_host, pack_bundle,
                      unpack_bundle)
-from .device import (CpuDevice, Device, DeviceType, RocmDevice, auto_detect, cpu, device_count,
-                     rocm)
+from .device import (CpuDevice, CudaDevice, Device, DeviceType, RocmDevice, SyclDevice, auto_detect, cpu, cuda,
+                     device_count, rocm, sycl)
 from .dlpack import DLPackExport, TensorView, extract, extract_many
 from .loopback import AmMessage, LoopbackAmContext
 from .memory import DevicePool, PoolBuffer, RocmMemoryResourceManager

@@ -91,6 +91,57 @@ class RocmDevice(Device):
         return f"RocmDevice(device_id={self.device_id})"
 
 
+class _DeclaredDevice(Device):
+    """A device kind the reference declares (axon/python/axon/device.py:86-128, 170-199) that this
+    build has no runtime for: the object carries what the caller gave it, so scripts written for
+    the reference construct and inspect it as before, and a runtime created with it moves host
+    tensors only (the reference's runtime likewise accepts the object and handles the missing
+    platform internally, axon/python/tests/test_device_api.py:106-112)."""
+
+    _kind: DeviceType
+
+    def __init__(self, device_id: int = 0, context: Optional[int] = None):
+        self.device_id = device_id
+        self._context = context
+
+    def get_type(self) -> DeviceType:
+        return self._kind
+
+    def get_type_string(self) -> str:
+        return self._kind.value
+
+    def get_context_handle(self) -> Optional[int]:
+        return self._context
+
+    def __repr__(self) -> str:
+        return f"{type(self).__name__}(device_id={self.device_id})"
+
+
+class CudaDevice(_DeclaredDevice):
+    _kind = DeviceType.CUDA
+
+    def __repr__(self) -> str:
+        if self._context is not None:
+            return f"CudaDevice(device_id={self.device_id}, context={self._context:#x})"
+        return super().__repr__()
+
+
+class SyclDevice(_DeclaredDevice):
+    _kind = DeviceType.SYCL
+
+    def __init__(self, device_id: int = 0, context: Optional[int] = None, queue: Optional[int] = None):
+        super().__init__(device_id, context)
+        self.queue = queue
+
+
+def cuda(device_id: int = 0, context: Optional[int] = None) -> CudaDevice:
+    return CudaDevice(device_id=device_id, context=context)
+
+
+def sycl(device_id: int = 0, context: Optional[int] = None, queue: Optional[int] = None) -> SyclDevice:
+    return SyclDevice(device_id=device_id, context=context, queue=queue)
+
+
 def cpu(numa_node: Optional[int] = None) -> CpuDevice:
     return CpuDevice(numa_node=numa_node)
 

@@ -540,6 +540,30 @@ def test_device_objects(pkg):
     c = pkg.cpu(numa_node=1)
     assert c.get_type_string() == "cpu" and c.get_context_handle() is None
     assert isinstance(pkg.auto_detect(), pkg.Device)
+    # the rest of the reference's device module (axon/python/tests/test_device_api.py:7-131)
+    for name in ("CPU", "CUDA", "ROCM", "SYCL"):
+        assert hasattr(pkg.DeviceType, name)
+    assert pkg.CpuDevice().get_type() == pkg.DeviceType.CPU and "CpuDevice" in repr(pkg.CpuDevice())
+    assert c.numa_node == 1 and "numa_node=1" in repr(c) and pkg.cpu(numa_node=0).numa_node == 0
+    cuda_dev = pkg.CudaDevice(device_id=0)
+    assert cuda_dev.get_type() == pkg.DeviceType.CUDA and cuda_dev.get_type_string() == "cuda"
+    assert cuda_dev.device_id == 0 and "CudaDevice" in repr(cuda_dev)
+    with_context = pkg.CudaDevice(device_id=1, context=0x12345678)
+    assert with_context.device_id == 1 and with_context.get_context_handle() == 0x12345678
+    sycl_dev = pkg.SyclDevice(device_id=0)
+    assert sycl_dev.get_type() == pkg.DeviceType.SYCL and sycl_dev.get_type_string() == "sycl"
+    assert sycl_dev.device_id == 0 and "SyclDevice" in repr(sycl_dev)
+    assert isinstance(pkg.cuda(), pkg.CudaDevice) and pkg.cuda(device_id=1).device_id == 1
+    assert isinstance(pkg.rocm(), pkg.RocmDevice) and isinstance(pkg.sycl(), pkg.SyclDevice)
+    # a runtime takes any of them (and none); with a host device its whole lifecycle runs here
+    for device in (pkg.cpu(), pkg.cuda(context=None), None):
+        assert pkg.AxonRuntime("test_worker", device=device) is not None
+    runtime = pkg.AxonRuntime("test_worker", device=pkg.cpu())
+    runtime.start()
+    assert len(runtime.get_local_address()) > 0
+    runtime.stop()
+    runtime.stop()                                                   # stopping twice is harmless
+    pkg.AxonRuntime("never_started", device=pkg.cpu()).stop()        # so is stopping without a start
 
 
 # ------------------------------------------------------------------ no device: fail loudly
