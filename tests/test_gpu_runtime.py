@@ -371,3 +371,27 @@ def test_a_tensor_the_handler_keeps_outlives_the_call(pkg, gpu):
     kept.clear()
     gc.collect()
     assert pkg.DevicePool.default().stats()["live_blocks"] == 0
+
+
+def test_server_memory_policy_objects_reach_the_handler_twice(pkg, gpu):
+    """axon/python/tests/test_server_memory_policy.py:14-125: the handler receives the very object
+    the registered policy created, with the data in it, on a first call and on a second one."""
+    async def rpc_handler(arr):
+        return bool(isinstance(arr, TrackedArray) and id(arr) in created_objects and np.allclose(arr, 1.0))
+
+    async def body():
+        server, client = pair(pkg, "test_memory_policy_worker", "client_worker_memfail")
+        try:
+            server.register_function(rpc_handler, 0, memory_policy=tracked_policy, from_dlpack_fn=np.from_dlpack)
+            await client.connect_endpoint_async(server.get_local_address(), "test_memory_policy_worker")
+            large_arr = np.ones((1024, 1024), dtype=np.float32)        # 4 MB: rendezvous
+            kw = dict(worker_name="test_memory_policy_worker", session_id=0, function=0)
+            assert await client.invoke(large_arr, **kw) is True
+            assert await client.invoke(large_arr, **kw) is True
+            # a payload small enough to travel eagerly bypasses the policy (axon_worker.cpp:1150-1172)
+            assert await client.invoke(np.ones(4, dtype=np.float32), **kw) is False
+        finally:
+            client.stop()
+            server.stop()
+    run(body())
+    assert pkg.DevicePool.default().stats()["live_blocks"] == 0
