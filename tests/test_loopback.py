@@ -554,3 +554,17 @@ def test_the_pytorch_rocm_example_runs(gpu):
                          capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "pytorch_rocm_example ok" in out.stdout and "all elements == 3.0" in out.stdout
+
+
+@pytest.mark.gpu
+def test_the_pytorch_host_example_runs(gpu):
+    """examples/pytorch_host_example.py: the reference's host torch example (handler without a
+    policy, rendezvous reply into the caller's policy, eager reply past it)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, os.path.join(root, "examples", "pytorch_host_example.py")],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "pytorch_host_example ok" in out.stdout and "FAILED" not in out.stdout
