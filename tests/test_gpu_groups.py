@@ -218,3 +218,70 @@ def test_random_mixtures_of_short_long_strided_and_empty_tensors(pkg, orc, gpu, 
         assert np.array_equal(o.contiguous().reshape(-1).cpu().numpy(), c)
     rplan.close()
     plan.close()
+
+
+@pytest.mark.parametrize("align", [1, 64])
+def test_more_than_a_million_tensors(pkg, gpu, align):
+    """1.2 million tensors of 0-48 bytes (and a few of 100 KB) in one bundle: beyond the 2^20
+    tensors up to which the device builds the tables, with tensor, tile and table counts that no
+    longer fit 16 or 20 bits anywhere.  The expected payload is built with numpy index
+    arithmetic (offset rule of the aligned layout: every tensor starts at the next multiple of
+    `align`), the descriptors are written as one numpy record array, through the C ABI."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    record = np.dtype([("data", "<u8"), ("device_type", "<i4"), ("device_id", "<i4"), ("ndim", "<i4"),
+                       ("code", "u1"), ("bits", "u1"), ("lanes", "<u2"), ("shape", "<u8"),
+                       ("strides", "<u8"), ("byte_offset", "<u8")])
+    assert record.itemsize == C.sizeof(capi.Tensor)
+    n = 1_200_000
+    rng = np.random.default_rng(align)
+    sizes = rng.integers(1, 49, size=n).astype(np.int64)
+    sizes[::150_000] = rng.integers(50_000, 200_000, size=len(sizes[::150_000]))
+    sizes[rng.integers(0, n, size=n // 50)] = 0
+    starts = np.cumsum(sizes + rng.integers(0, 3, size=n) * 7) - sizes
+    arena_bytes = int(starts[-1] + sizes[-1] + 64)
+    src = torch.randint(0, 256, (arena_bytes,), dtype=torch.uint8, device=gpu)
+    dst = torch.full((arena_bytes,), 0x55, dtype=torch.uint8, device=gpu)
+
+    def descriptors(base):
+        d = np.zeros(n, record)
+        d["data"], d["device_type"], d["ndim"], d["code"], d["bits"], d["lanes"] = base + starts, 10, 1, 1, 8, 1
+        d["shape"] = sizes.ctypes.data + 8 * np.arange(n, dtype=np.uint64)
+        return d, C.cast(C.c_void_p(d.ctypes.data), C.POINTER(capi.Tensor))
+
+    _keep_s, sd = descriptors(src.data_ptr())
+    _keep_d, dd = descriptors(dst.data_ptr())
+    plan, rplan = C.c_void_p(), C.c_void_p()
+    capi.check(lib.axr_plan_create(sd, n, align, 0, C.byref(plan)))
+    try:
+        nbytes = C.c_uint64()
+        capi.check(lib.axr_plan_payload_bytes(plan, C.byref(nbytes)))
+        padded = (sizes + align - 1) & ~(align - 1)
+        offsets = np.cumsum(padded) - padded
+        total = int(offsets[-1] + sizes[-1])
+        assert nbytes.value == total
+        payload = torch.full((total + 64,), POISON, dtype=torch.uint8, device=gpu)
+        torch.cuda.synchronize()
+        capi.check(lib.axr_pack(plan, payload.data_ptr(), total, None))
+        header, header_bytes = C.c_void_p(), C.c_size_t()
+        capi.check(lib.axr_plan_header(plan, C.byref(header), C.byref(header_bytes)))
+        capi.check(lib.axr_plan_from_header_bind(header, header_bytes.value, dd, n, C.byref(rplan)))
+        capi.check(lib.axr_unpack(rplan, payload.data_ptr(), total, None))
+        torch.cuda.synchronize()
+        host = src.cpu().numpy()
+        filled = sizes > 0
+        within = np.arange(int(sizes.sum())) - np.repeat(np.cumsum(sizes[filled]) - sizes[filled], sizes[filled])
+        from_arena = np.repeat(starts[filled], sizes[filled]) + within
+        to_payload = np.repeat(offsets[filled], sizes[filled]) + within
+        want = np.zeros(total, np.uint8)
+        want[to_payload] = host[from_arena]
+        got = payload.cpu().numpy()
+        assert np.array_equal(got[:total], want)
+        assert (got[total:] == POISON).all()
+        expect = np.full(arena_bytes, 0x55, np.uint8)
+        expect[from_arena] = host[from_arena]
+        assert np.array_equal(dst.cpu().numpy(), expect)
+    finally:
+        capi.check(lib.axr_plan_free(plan))
+        if rplan:
+            capi.check(lib.axr_plan_free(rplan))
