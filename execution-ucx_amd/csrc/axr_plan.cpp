@@ -232,7 +232,7 @@ PlanShells& plan_shells() {
   return shells;
 }
 constexpr size_t kMaxIdlePlans = 8;
-constexpr size_t kMaxIdlePlanBytes = 16u << 20;
+constexpr size_t kMaxIdlePlanBytes = 32u << 20;
 
 axr_plan* plan_new() {
   {
@@ -258,7 +258,8 @@ void plan_delete(axr_plan* p) {
   RawVec<uint8_t> header;
   std::vector<Seg> segs;
   std::vector<Dims> dims;
-  std::vector<uint32_t> wave_seg;
+  std::vector<uint32_t> wave_seg, seg_tensor, member_tensor;
+  std::vector<uint8_t> group_blocks;
   tensors.swap(p->tensors);
   dims64.swap(p->dims64);
   tensors2.swap(p->staged_tensors);
@@ -267,8 +268,11 @@ void plan_delete(axr_plan* p) {
   segs.swap(p->segs);
   dims.swap(p->dims);
   wave_seg.swap(p->wave_seg);
+  seg_tensor.swap(p->seg_tensor);
+  member_tensor.swap(p->member_tensor);
+  group_blocks.swap(p->group_blocks);
   const size_t bytes = keep(tensors) + keep(dims64) + keep(header) + keep(segs) + keep(dims) + keep(wave_seg) +
-                       keep(tensors2) + keep(dims64_2);
+                       keep(tensors2) + keep(dims64_2) + keep(seg_tensor) + keep(member_tensor) + keep(group_blocks);
   if (bytes > kMaxIdlePlanBytes) {
     delete p;
     return;
@@ -283,6 +287,9 @@ void plan_delete(axr_plan* p) {
   segs.swap(p->segs);
   dims.swap(p->dims);
   wave_seg.swap(p->wave_seg);
+  seg_tensor.swap(p->seg_tensor);
+  member_tensor.swap(p->member_tensor);
+  group_blocks.swap(p->group_blocks);
   PlanShells& shells = plan_shells();
   std::lock_guard<std::mutex> lock(shells.mu);
   if (shells.idle.size() < kMaxIdlePlans) {
