@@ -522,3 +522,57 @@ def test_two_jobs_whose_wavefronts_take_several_tiles(pkg, orc, gpu):
         assert np.array_equal(chunk_of(o), chunk_of(t))      # bytes: the random bit patterns hold NaNs
     for p in plans + [rplan]:
         p.close()
+
+
+def test_a_joint_launch_in_a_hip_graph(pkg, orc, gpu):
+    """axr_submit under stream capture: the pack of one bundle and the unpack of another share
+    one captured launch (the step a worker repeats).  Plans that were not prepared are refused
+    and record nothing; the graph is replayed several times with eager work and
+    synchronisations in between, every replay checked against the oracle."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    rng = np.random.default_rng(404)
+    a = random_tensors(rng, gpu, 300)
+    b = random_tensors(rng, gpu, 300)
+    b_out = zeros_like_views(b)
+    plan_a = pkg.BundlePlan.create(a, align=256)
+    plan_b = pkg.BundlePlan.create(b, align=256)
+    rplan_b = pkg.BundlePlan.from_header(plan_b.header).bind(b_out)
+    buf_a = torch.full((plan_a.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu)
+    buf_b = torch.full((plan_b.payload_bytes + 64,), POISON, dtype=torch.uint8, device=gpu)
+    side = torch.cuda.Stream()
+    jobs = job_array(capi, [(plan_a, 0, buf_a.data_ptr(), plan_a.payload_bytes, 0),
+                            (rplan_b, 1, buf_b.data_ptr(), plan_b.payload_bytes, 0)])
+    refused = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(refused, stream=side):
+        rc = lib.axr_submit(jobs, 2, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == capi.AXR_ERR_INVALID
+    del refused
+    plan_a.prepare()
+    rplan_b.prepare()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        capi.check(lib.axr_submit(jobs, 2, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    try:
+        for replay in range(4):
+            for t in a:
+                t.view(torch.uint8).add_(replay + 1)
+            for t in b:
+                t.view(torch.uint8).add_(2 * replay + 1)
+            for o in b_out:
+                o.zero_()
+            buf_a.fill_(POISON)
+            plan_b.pack(buf_b.data_ptr(), plan_b.payload_bytes)          # eager, on the default stream
+            torch.cuda.synchronize()
+            want_a = orc.pack([chunk_of(t) for t in a], 256)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = buf_a.cpu().numpy()
+            assert np.array_equal(got[:plan_a.payload_bytes], want_a), replay
+            assert (got[plan_a.payload_bytes:] == POISON).all(), replay
+            for o, t in zip(b_out, b):
+                assert np.array_equal(chunk_of(o), chunk_of(t)), replay
+    finally:
+        del graph
+        for p in (plan_a, plan_b, rplan_b):
+            p.close()
