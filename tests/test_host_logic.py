@@ -959,6 +959,42 @@ def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
         asyncio.run(client.invoke(1, worker_name="cpu_server", session_id=0, function=1))
 
 
+def test_runtime_calls_itself_by_name(pkg):
+    """axon/python/tests/test_invoke_by_name.py:11-84: one runtime started as server and client,
+    connected to its own address, a function registered without an id (and then without a name
+    either: the callable's __name__), invoked by name."""
+    import asyncio
+
+    def simple_echo(x):
+        return x
+
+    async def body():
+        runtime = pkg.AxonRuntime("test_worker_name_func", device=pkg.cpu())
+        runtime.start_server()
+        runtime.start_client()
+        try:
+            runtime.register_function(callable=simple_echo, function_id=None, function_name="named_echo")
+            await runtime.connect_endpoint_async(runtime.get_local_address(), "test_worker_name_func")
+            assert await runtime.invoke(42, worker_name="test_worker_name_func", session_id=1,
+                                        function="named_echo", workflow_id=1) == 42
+        finally:
+            runtime.stop()
+        implicit = pkg.AxonRuntime("test_worker_implicit", device=pkg.cpu())
+        implicit.start()
+        try:
+            implicit.register_function(callable=simple_echo, function_id=None)
+            await implicit.connect_endpoint_async(implicit.get_local_address(), "test_worker_implicit")
+            assert await implicit.invoke(100, worker_name="test_worker_implicit", session_id=1,
+                                         function="simple_echo", workflow_id=1) == 100
+            # addresses that name no worker of this process are refused, empty ones included
+            for bad in (bytes([]), bytes([0] * 100)):
+                with pytest.raises(RuntimeError, match="no worker at this address"):
+                    await implicit.connect_endpoint_async(bad, "non_existent_worker")
+        finally:
+            implicit.stop()
+    asyncio.run(body())
+
+
 def test_runtime_concurrent_calls_keep_their_replies(pkg):
     """Calls that overlap in one event loop: two clients on one server (served one at a time)
     and one client on two servers whose handlers finish in the opposite order."""
