@@ -341,8 +341,10 @@ _next_export = [1]
 
 @_DELETER
 def _managed_deleter(ptr):  # called by the consumer when it drops the tensor
-    key = ptr.contents.manager_ctx
-    entry = _live_exports.pop(key, None)
+    exports = _live_exports
+    if exports is None:     # interpreter shutdown, this module's globals are already cleared: the
+        return              # process is ending, nothing is given back
+    entry = exports.pop(ptr.contents.manager_ctx, None)
     if entry is not None and entry[3] is not None:
         entry[3]()
 
@@ -354,6 +356,15 @@ def _capsule_destructor(capsule_ptr):
         ptr = _raw_get_pointer(capsule_ptr, _NAME)
         managed = C.cast(ptr, C.POINTER(_ManagedTensor))
         managed.contents.deleter(managed)
+
+
+# A consumer may keep its tensor until the interpreter shuts down and drop it after this module
+# has been cleared: the C entry points of the two callbacks above must stay valid until the
+# process ends, so they are never freed.
+_py.Py_IncRef.argtypes = [C.py_object]
+_py.Py_IncRef.restype = None
+_py.Py_IncRef(_managed_deleter)
+_py.Py_IncRef(_capsule_destructor)
 
 
 class DLPackExport:

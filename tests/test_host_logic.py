@@ -532,6 +532,30 @@ def test_dlpack_export_single_consume(pkg):
     assert released[-1] == 9
 
 
+def test_exported_tensors_may_outlive_the_interpreter(pkg):
+    """A consumer that still holds tensors made from this package's capsules when the interpreter
+    shuts down (script globals) must not bring the process down: the tensors are dropped after the
+    modules have been cleared, and the deleters they call have to be valid and quiet then."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import numpy as np, torch\n"
+        "import __graft_entry__ as e\n"
+        "pkg = e.load_package()\n"
+        "buf = np.arange(8, dtype=np.float32)\n"
+        "x = np.from_dlpack(pkg.DLPackExport(buf.ctypes.data, (8,), (2, 32, 1), 1, 0, release=lambda: None))\n"
+        "y = torch.from_dlpack(pkg.DLPackExport(buf.ctypes.data, (2, 4), (2, 32, 1), 1, 0, release=lambda: None))\n"
+        "z = pkg.DLPackExport(buf.ctypes.data, (8,), (2, 32, 1), 1, 0).__dlpack__()   # a capsule nobody consumed\n"
+        "print('end', float(x.sum()), float(y.sum()))\n" % root)
+    out = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, (out.returncode, out.stderr[-800:])
+    assert "end 28.0 28.0" in out.stdout
+    assert "Exception ignored" not in out.stderr and "Traceback" not in out.stderr, out.stderr[-800:]
+
+
 def test_device_objects(pkg):
     d = pkg.rocm(3)
     assert d.get_type() == pkg.DeviceType.ROCM and d.get_type_string() == "rocm"
