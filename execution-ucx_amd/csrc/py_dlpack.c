@@ -216,16 +216,25 @@ done:
   return result;
 }
 
-/* new_capsule(address) -> a capsule named "dltensor" over the DLManagedTensor at `address`
- * (one that this package exports).  An unconsumed capsule still owns the tensor, so its
- * destructor runs the tensor's deleter.  A consumer that refuses a capsule drops it on its
- * error path, with its exception pending: the deleter calls back into Python, which must
- * find no error set, and the consumer's exception has to survive the call. */
+/* new_capsule(address, versioned) -> a capsule named "dltensor" over the DLManagedTensor at
+ * `address`, or named "dltensor_versioned" over a DLManagedTensorVersioned (structs that this
+ * package exports).  An unconsumed capsule still owns the tensor, so its destructor runs the
+ * tensor's deleter.  A consumer that refuses a capsule drops it on its error path, with its
+ * exception pending: the deleter calls back into Python, which must find no error set, and the
+ * consumer's exception has to survive the call. */
 typedef struct axr_managed_tensor {
   axr_tensor_t dl_tensor;
   void* manager_ctx;
   void (*deleter)(struct axr_managed_tensor*);
 } axr_managed_tensor;
+
+typedef struct axr_managed_tensor_versioned {
+  uint32_t major, minor;
+  void* manager_ctx;
+  void (*deleter)(struct axr_managed_tensor_versioned*);
+  uint64_t flags;
+  axr_tensor_t dl_tensor;
+} axr_managed_tensor_versioned;
 
 static void export_capsule_destructor(PyObject* capsule) {
   PyObject *type = NULL, *value = NULL, *traceback = NULL;
@@ -233,24 +242,32 @@ static void export_capsule_destructor(PyObject* capsule) {
   if (PyCapsule_IsValid(capsule, "dltensor")) {
     axr_managed_tensor* managed = (axr_managed_tensor*)PyCapsule_GetPointer(capsule, "dltensor");
     if (managed && managed->deleter) managed->deleter(managed);
+  } else if (PyCapsule_IsValid(capsule, "dltensor_versioned")) {
+    axr_managed_tensor_versioned* managed =
+        (axr_managed_tensor_versioned*)PyCapsule_GetPointer(capsule, "dltensor_versioned");
+    if (managed && managed->deleter) managed->deleter(managed);
   }
   PyErr_Clear();
   PyErr_Restore(type, value, traceback);
 }
 
-static PyObject* new_capsule(PyObject* self, PyObject* address) {
+static PyObject* new_capsule(PyObject* self, PyObject* args) {
   (void)self;
+  PyObject* address = NULL;
+  int versioned = 0;
+  if (!PyArg_ParseTuple(args, "O|p", &address, &versioned)) return NULL;
   void* managed = PyLong_AsVoidPtr(address);
   if (!managed) {
     if (!PyErr_Occurred()) PyErr_SetString(PyExc_ValueError, "new_capsule: null address");
     return NULL;
   }
-  return PyCapsule_New(managed, "dltensor", export_capsule_destructor);
+  return PyCapsule_New(managed, versioned ? "dltensor_versioned" : "dltensor", export_capsule_destructor);
 }
 
 static PyMethodDef methods[] = {
-    {"new_capsule", new_capsule, METH_O,
-     "new_capsule(address) -> 'dltensor' capsule that owns the DLManagedTensor at address until consumed"},
+    {"new_capsule", new_capsule, METH_VARARGS,
+     "new_capsule(address[, versioned]) -> 'dltensor' (or 'dltensor_versioned') capsule that owns the "
+     "managed tensor at address until consumed"},
     {"describe", describe, METH_VARARGS,
      "describe(sequence[, fast_type, fast_export, device_id, stream]) -> "
      "(descs bytearray, dims bytearray, owners list)"},

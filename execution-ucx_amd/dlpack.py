@@ -358,13 +358,35 @@ def _capsule_destructor(capsule_ptr):
         managed.contents.deleter(managed)
 
 
+_DELETER_VERSIONED = C.CFUNCTYPE(None, C.c_void_p)
+
+
+@_DELETER_VERSIONED
+def _managed_deleter_versioned(address):   # the same for a DLManagedTensorVersioned
+    exports = _live_exports
+    if exports is None:
+        return
+    managed = C.cast(address, C.POINTER(_ManagedTensorVersioned)).contents
+    entry = exports.pop(managed.manager_ctx, None)
+    if entry is not None and entry[3] is not None:
+        entry[3]()
+
+
+@_CAPSULE_DTOR
+def _capsule_destructor_versioned(capsule_ptr):
+    if _raw_is_valid(capsule_ptr, _NAME_VERSIONED):
+        ptr = _raw_get_pointer(capsule_ptr, _NAME_VERSIONED)
+        managed = C.cast(ptr, C.POINTER(_ManagedTensorVersioned)).contents
+        _DELETER_VERSIONED(managed.deleter)(ptr)
+
+
 # A consumer may keep its tensor until the interpreter shuts down and drop it after this module
 # has been cleared: the C entry points of the two callbacks above must stay valid until the
 # process ends, so they are never freed.
 _py.Py_IncRef.argtypes = [C.py_object]
 _py.Py_IncRef.restype = None
-_py.Py_IncRef(_managed_deleter)
-_py.Py_IncRef(_capsule_destructor)
+for _callback in (_managed_deleter, _capsule_destructor, _managed_deleter_versioned, _capsule_destructor_versioned):
+    _py.Py_IncRef(_callback)
 
 
 class DLPackExport:
@@ -406,7 +428,14 @@ class DLPackExport:
             raise RuntimeError("copy=True is not supported; this implementation is zero-copy only")
         nd = len(self._shape)
         shape = (C.c_int64 * max(nd, 1))(*self._shape)
-        managed = _ManagedTensor()
+        # A consumer that speaks DLPack 1.0 (max_version) gets a DLManagedTensorVersioned with no
+        # flag set; one that does not gets the unversioned struct, which cannot say whether the
+        # memory may be written (numpy then hands out a read-only array).  The reference's wrapper
+        # always returns the unversioned form (dlpack_helpers.hpp:149-152).
+        versioned = max_version is not None and int(tuple(max_version)[0]) >= 1
+        managed = _ManagedTensorVersioned() if versioned else _ManagedTensor()
+        if versioned:
+            managed.major, managed.minor, managed.flags = 1, 0, 0
         dl = managed.dl_tensor
         dl.data = self._data
         dl.device_type, dl.device_id = self._device
@@ -418,14 +447,19 @@ class DLPackExport:
         key = _next_export[0]
         _next_export[0] += 1
         managed.manager_ctx = key
-        managed.deleter = _managed_deleter
+        if versioned:
+            managed.deleter = C.cast(_managed_deleter_versioned, C.c_void_p).value
+        else:
+            managed.deleter = _managed_deleter
         _live_exports[key] = (managed, shape, self, self._release)
         self._exported = True
         native = _native()
         if native is not None and hasattr(native, "new_capsule"):
             # the C destructor keeps a consumer's pending exception intact when a refused
             # capsule is dropped; the ctypes one below cannot run under a pending exception
-            return native.new_capsule(C.addressof(managed))
+            return native.new_capsule(C.addressof(managed), versioned)
+        if versioned:
+            return _py.PyCapsule_New(C.addressof(managed), _NAME_VERSIONED, _capsule_destructor_versioned)
         return _py.PyCapsule_New(C.addressof(managed), _NAME, _capsule_destructor)
 
     def __del__(self):

@@ -333,6 +333,10 @@ def test_a_tensor_the_handler_keeps_outlives_the_call(pkg, gpu):
         kept["tmp"] = None
         return total
 
+    def add_one_in_place(a):
+        a += 1
+        return a
+
     async def body():
         server, client = pair(pkg, "test_lifetime_server", "test_lifetime_client")
         try:
@@ -356,6 +360,13 @@ def test_a_tensor_the_handler_keeps_outlives_the_call(pkg, gpu):
             np.testing.assert_array_equal(result, big + big)
             del result
             kept["a"] = None
+            # a handler may change what it received in place and hand the same array back
+            server.register_function(add_one_in_place, 202, from_dlpack_fn=np.from_dlpack)
+            for values in (np.arange(6, dtype=np.float64), np.arange(1 << 18, dtype=np.float64)):
+                echoed = await client.invoke(values, function=202, **kw)
+                np.testing.assert_array_equal(echoed, values + 1)
+                assert echoed.flags.writeable
+                del echoed
             c = np.array([3.0, 4.0, 5.0, 6.0], dtype=np.float64)
             assert await client.invoke(c, function=201, **kw) == int(np.sum(c))
             for _ in range(10):

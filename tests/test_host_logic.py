@@ -480,6 +480,11 @@ def test_dlpack_extract_numpy(pkg):
         pkg.extract(object())
 
 
+def fresh_of(pkg, array, released, tag):
+    dtype = {np.dtype(np.int32): (0, 32, 1), np.dtype(np.float32): (2, 32, 1)}[array.dtype]
+    return pkg.DLPackExport(array.ctypes.data, array.shape, dtype, 1, 0, release=lambda: released.append(tag))
+
+
 def test_dlpack_export_single_consume(pkg):
     released = []
     src = np.arange(40, dtype=np.int32)
@@ -522,6 +527,26 @@ def test_dlpack_export_single_consume(pkg):
     del capsule, ok
     gc.collect()
     assert released[-1] == 8
+    # a consumer that speaks DLPack 1.0 is given the versioned struct with no flag set: numpy's
+    # array over it is writable and can be exported again (a handler may modify or return it)
+    mine = np.arange(6, dtype=np.int32)
+    taken = np.from_dlpack(fresh_of(pkg, mine, released, 20))
+    assert taken.flags.writeable
+    taken[0] = 77
+    assert mine[0] == 77 and pkg.extract(taken).shape == (6,)
+    del taken
+    gc.collect()
+    assert released[-1] == 20
+    versioned = fresh_of(pkg, mine, released, 21).__dlpack__(max_version=(1, 0))
+    legacy = fresh_of(pkg, mine, released, 22).__dlpack__(max_version=(0, 8))
+    assert '"dltensor_versioned"' in repr(versioned) and '"dltensor"' in repr(legacy)
+    assert pkg.extract(versioned).shape == (6,) and pkg.extract(legacy).shape == (6,)
+    del versioned
+    gc.collect()
+    assert released[-1] == 21
+    del legacy
+    gc.collect()
+    assert released[-1] == 22
     # a consumer that refuses the capsule (numpy takes host memory only) drops it with its own
     # exception pending: that exception is what the caller sees, and the memory is released
     refused = pkg.DLPackExport(0x1000, (4,), (2, 32, 1), 10, 0, release=lambda: released.append(9))
