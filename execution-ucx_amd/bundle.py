@@ -322,9 +322,22 @@ def unpack_bundle(header: bytes, payload: Any, payload_bytes: Optional[int] = No
     device = C.c_int(0)
     _capi.check(_capi.load().axr_device_get(C.byref(device)))
     results = []
+    scalars = None
     for (p, n), m in zip(pieces, metas):
+        keep = owner
+        if len(m.shape) == 0:
+            # A 0-d tensor has no bytes in the payload (the reference's size rule,
+            # rpc_core/utils/tensor_meta.hpp:91-104), yet its consumer will read one element:
+            # it is pointed at a zeroed block of its own instead of at whatever follows its
+            # offset in the payload (possibly the end of the allocation).
+            if scalars is None:
+                lib = _capi.load()
+                scalars = DevicePool.default().alloc(256, 256)
+                _capi.check(lib.axr_memset_async(scalars.data, 0, 256, None))
+                _capi.check(lib.axr_stream_synchronize(None))
+            p, keep = scalars.data, scalars
         exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLROCM, device.value,
-                           release=(lambda keep=owner: None))
+                           release=(lambda keep=keep: None))
         results.append(from_dlpack_fn(exp) if from_dlpack_fn else exp)
     plan.close()
     return results

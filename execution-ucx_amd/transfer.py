@@ -70,10 +70,15 @@ def _host_views(plan: BundlePlan, metas: Sequence[TensorMeta], host, from_dlpack
     """kDLCPU producers over ``host`` (a numpy byte array holding the whole payload), split at
     the header's offsets; every view keeps the array alive."""
     from .dlpack import DLPackExport
+    import numpy as np
     pieces = plan.split(host.ctypes.data if host.size else 0, host.size)
     out = []
     for (p, _n), m in zip(pieces, metas):
-        exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLCPU, 0, release=(lambda keep=host: None))
+        keep = host
+        if len(m.shape) == 0:       # no bytes in the payload, one element read by the consumer
+            keep = np.zeros(32, dtype=np.uint8)
+            p = keep.ctypes.data
+        exp = DLPackExport(p, m.shape, m.dtype, _capi.kDLCPU, 0, release=(lambda keep=keep: None))
         out.append(from_dlpack_fn(exp) if from_dlpack_fn else exp)
     return out
 

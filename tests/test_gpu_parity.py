@@ -1585,3 +1585,28 @@ def test_die_contiguous_tile_ranges(pkg, orc, gpu):
                 assert np.array_equal(tbytes(v), tbytes(tv_)), tune
         finally:
             pkg.tune(xcd_remap=-1)
+
+
+def test_zero_dim_tensors_take_no_payload_bytes(pkg, orc, gpu):
+    """The reference's size rule gives a 0-d tensor no bytes (rpc_core/utils/tensor_meta.hpp:91-104):
+    it gets an offset and a header record, nothing is moved for it, a destination bound for it
+    stays as it was, and a zero-copy view of it reads a zero of its own, not what follows its
+    offset in the payload (here: the end of the payload)."""
+    import torch
+    a = torch.arange(64, dtype=torch.float32, device=gpu)
+    scalar = torch.tensor(7.5, device=gpu)
+    tensors = [a, scalar]
+    for align in (1, 256):
+        got, plan, buf = run_pack(pkg, tensors, align, gpu)
+        assert plan.payload_bytes == 256 and np.array_equal(got, orc.pack([tbytes(a), np.zeros(0, np.uint8)], align))
+        metas = plan.metas()
+        assert metas[1].shape == () and metas[1].nbytes == 0 and metas[1].offset == 256
+        outs = [torch.zeros_like(a), torch.tensor(-1.0, device=gpu)]
+        rplan = pkg.unpack_bundle(plan.header, buf.data_ptr(), payload_bytes=plan.payload_bytes, out=outs)
+        rplan.close()
+        assert torch.equal(outs[0], a) and float(outs[1]) == -1.0
+        views = pkg.unpack_bundle(plan.header, buf.data_ptr(), payload_bytes=plan.payload_bytes,
+                                  from_dlpack_fn=torch.from_dlpack)
+        assert torch.equal(views[0], a) and views[1].shape == () and float(views[1]) == 0.0
+        del views
+        plan.close()
