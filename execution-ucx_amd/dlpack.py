@@ -22,6 +22,7 @@ runtime refuses a rocm device (bindings_runtime.cpp:131-141).
 from __future__ import annotations
 
 import ctypes as C
+import itertools
 from dataclasses import dataclass
 from typing import Any, Callable, List, Optional, Sequence, Tuple
 
@@ -336,7 +337,7 @@ def _native_torch():
 # ---------------------------------------------------------------- export
 
 _live_exports = {}  # id -> (managed struct, shape array, release callback)
-_next_export = [1]
+_next_export = itertools.count(1)   # next() is one step under the interpreter lock: exports may come from several threads
 
 
 @_DELETER
@@ -444,8 +445,7 @@ class DLPackExport:
         dl.shape = C.cast(shape, C.POINTER(C.c_int64))
         dl.strides = None
         dl.byte_offset = 0
-        key = _next_export[0]
-        _next_export[0] += 1
+        key = next(_next_export)
         managed.manager_ctx = key
         if versioned:
             managed.deleter = C.cast(_managed_deleter_versioned, C.c_void_p).value
