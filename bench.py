@@ -897,6 +897,18 @@ def ceilings(h):
                                      "rotating_buffer_pairs": copies}
         ms = h.time_steps(lambda i: check(lib.axr_memset_async(b[i % copies].data_ptr(), 7, n, h.stream)), k, 3)
         out["fill_kernel"][label] = {"GBps": round(1.0 * n * k / (ms * 1e-3) / 1e9, 1)}
+        # the same copy in the shapes of the bundle kernels' wavefronts (threads per workgroup,
+        # KiB per wavefront, streaming hint): what a shape allows with no table in front of it
+        whole = n // 4096 * 4096
+        shaped = {}
+        for threads, kib, nt in ((64, 1, 1), (64, 1, 0), (256, 1, 1), (128, 2, 1), (256, 2, 1), (256, 2, 0), (256, 4, 1)):
+            ms = h.time_steps(lambda i: check(lib.axr_copy_reference_shaped(
+                b[i % copies].data_ptr(), a[i % copies].data_ptr(), whole, threads, kib, nt, h.stream)), k, 3)
+            shaped[f"{threads} threads, {kib} KiB per wavefront, {'streaming' if nt else 'cacheable'}"] = {
+                "GBps": round(2.0 * whole * k / (ms * 1e-3) / 1e9, 1), "us_per_launch": round(ms * 1e3 / k, 2)}
+        if not bool(torch.equal(a[0][:whole], b[0][:whole])):
+            raise SystemExit("bench.py: the shaped copy kernel did not copy")
+        out.setdefault("copy_kernel_shaped", {})[label] = shaped
         del a, b
         torch.cuda.empty_cache()
     for label, run, pitch, rows in (("100 B rows at a 256 B pitch", 100, 256, 1 << 21),

@@ -298,6 +298,7 @@ PROTOTYPES = {
     "axr_compare": (C.c_int, [_vp, _vp, _sz, _u64p]),
     "axr_checksum": (C.c_int, [_vp, _sz, C.c_uint64, _u64p]),
     "axr_copy_reference": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "axr_copy_reference_shaped": (C.c_int, [_vp, _vp, _sz, C.c_uint32, C.c_uint32, C.c_int, _vp]),
     "axr_rows_reference": (C.c_int, [_vp, _sz, _vp, _sz, _sz, C.c_int, C.c_uint32, _vp]),
 }
 

@@ -1317,6 +1317,26 @@ __global__ __launch_bounds__(256) void checksum_kernel(const uint8_t* data, size
   block_atomic_add(sum, local);
 }
 
+// Plain copy in the shape of the bundle kernels' wavefronts: every wavefront moves KIB KiB (KIB
+// 16-byte loads per lane, all issued before the stores), with or without the streaming hint,
+// in workgroups of the launch's choosing.  No tables, no segments: what this kernel reaches is
+// what a wavefront shape allows on the device.
+template <bool NT, uint32_t KIB>
+__global__ __launch_bounds__(1024) void copy_shaped_kernel(uint8_t* dst_arg, const uint8_t* src_arg,
+                                                           uint64_t waves, uint32_t waves_per_group) {
+  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
+  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * waves_per_group + (threadIdx.x >> 6);
+  if (wave >= waves) return;
+  const uint64_t off = wave * (1024ull * KIB) + lane * kVecBytes;
+  gcbytes src = reinterpret_cast<gcbytes>(reinterpret_cast<uintptr_t>(src_arg)) + off;
+  gbytes dst = reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(dst_arg)) + off;
+  u32x4 v[KIB];
+#pragma unroll
+  for (uint32_t u = 0; u < KIB; ++u) v[u] = load16<NT>(src + u * 1024u);
+#pragma unroll
+  for (uint32_t u = 0; u < KIB; ++u) store16<NT>(dst + u * 1024u, v[u]);
+}
+
 __global__ __launch_bounds__(256) void copy_reference_kernel(u32x4* __restrict__ dst,
                                                              const u32x4* __restrict__ src,
                                                              size_t nvec) {
@@ -1746,6 +1766,41 @@ static int copy_reference_body(void* dst, const void* src, size_t bytes, void* s
 }
 int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream) {
   return guarded([&] { return copy_reference_body(dst, src, bytes, stream); });
+}
+
+static int copy_reference_shaped_body(void* dst, const void* src, size_t bytes, uint32_t threads,
+                                      uint32_t kib_per_wave, int nontemporal, void* stream) {
+  if (bytes == 0) return AXR_OK;
+  if (!dst || !src) return fail(AXR_ERR_INVALID, "axr_copy_reference_shaped: null range");
+  if (threads < kWaveLanes || threads > 1024 || threads % kWaveLanes)
+    return fail(AXR_ERR_INVALID, "axr_copy_reference_shaped: threads must be a multiple of 64 in [64, 1024]");
+  if (kib_per_wave != 1 && kib_per_wave != 2 && kib_per_wave != 4)
+    return fail(AXR_ERR_INVALID, "axr_copy_reference_shaped: 1, 2 or 4 KiB per wavefront");
+  if (bytes % (1024ull * kib_per_wave))
+    return fail(AXR_ERR_INVALID, "axr_copy_reference_shaped: size must be a whole number of wavefront tiles");
+  const uint64_t waves = bytes / (1024ull * kib_per_wave);
+  const uint32_t per_group = threads / kWaveLanes;
+  const uint64_t groups = (waves + per_group - 1) / per_group;
+  if (groups > 0x7fffffffull) return fail(AXR_ERR_UNSUPPORTED, "axr_copy_reference_shaped: range too long for one launch");
+  const dim3 grid(static_cast<uint32_t>(groups)), block(threads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t* d = static_cast<uint8_t*>(dst);
+  const uint8_t* s = static_cast<const uint8_t*>(src);
+#define AXR_SHAPED(NT, KIB) hipLaunchKernelGGL((copy_shaped_kernel<NT, KIB>), grid, block, 0, st, d, s, waves, per_group)
+  switch (kib_per_wave * 2 + (nontemporal ? 1 : 0)) {
+    case 2: AXR_SHAPED(false, 1); break;
+    case 3: AXR_SHAPED(true, 1); break;
+    case 4: AXR_SHAPED(false, 2); break;
+    case 5: AXR_SHAPED(true, 2); break;
+    case 8: AXR_SHAPED(false, 4); break;
+    default: AXR_SHAPED(true, 4); break;
+  }
+#undef AXR_SHAPED
+  return check_hip(hipGetLastError(), "copy_reference_shaped launch");
+}
+int axr_copy_reference_shaped(void* dst, const void* src, size_t bytes, uint32_t threads, uint32_t kib_per_wave,
+                              int nontemporal, void* stream) {
+  return guarded([&] { return copy_reference_shaped_body(dst, src, bytes, threads, kib_per_wave, nontemporal, stream); });
 }
 
 static int rows_reference_body(void* strided, size_t pitch, void* packed, size_t run_bytes, size_t rows,

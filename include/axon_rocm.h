@@ -687,7 +687,7 @@ AXR_API int axr_compare(const void* a, const void* b, size_t bytes, uint64_t* mi
 AXR_API int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_t* sum);
 /* --------------------------------------------------------------- calibration */
 
-/* The two entry points below are NOT part of the drop-in surface: nothing of the reference
+/* The entry points below are NOT part of the drop-in surface: nothing of the reference
  * corresponds to them and no caller of the bundle path needs them.  They are the yardsticks
  * the measurements are read against (what a plain copy, and a plain gather of equal rows,
  * reach on the same device), kept in the library so that they run with the same compiler
@@ -696,6 +696,15 @@ AXR_API int axr_checksum(const void* data, size_t bytes, uint64_t start, uint64_
 /* Plain device copy kernel (16 B per lane, grid-stride); calibration
  * reference for profiler counters and bandwidth. */
 AXR_API int axr_copy_reference(void* dst, const void* src, size_t bytes, void* stream);
+
+/* Plain device copy in the shape of the bundle kernels' wavefronts: workgroups of `threads`
+ * threads (a multiple of 64 up to 1024), every wavefront moving kib_per_wave KiB (1, 2 or 4:
+ * that many 16-byte loads per lane, issued before the stores), streaming accesses when
+ * nontemporal != 0.  `bytes` must be a whole number of wavefront tiles.  No tables and no
+ * segments: the ceiling of a wavefront shape on this device, next to which the bundle
+ * kernels' rates are read. */
+AXR_API int axr_copy_reference_shaped(void* dst, const void* src, size_t bytes, uint32_t threads,
+                                      uint32_t kib_per_wave, int nontemporal, void* stream);
 
 /* Plain gather (scatter == 0) or scatter of `rows` rows of run_bytes bytes that lie
  * `pitch` bytes apart at `strided` and back to back at `packed`: one 16-byte access per

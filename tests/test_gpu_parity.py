@@ -1378,6 +1378,26 @@ def test_pool_and_copy_table(pkg, gpu):
         assert devobj.get_type_string() == "rocm" and devobj.get_context_handle() == 0
 
 
+def test_shaped_copy_reference_kernel(pkg, gpu):
+    """The calibration copy in every wavefront shape copies exactly its range and refuses
+    shapes and sizes it does not cover."""
+    import torch
+    lib, capi = pkg._capi.load(), pkg._capi
+    n = 3 * 4096 * 37
+    src = torch.randint(0, 256, (n + 64,), dtype=torch.uint8, device=gpu)
+    for threads in (64, 128, 256, 1024):
+        for kib in (1, 2, 4):
+            for nt in (0, 1):
+                dst = torch.full((n + 64,), POISON, dtype=torch.uint8, device=gpu)
+                torch.cuda.synchronize()
+                capi.check(lib.axr_copy_reference_shaped(dst.data_ptr(), src.data_ptr(), n, threads, kib, nt, None))
+                torch.cuda.synchronize()
+                assert torch.equal(dst[:n], src[:n]) and bool((dst[n:] == POISON).all()), (threads, kib, nt)
+    for bad in ((n, 96, 1), (n, 64, 3), (n + 1024, 64, 4), (n, 2048, 1)):
+        assert lib.axr_copy_reference_shaped(dst.data_ptr(), src.data_ptr(), bad[0], bad[1], bad[2], 1, None) == capi.AXR_ERR_INVALID
+    assert lib.axr_copy_reference_shaped(dst.data_ptr(), src.data_ptr(), 0, 64, 1, 1, None) == 0
+
+
 @pytest.mark.parametrize("nontemporal", [0, 3])
 def test_rows_reference_kernel(pkg, gpu, nontemporal):
     """The plain row gather / scatter kernel (the calibration reference of the strided modes)
