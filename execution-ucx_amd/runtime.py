@@ -170,6 +170,23 @@ def _unframe(header: bytes) -> Tuple[dict, bytes]:
     return json.loads(header[8:8 + n].decode()), header[8 + n:]
 
 
+def _timeout_milliseconds(timeout: Any) -> int:
+    """ConvertTimeout (axon/python/src/bindings_runtime_helpers.cpp:253-276): None is 300 ms, an
+    int is milliseconds, a float is seconds, a timedelta is itself; anything else is refused."""
+    import datetime
+    if timeout is None:
+        return 300
+    if isinstance(timeout, bool):
+        return int(timeout)
+    if isinstance(timeout, int):
+        return timeout
+    if isinstance(timeout, float):
+        return int(timeout * 1000.0)
+    if isinstance(timeout, datetime.timedelta):
+        return int(timeout.total_seconds() * 1000.0)
+    raise RuntimeError("timeout must be int (milliseconds), float (seconds), or timedelta")
+
+
 class AxonRuntime:
     def __init__(self, worker_name: str, thread_pool_size: int = 4, timeout: Any = None,
                  device: Optional[Device] = None, resource_manager: Any = None):
@@ -178,6 +195,7 @@ class AxonRuntime:
         self.worker_name = worker_name
         self.thread_pool_size = thread_pool_size
         self.timeout = timeout
+        self.timeout_ms = _timeout_milliseconds(timeout)    # kept; in-process calls wait for nothing
         self.device = device if device is not None else auto_detect()
         self.resource_manager = resource_manager
         self._pool: Optional[DevicePool] = getattr(resource_manager, "pool", None)

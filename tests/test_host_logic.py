@@ -944,6 +944,12 @@ def test_runtime_registration_addresses_and_plain_calls_without_a_gpu(pkg):
     rt = pkg.runtime
     with pytest.raises(ValueError):
         pkg.AxonRuntime("")
+    # the timeout argument in the reference's forms (bindings_runtime_helpers.cpp:253-276)
+    import datetime
+    for given, ms in ((None, 300), (3000, 3000), (1.5, 1500), (datetime.timedelta(seconds=2), 2000)):
+        assert pkg.AxonRuntime("t", timeout=given, device=pkg.cpu()).timeout_ms == ms
+    with pytest.raises(RuntimeError, match="timeout must be int"):
+        pkg.AxonRuntime("t", timeout="soon", device=pkg.cpu())
     server = pkg.AxonRuntime("cpu_server", device=pkg.cpu())
     with pytest.raises(RuntimeError, match="not been started"):
         server.get_local_address()
