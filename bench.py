@@ -1045,6 +1045,36 @@ def small_segments(h, tensors=65536, lo=8, hi=512, copies=4, steps=400):
     return out
 
 
+def plain_copy_of(h, nbytes):
+    """A plain device copy that reads and writes as many bytes as one step of the headline does
+    (`nbytes` read, `nbytes` written), with rotating buffers, in the library's grid-stride copy
+    kernel and in the best of its wavefront-shaped ones: the yardstick without tables, segments,
+    gaps or partly filled tiles."""
+    torch, lib, check = h.torch, h.lib, h.capi.check
+    n = nbytes // 4096 * 4096
+    copies = max(2, int((600 << 20) // (2 * n)) + 1)
+    a = [torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda") for _ in range(copies)]
+    b = [torch.empty_like(x) for x in a]
+    h.sync()
+    k = max(50, int(2e10 // n) // 10)
+    out = {"bytes_read": n, "bytes_written": n, "rotating_buffer_pairs": copies}
+    ms = h.time_steps(lambda i: check(lib.axr_copy_reference(b[i % copies].data_ptr(), a[i % copies].data_ptr(),
+                                                             n, h.stream)), k, 5)
+    out["grid_stride_256_threads"] = {"GBps": round(2.0 * n * k / (ms * 1e-3) / 1e9, 1), "us_per_launch": round(ms * 1e3 / k, 2)}
+    best = None
+    for threads, kib, nt in ((64, 1, 1), (256, 1, 1), (128, 2, 1), (256, 2, 1), (256, 2, 0)):
+        ms = h.time_steps(lambda i: check(lib.axr_copy_reference_shaped(
+            b[i % copies].data_ptr(), a[i % copies].data_ptr(), n, threads, kib, nt, h.stream)), k, 5)
+        res = {"GBps": round(2.0 * n * k / (ms * 1e-3) / 1e9, 1), "us_per_launch": round(ms * 1e3 / k, 2),
+               "shape": f"{threads} threads, {kib} KiB per wavefront, {'streaming' if nt else 'ordinary'} accesses"}
+        if best is None or res["GBps"] > best["GBps"]:
+            best = res
+    if not bool(torch.equal(a[0], b[0])):
+        raise SystemExit("bench.py: the plain copy did not copy")
+    out["best_shape"] = best
+    return out
+
+
 def load_traffic(kernel_key):
     path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
     try:
@@ -1230,6 +1260,7 @@ def main():
         # same geometry, both sides non-temporal (lowering payload_cache_bytes instead would also
         # switch the bundle to the tile geometry of payloads that stream)
         extras["c2_payload_streaming"] = c2_variant(nontemporal=3)
+        extras["plain_copy_of_the_step_bytes"] = plain_copy_of(h, 2 * P)
         extras.update({k: round(v, 2) for k, v in end_to_end_us(h, spec).items()})
         extras["fresh_bundle_from_cpp"] = end_to_end_from_cpp()
         del sets
