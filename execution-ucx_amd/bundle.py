@@ -73,13 +73,19 @@ def _stream_handle(stream) -> Optional[int]:
     raise TypeError(f"cannot take a stream handle from {type(stream).__name__}")
 
 
+def _refuse_readonly_destinations(arr: TensorArray) -> None:
+    if getattr(arr, "readonly", False):
+        raise BufferError("a read-only tensor cannot be the destination of an unpack")
+
+
 class BundlePlan:
     """Layout + device tables of one bundle (``axr_plan_t``)."""
 
-    def __init__(self, handle: int, keepalive: Any = None):
+    def __init__(self, handle: int, keepalive: Any = None, receiver: bool = False):
         self._lib = _capi.load()
         self._h = handle
         self._keep = keepalive
+        self._receiver = receiver      # made from a header: its tensors are written by unpack
 
     # ---- construction
     @classmethod
@@ -102,7 +108,7 @@ class BundlePlan:
         buf = bytes(header)
         h = C.c_void_p()
         _capi.check(lib.axr_plan_from_header(buf, len(buf), C.byref(h)))
-        return cls(h.value)
+        return cls(h.value, receiver=True)
 
     @classmethod
     def from_header_bound(cls, header: bytes, tensors: Sequence[Any]) -> "BundlePlan":
@@ -110,13 +116,16 @@ class BundlePlan:
         lib = _capi.load()
         buf = bytes(header)
         arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(tensors)
+        _refuse_readonly_destinations(arr)
         h = C.c_void_p()
         _capi.check(lib.axr_plan_from_header_bind(buf, len(buf), arr.pointer(), arr.count, C.byref(h)))
-        return cls(h.value, keepalive=arr)
+        return cls(h.value, keepalive=arr, receiver=True)
 
     def bind(self, tensors: Sequence[Any], stream=None) -> "BundlePlan":
         arr = tensors if isinstance(tensors, TensorArray) else TensorArray.from_objects(
             tensors, stream=_dlpack_stream(stream))
+        if self._receiver:
+            _refuse_readonly_destinations(arr)
         _capi.check(self._lib.axr_plan_bind(self._h, arr.pointer(), arr.count))
         self._keep = arr
         return self

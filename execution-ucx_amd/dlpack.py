@@ -87,6 +87,7 @@ class TensorView:
     strides: Optional[Tuple[int, ...]]  # elements; None = compact row-major
     byte_offset: int = 0
     owner: Any = None
+    readonly: bool = False      # the producer's DLPack 1.0 flag: may be read, must not be written
 
     @property
     def ndim(self) -> int:
@@ -107,7 +108,7 @@ class TensorView:
         return n * self.itemsize
 
 
-def _read(dl: _capi.Tensor, owner: Any) -> TensorView:
+def _read(dl: _capi.Tensor, owner: Any, readonly: bool = False) -> TensorView:
     nd = dl.ndim
     shape = tuple(dl.shape[i] for i in range(nd))
     strides = tuple(dl.strides[i] for i in range(nd)) if dl.strides else None
@@ -120,6 +121,7 @@ def _read(dl: _capi.Tensor, owner: Any) -> TensorView:
         strides=strides,
         byte_offset=dl.byte_offset,
         owner=owner,
+        readonly=readonly,
     )
 
 
@@ -154,7 +156,13 @@ def extract(obj: Any, stream: Optional[int] = None) -> TensorView:
             except Exception:  # noqa: BLE001 - host producers and older protocols refuse the argument
                 capsule = None
         if capsule is None:
-            capsule = obj.__dlpack__()
+            try:
+                capsule = obj.__dlpack__()
+            except BufferError:
+                # a producer whose memory is read-only (a numpy array over bytes, a broadcast
+                # view) can only say so in DLPack 1.0: ask for that form.  It may be packed
+                # from; binding it as a destination is refused.
+                capsule = obj.__dlpack__(max_version=(1, 0))
     if _py.PyCapsule_IsValid(capsule, _NAME):
         ptr = _py.PyCapsule_GetPointer(capsule, _NAME)
         managed = C.cast(ptr, C.POINTER(_ManagedTensor)).contents
@@ -163,7 +171,7 @@ def extract(obj: Any, stream: Optional[int] = None) -> TensorView:
     if _py.PyCapsule_IsValid(capsule, _NAME_VERSIONED):
         ptr = _py.PyCapsule_GetPointer(capsule, _NAME_VERSIONED)
         managed = C.cast(ptr, C.POINTER(_ManagedTensorVersioned)).contents
-        return _read(managed.dl_tensor, (capsule, obj))
+        return _read(managed.dl_tensor, (capsule, obj), readonly=bool(managed.flags & 1))
     raise NotDLPackError(
         f"Invalid dlpack object {obj!r} when extracting: missing __dlpack__ method "
         "or a capsule not named 'dltensor'"
@@ -180,6 +188,7 @@ class TensorArray:
     def __init__(self, views: Sequence[TensorView]):
         self._views = list(views)
         self._owners = None
+        self.readonly = any(v.readonly for v in self._views)   # some tensor must not be written
         n = len(self._views)
         self.array = (_capi.Tensor * max(n, 1))()
         total = sum(v.ndim * (2 if v.strides is not None else 1) for v in self.views)
@@ -221,15 +230,19 @@ class TensorArray:
             if direct is not None:
                 described = direct.describe(objs, exporter[2])
         if described is None and native is not None:
-            if stream is None:
-                described = native.describe(objs, *exporter)
-            else:
-                described = native.describe(objs, *(exporter or (None, None, -1)), stream)
+            try:
+                if stream is None:
+                    described = native.describe(objs, *exporter)
+                else:
+                    described = native.describe(objs, *(exporter or (None, None, -1)), stream)
+            except BufferError:     # a read-only producer: the slower path asks it in DLPack 1.0
+                described = None
         if described is None:   # no helper, or something that is not a DLPack producer
             return cls(extract_many(objs, stream))
         descs, dims, owners = described
         self = cls.__new__(cls)
         n = len(owners)
+        self.readonly = False
         self.count = n
         self._descs, self._dims, self._owners = descs, dims, (owners, list(objs))
         self.array = (_capi.Tensor * max(n, 1)).from_buffer(descs) if n else (_capi.Tensor * 1)()

@@ -1630,3 +1630,26 @@ def test_zero_dim_tensors_take_no_payload_bytes(pkg, orc, gpu):
         assert torch.equal(views[0], a) and views[1].shape == () and float(views[1]) == 0.0
         del views
         plan.close()
+
+
+def test_read_only_host_sources(pkg, orc, gpu):
+    """Host arrays that may not be written (over bytes, broadcast) are packed like any other
+    source and come back in writable destinations."""
+    frozen = np.frombuffer(bytes(range(200)) * 50, dtype=np.uint8)
+    spread = np.broadcast_to(np.arange(5, dtype=np.float32), (7, 5))
+    plain = np.arange(33, dtype=np.int16)
+    sources = [plain, frozen, spread]
+    bundle = pkg.pack_bundle(sources, align=256)
+    chunks = [np.ascontiguousarray(x).view(np.uint8).reshape(-1) for x in sources]
+    payload = pkg.bundle_to_host(bundle.header, bundle.payload, payload_bytes=bundle.payload_bytes)
+    for got, want in zip(payload, chunks):
+        assert np.array_equal(got, want)
+    outs = [np.zeros_like(plain), np.zeros(frozen.shape, np.uint8), np.zeros((7, 5), np.float32)]
+    plan = pkg.unpack_bundle(bundle.header, bundle.payload, payload_bytes=bundle.payload_bytes, out=outs)
+    plan.close()
+    for out, src in zip(outs, sources):
+        assert np.array_equal(out, src)
+    with pytest.raises(BufferError, match="read-only"):
+        pkg.unpack_bundle(bundle.header, bundle.payload, payload_bytes=bundle.payload_bytes,
+                          out=[np.zeros_like(plain), frozen, np.zeros((7, 5), np.float32)])
+    bundle.close()

@@ -478,6 +478,25 @@ def test_dlpack_extract_numpy(pkg):
     assert v.nbytes == 48
     with pytest.raises(TypeError):
         pkg.extract(object())
+    # read-only producers (an array over bytes, a broadcast view) refuse the unversioned export;
+    # they are asked in DLPack 1.0, may be packed from, and are refused as unpack destinations
+    frozen = np.frombuffer(bytes(range(64)), dtype=np.uint8)
+    spread = np.broadcast_to(np.float32(3), (4, 2))
+    assert not frozen.flags.writeable
+    v = pkg.extract(frozen)
+    assert v.readonly and v.shape == (64,) and v.data == frozen.ctypes.data
+    assert pkg.extract(spread).strides == (0, 0) and not pkg.extract(a).readonly
+    plan = pkg.BundlePlan.create([a, frozen, spread], align=1)
+    assert plan.payload_bytes == 96 + 64 + 32
+    receiver = pkg.BundlePlan.from_header(plan.header)
+    with pytest.raises(BufferError, match="read-only"):
+        receiver.bind([np.zeros_like(a), frozen, np.zeros((4, 2), np.float32)])
+    with pytest.raises(BufferError, match="read-only"):
+        pkg.BundlePlan.from_header_bound(plan.header, [np.zeros_like(a), frozen, np.zeros((4, 2), np.float32)])
+    receiver.bind([np.zeros_like(a), np.zeros(64, np.uint8), np.zeros((4, 2), np.float32)])
+    plan.bind([a, frozen, spread])                      # a sender's plan takes them again
+    plan.close()
+    receiver.close()
 
 
 def fresh_of(pkg, array, released, tag):
